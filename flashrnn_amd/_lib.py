@@ -1,0 +1,69 @@
+"""ctypes binding of libflashrnn_hip.so (declarations: include/flashrnn_hip.h)."""
+from __future__ import annotations
+
+import ctypes
+import os
+import subprocess
+from ctypes import c_char_p, c_int, c_size_t, c_void_p, POINTER
+
+_HERE = os.path.dirname(os.path.abspath(__file__))
+_LIB = None
+
+FUNCTION_IDS = {"lstm": 0, "slstm": 1, "gru": 2, "elman": 3}
+DTYPE_IDS = {"bfloat16": 0, "float32": 1}
+
+# error codes of include/flashrnn_hip.h
+E_ARG, E_UNSUPPORTED, E_NULL, E_ALIGN, E_WORKSPACE, E_DEVICE = -1, -2, -3, -4, -5, -6
+
+_P6 = [c_int] * 6
+_SIGNATURES = {
+    "frnn_last_error": (c_char_p, []),
+    "frnn_version": (c_char_p, []),
+    "frnn_function_dims": (c_int, [c_int] + [POINTER(c_int)] * 5),
+    "frnn_fused_supported": (c_int, [c_int] * 5),
+    "frnn_fused_plan": (c_int, [c_int] * 6 + [POINTER(c_int)] * 4),
+    "frnn_fused_cache_bytes": (c_size_t, _P6),
+    "frnn_fused_workspace_bytes": (c_size_t, _P6 + [c_int]),
+    "frnn_fused_forward": (c_int, [c_int] * 7 + [c_void_p] * 7 + [c_size_t, c_void_p]),
+    "frnn_fused_backward": (c_int, _P6 + [c_void_p] * 11 + [c_size_t, c_void_p]),
+    "frnn_alt_supported": (c_int, [c_int] * 5),
+    "frnn_alt_cache_bytes": (c_size_t, _P6),
+    "frnn_alt_workspace_bytes": (c_size_t, _P6 + [c_int]),
+    "frnn_alt_forward": (c_int, [c_int] * 7 + [c_void_p] * 7 + [c_size_t, c_void_p]),
+    "frnn_alt_backward": (c_int, _P6 + [c_void_p] * 11 + [c_size_t, c_void_p]),
+}
+EXPORTED_SYMBOLS = tuple(_SIGNATURES)
+
+
+def library_path() -> str:
+    return os.path.join(_HERE, "libflashrnn_hip.so")
+
+
+def build_library(jobs: int = 8, force: bool = False) -> str:
+    """Compile the HIP sources for gfx950 with hipcc (cross-compiles without a GPU)."""
+    src = os.path.join(_HERE, "csrc")
+    if force:
+        subprocess.run(["make", "-C", src, "clean"], check=True, stdout=subprocess.DEVNULL)
+    subprocess.run(["make", "-C", src, f"-j{jobs}"], check=True)
+    return library_path()
+
+
+def load_library():
+    """Load the prebuilt library; raises if it is missing (there is no fallback path)."""
+    global _LIB
+    if _LIB is None:
+        path = library_path()
+        if not os.path.exists(path):
+            raise RuntimeError(
+                f"{path} is missing: build it with `make -C {os.path.join(_HERE, 'csrc')}` "
+                "(flashrnn_amd has no CPU or PyTorch fallback)")
+        lib = ctypes.CDLL(path)
+        for name, (res, args) in _SIGNATURES.items():
+            fn = getattr(lib, name)
+            fn.restype, fn.argtypes = res, args
+        _LIB = lib
+    return _LIB
+
+
+def last_error() -> str:
+    return load_library().frnn_last_error().decode()

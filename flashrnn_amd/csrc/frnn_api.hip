@@ -1,0 +1,426 @@
+// extern "C" surface of libflashrnn_hip.so: argument validation (host only, before any launch),
+// workspace carving, launch sequencing.  No device allocation, no hidden streams, no
+// device-wide synchronisation.
+#include <stdarg.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include "frnn_alt.h"
+#include "frnn_fused_bwd.h"
+#include "frnn_fused_fwd.h"
+#include "frnn_grad.h"
+#include "frnn_launch.h"
+
+namespace frnn {
+
+static thread_local char g_err[512] = "";
+static int fail(int code, const char* fmt, ...) __attribute__((format(printf, 2, 3)));
+static int fail(int code, const char* fmt, ...) {
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(g_err, sizeof(g_err), fmt, ap);
+  va_end(ap);
+  return code;
+}
+static int hip_fail(int e, const char* what) {
+  if (e > 0) snprintf(g_err, sizeof(g_err), "%s: %s", what, hipGetErrorString((hipError_t)e));
+  else if (e == FRNN_E_UNSUPPORTED) snprintf(g_err, sizeof(g_err), "%s: tiling not compiled in", what);
+  return e;
+}
+
+// ---- plan table -------------------------------------------------------------------------------
+#define FRNN_ROW(Dv, VAR, W, U, K) {Dv, VAR, W, U, K},
+static const Plan kFwd4B[] = {FRNN_PLANS_GR4_BF16(FRNN_ROW)};
+static const Plan kFwd4F[] = {FRNN_PLANS_GR4_F32(FRNN_ROW)};
+static const Plan kFwd3B[] = {FRNN_PLANS_GR3_BF16(FRNN_ROW)};
+static const Plan kFwd3F[] = {FRNN_PLANS_GR3_F32(FRNN_ROW)};
+static const Plan kFwd1B[] = {FRNN_PLANS_GR1_BF16(FRNN_ROW)};
+static const Plan kFwd1F[] = {FRNN_PLANS_GR1_F32(FRNN_ROW)};
+static const Plan kBwd4B[] = {FRNN_BWD_PLANS_GR4_BF16(FRNN_ROW)};
+static const Plan kBwd4F[] = {FRNN_BWD_PLANS_GR4_F32(FRNN_ROW)};
+static const Plan kBwd3B[] = {FRNN_BWD_PLANS_GR3_BF16(FRNN_ROW)};
+static const Plan kBwd3F[] = {FRNN_BWD_PLANS_GR3_F32(FRNN_ROW)};
+static const Plan kBwd1B[] = {FRNN_BWD_PLANS_GR1_BF16(FRNN_ROW)};
+static const Plan kBwd1F[] = {FRNN_BWD_PLANS_GR1_F32(FRNN_ROW)};
+#undef FRNN_ROW
+
+bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out) {
+  const Plan* tab = nullptr;
+  size_t n = 0;
+#define PICK(T) { tab = T; n = sizeof(T) / sizeof(Plan); }
+  if (!backward) {
+    if (GR == 4) { if (dtype == FRNN_BF16) PICK(kFwd4B) else PICK(kFwd4F) }
+    else if (GR == 3) { if (dtype == FRNN_BF16) PICK(kFwd3B) else PICK(kFwd3F) }
+    else { if (dtype == FRNN_BF16) PICK(kFwd1B) else PICK(kFwd1F) }
+  } else {
+    if (GR == 4) { if (dtype == FRNN_BF16) PICK(kBwd4B) else PICK(kBwd4F) }
+    else if (GR == 3) { if (dtype == FRNN_BF16) PICK(kBwd3B) else PICK(kBwd3F) }
+    else { if (dtype == FRNN_BF16) PICK(kBwd1B) else PICK(kBwd1F) }
+  }
+#undef PICK
+  const Plan* dflt = nullptr;
+  for (size_t i = 0; i < n; ++i) {
+    if (tab[i].D != D) continue;
+    if (tab[i].variant == variant) { *out = tab[i]; return true; }
+    if (tab[i].variant == 0) dflt = &tab[i];
+  }
+  if (dflt) { *out = *dflt; return true; }
+  return false;
+}
+
+static int env_int(const char* name, int dflt) {
+  const char* v = getenv(name);
+  return (v && *v) ? atoi(v) : dflt;
+}
+
+// compute units of the current device; 256 (MI355X) if no device can be queried
+static int device_cus() {
+  static int cached[64] = {0};
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return 256;
+  if (cached[dev] == 0) {
+    int cu = 0;
+    if (hipDeviceGetAttribute(&cu, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess || cu <= 0) cu = 256;
+    cached[dev] = cu;
+  }
+  return cached[dev];
+}
+
+struct Bump {
+  unsigned char* base; size_t off;
+  void* take(size_t bytes) { void* p = base ? base + off : nullptr; off += (bytes + 255) & ~(size_t)255; return p; }
+};
+
+static int check_problem(int function, int dtype, int B, int T, int N, int D) {
+  if (function < 0 || function > 3) return fail(FRNN_E_ARG, "unknown function id %d", function);
+  if (dtype != FRNN_BF16 && dtype != FRNN_F32) return fail(FRNN_E_ARG, "unknown dtype id %d", dtype);
+  if (B <= 0 || T <= 0 || N <= 0 || D <= 0) return fail(FRNN_E_ARG, "non-positive size B=%d T=%d N=%d D=%d", B, T, N, D);
+  if ((long)B * T >= (1L << 31)) return fail(FRNN_E_ARG, "B*T too large");
+  return 0;
+}
+static int check_ptr(const void* p, const char* name) {
+  if (!p) return fail(FRNN_E_NULL, "%s is null", name);
+  if (((uintptr_t)p) & 15) return fail(FRNN_E_ALIGN, "%s is not 16-byte aligned", name);
+  return 0;
+}
+#define CHECK_PTR(p) { int e_ = check_ptr(p, #p); if (e_) return e_; }
+
+// ---- fused workspace layouts --------------------------------------------------------------------
+struct FusedFwdWs { int* status; u64* ll; size_t zero_bytes; size_t total; };
+static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, const Plan& p) {
+  Bump bp{(unsigned char*)ws, 0};
+  FusedFwdWs w;
+  w.status = (int*)bp.take(256);
+  const size_t groups = (size_t)N * ((B + 15) / 16);
+  const size_t llw = (size_t)16 * D / (dtype == FRNN_BF16 ? 2 : 1);
+  w.ll = (u64*)bp.take(p.kw > 1 ? groups * 2 * llw * 8 : 0);
+  w.zero_bytes = bp.off;  // status + exchange slots must start at zero for every call
+  w.total = bp.off;
+  return w;
+}
+struct FusedBwdWs { int* status; u64* ll; size_t zero_bytes; void* Rt; void* dgx; float* dbp; float* part; int splits; size_t total; };
+static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int T, int N, int D, const Plan& p) {
+  const CellDims c = cell_dims(function);
+  const size_t es = dtype_size(dtype);
+  Bump bp{(unsigned char*)ws, 0};
+  FusedBwdWs w;
+  w.status = (int*)bp.take(256);
+  const size_t bt = (B + 15) / 16, groups = (size_t)N * bt;
+  w.ll = (u64*)bp.take(p.kw > 1 ? groups * 2 * bwd_inbox_words(D, p.kw) * 8 : 0);
+  w.zero_bytes = bp.off;
+  w.Rt = bp.take((size_t)N * D * c.GR * D * es);
+  w.dgx = bp.take(function == FRNN_GRU ? (size_t)B * T * N * D * es : 0);
+  w.dbp = (float*)bp.take(bt * c.GT * N * D * 4);
+  w.splits = grad_gemm_splits(B, T, N, D, c.GR);
+  w.part = (float*)bp.take((size_t)w.splits * c.GR * N * D * D * 4);
+  w.total = bp.off;
+  return w;
+}
+
+template <int F> static int fused_fwd_dispatch(int dtype, const Plan& p, const FwdArgs& a, hipStream_t st) {
+  return dtype == FRNN_BF16 ? fused_fwd_launch<F, FRNN_BF16>(p, a, st) : fused_fwd_launch<F, FRNN_F32>(p, a, st);
+}
+template <int F> static int fused_bwd_dispatch(int dtype, const Plan& p, const BwdArgs& a, hipStream_t st) {
+  return dtype == FRNN_BF16 ? fused_bwd_launch<F, FRNN_BF16>(p, a, st) : fused_bwd_launch<F, FRNN_F32>(p, a, st);
+}
+
+// common tail of both backward paths: dR GEMM, final reductions
+static int weight_grads(int function, int dtype, int B, int T, int N, int D, const void* s0, const void* states,
+                        const void* dWx, const void* dgx, float* part, int splits, const float* dbp, int db_splits,
+                        float* dR, float* db, hipStream_t st) {
+  const CellDims c = cell_dims(function);
+  const size_t es = dtype_size(dtype);
+  const size_t ND = (size_t)N * D;
+  GradGemmArgs g;
+  memset(&g, 0, sizeof(g));
+  for (int k = 0; k < c.GR; ++k) {
+    if (function == FRNN_GRU) {
+      // R gates [g, r, z]: g lives in dgx, r and z are Wx gates 0 and 1
+      if (k == 0) { g.gsrc[k] = dgx; g.gld[k] = (long)ND; }
+      else { g.gsrc[k] = (const char*)dWx + (size_t)(k - 1) * ND * es; g.gld[k] = (long)(c.GW * ND); }
+    } else {
+      g.gsrc[k] = (const char*)dWx + (size_t)k * ND * es; g.gld[k] = (long)(c.GW * ND);
+    }
+  }
+  g.states_h = states; g.s0_h = s0; g.part = part;
+  g.B = B; g.T = T; g.N = N; g.D = D; g.GR = c.GR;
+  int e = launch_grad_gemm(dtype, g, splits, st);
+  if (e) return hip_fail(e, "dR gemm");
+  e = launch_grad_reduce(part, splits, (size_t)c.GR * N * D * D, dR, dbp, db_splits, (size_t)c.GT * ND, db, st);
+  if (e) return hip_fail(e, "gradient reduction");
+  return 0;
+}
+
+}  // namespace frnn
+
+using namespace frnn;
+
+extern "C" {
+
+const char* frnn_last_error(void) { return g_err; }
+const char* frnn_version(void) { return "flashrnn_hip 0.1 (gfx950)"; }
+
+int frnn_function_dims(int function, int* G_r, int* G_w, int* G_t, int* S, int* cache_vals) {
+  if (function < 0 || function > 3) return fail(FRNN_E_ARG, "unknown function id %d", function);
+  const CellDims c = cell_dims(function);
+  if (G_r) *G_r = c.GR;
+  if (G_w) *G_w = c.GW;
+  if (G_t) *G_t = c.GT;
+  if (S) *S = c.S;
+  if (cache_vals) *cache_vals = c.NC;
+  return 0;
+}
+
+// ---- fused ----------------------------------------------------------------------------------------
+int frnn_fused_supported(int function, int dtype, int B, int N, int D) {
+  int e = check_problem(function, dtype, B, 1, N, D);
+  if (e) return e;
+  Plan pf, pb;
+  const int GR = cell_dims(function).GR;
+  if (!find_plan(GR, dtype, D, 0, 0, &pf) || !find_plan(GR, dtype, D, 0, 1, &pb))
+    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  return 0;
+}
+
+int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
+                    int* waves, int* tiles_per_wave, int* wgs_per_head, int* active_wgs) {
+  int e = check_problem(function, dtype, B, 1, N, D);
+  if (e) return e;
+  Plan p;
+  if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p))
+    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  if (waves) *waves = p.waves;
+  if (tiles_per_wave) *tiles_per_wave = p.utw;
+  if (wgs_per_head) *wgs_per_head = p.kw;
+  if (active_wgs) *active_wgs = N * ((B + 15) / 16) * p.kw;
+  return 0;
+}
+
+size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int D) {
+  if (check_problem(function, dtype, B, T, N, D)) return 0;
+  return (size_t)T * N * ((B + 15) / 16) * 16 * D * cell_dims(function).NC * dtype_size(dtype);
+}
+
+size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
+  if (check_problem(function, dtype, B, T, N, D)) return 0;
+  Plan p;
+  if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p)) return 0;
+  return backward ? carve_fused_bwd(nullptr, function, dtype, B, T, N, D, p).total
+                  : carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
+}
+
+int frnn_fused_forward(int function, int dtype, int training, int B, int T, int N, int D,
+                       const void* Wx, const void* R, const void* b, const void* s0,
+                       void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int e = check_problem(function, dtype, B, T, N, D);
+  if (e) return e;
+  Plan p;
+  if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
+    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
+  const bool need_cache = training && cell_dims(function).NC > 0;
+  if (need_cache) CHECK_PTR(cache)
+  const FusedFwdWs w = carve_fused_fwd(workspace, dtype, B, N, D, p);
+  if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
+  hipStream_t st = (hipStream_t)stream;
+  e = launch_fill_zero(workspace, w.zero_bytes, st);
+  if (e) return hip_fail(e, "workspace clear");
+  const int groups = N * ((B + 15) / 16);
+  int per_launch = groups;
+  if (p.kw > 1) {  // workgroups that wait for each other must all be resident
+    per_launch = device_cus() / p.kw;
+    if (per_launch < 1) return fail(FRNN_E_DEVICE, "device has fewer compute units than the %d workgroups of one head", p.kw);
+  }
+  FwdArgs a;
+  a.Wx = Wx; a.R = R; a.b = b; a.s0 = s0; a.states = states; a.cache = cache;
+  a.ll = w.ll; a.status = w.status;
+  a.B = B; a.T = T; a.N = N; a.groups_total = groups;
+  a.training = need_cache ? 1 : 0;
+  a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  for (int g0 = 0; g0 < groups; g0 += per_launch) {
+    a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
+    switch (function) {
+      case FRNN_LSTM:  e = fused_fwd_dispatch<FRNN_LSTM>(dtype, p, a, st); break;
+      case FRNN_SLSTM: e = fused_fwd_dispatch<FRNN_SLSTM>(dtype, p, a, st); break;
+      case FRNN_GRU:   e = fused_fwd_dispatch<FRNN_GRU>(dtype, p, a, st); break;
+      default:         e = fused_fwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
+    }
+    if (e) return hip_fail(e, "fused forward launch");
+  }
+  return 0;
+}
+
+int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
+                        const void* R, const void* b, const void* s0, const void* states,
+                        const void* cache, const void* dstates,
+                        void* dWx, void* ds0, float* dR, float* db,
+                        void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  (void)b;
+  int e = check_problem(function, dtype, B, T, N, D);
+  if (e) return e;
+  const CellDims c = cell_dims(function);
+  Plan p;
+  if (!find_plan(c.GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
+    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
+  CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
+  if (c.NC > 0) CHECK_PTR(cache)
+  const FusedBwdWs w = carve_fused_bwd(workspace, function, dtype, B, T, N, D, p);
+  if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
+  hipStream_t st = (hipStream_t)stream;
+  e = launch_fill_zero(workspace, w.zero_bytes, st);
+  if (e) return hip_fail(e, "workspace clear");
+  e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
+  if (e) return hip_fail(e, "R transpose");
+  const int bt = (B + 15) / 16, groups = N * bt;
+  int per_launch = groups;
+  if (p.kw > 1) {
+    per_launch = device_cus() / p.kw;
+    if (per_launch < 1) return fail(FRNN_E_DEVICE, "device has fewer compute units than the %d workgroups of one head", p.kw);
+  }
+  BwdArgs a;
+  a.Rt = w.Rt; a.s0 = s0; a.states = states; a.cache = cache; a.dstates = dstates;
+  a.dWx = dWx; a.dgx = w.dgx; a.ds0 = ds0; a.dbp = w.dbp;
+  a.ll = w.ll; a.status = w.status;
+  a.B = B; a.T = T; a.N = N; a.groups_total = groups;
+  a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  for (int g0 = 0; g0 < groups; g0 += per_launch) {
+    a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
+    switch (function) {
+      case FRNN_LSTM:  e = fused_bwd_dispatch<FRNN_LSTM>(dtype, p, a, st); break;
+      case FRNN_SLSTM: e = fused_bwd_dispatch<FRNN_SLSTM>(dtype, p, a, st); break;
+      case FRNN_GRU:   e = fused_bwd_dispatch<FRNN_GRU>(dtype, p, a, st); break;
+      default:         e = fused_bwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
+    }
+    if (e) return hip_fail(e, "fused backward launch");
+  }
+  return weight_grads(function, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, bt, dR, db, st);
+}
+
+// ---- alternating --------------------------------------------------------------------------------------
+int frnn_alt_supported(int function, int dtype, int B, int N, int D) {
+  int e = check_problem(function, dtype, B, 1, N, D);
+  if (e) return e;
+  if (D % 32 != 0) return fail(FRNN_E_UNSUPPORTED, "alternating kernels need a head dim that is a multiple of 32 (got %d)", D);
+  return 0;
+}
+
+size_t frnn_alt_cache_bytes(int function, int dtype, int B, int T, int N, int D) {
+  if (check_problem(function, dtype, B, T, N, D)) return 0;
+  return (size_t)T * B * N * D * cell_dims(function).NC * dtype_size(dtype);
+}
+
+namespace {
+struct AltWs { float* ry; void* Rt; void* dgx; void* dg; float* dsr; float* dh; float* dbp; int bsplits; float* part; int splits; size_t total; };
+AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, int backward) {
+  const CellDims c = cell_dims(function);
+  const size_t es = dtype_size(dtype), ND = (size_t)N * D, BND = (size_t)B * ND;
+  Bump bp{(unsigned char*)ws, 0};
+  AltWs w;
+  memset(&w, 0, sizeof(w));
+  if (!backward) {
+    w.ry = (float*)bp.take(BND * c.GR * 4);
+  } else {
+    w.Rt = bp.take(ND * c.GR * D * es);
+    w.dgx = bp.take(function == FRNN_GRU ? (size_t)T * BND * es : 0);
+    w.dg = bp.take(BND * c.GR * es);
+    w.dsr = (float*)bp.take(((size_t)c.S * BND + BND) * 4);
+    w.dh = w.dsr + (size_t)c.S * BND;
+    const long rows = (long)B * T;
+    w.bsplits = rows < 64 ? (int)rows : 64;
+    w.dbp = (float*)bp.take((size_t)w.bsplits * c.GT * ND * 4);
+    w.splits = grad_gemm_splits(B, T, N, D, c.GR);
+    w.part = (float*)bp.take((size_t)w.splits * c.GR * ND * D * 4);
+  }
+  w.total = bp.off;
+  return w;
+}
+}  // namespace
+
+size_t frnn_alt_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
+  if (check_problem(function, dtype, B, T, N, D)) return 0;
+  return carve_alt(nullptr, function, dtype, B, T, N, D, backward).total;
+}
+
+int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N, int D,
+                     const void* Wx, const void* R, const void* b, const void* s0,
+                     void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  int e = frnn_alt_supported(function, dtype, B, N, D);
+  if (e) return e;
+  if (T <= 0) return fail(FRNN_E_ARG, "non-positive T=%d", T);
+  CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
+  const bool need_cache = training && cell_dims(function).NC > 0;
+  if (need_cache) CHECK_PTR(cache)
+  const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 0);
+  if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
+  AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0};
+  AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.ry};
+  e = alt_forward(p, bf, (hipStream_t)stream);
+  return e ? hip_fail(e, "alternating forward launch") : 0;
+}
+
+int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
+                      const void* R, const void* b, const void* s0, const void* states,
+                      const void* cache, const void* dstates,
+                      void* dWx, void* ds0, float* dR, float* db,
+                      void* workspace, size_t workspace_bytes, void* stream) {
+  g_err[0] = 0;
+  (void)b;
+  int e = frnn_alt_supported(function, dtype, B, N, D);
+  if (e) return e;
+  if (T <= 0) return fail(FRNN_E_ARG, "non-positive T=%d", T);
+  const CellDims c = cell_dims(function);
+  CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
+  CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
+  if (c.NC > 0) CHECK_PTR(cache)
+  const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 1);
+  if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
+  hipStream_t st = (hipStream_t)stream;
+  e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
+  if (e) return hip_fail(e, "R transpose");
+  AltProblem p{function, dtype, B, T, N, D, 1};
+  AltBwdBuffers bf{w.Rt, s0, states, cache, dstates, dWx, w.dgx, ds0, w.dg, w.dsr, w.dh};
+  e = alt_backward_scan(p, bf, st);
+  if (e) return hip_fail(e, "alternating backward launch");
+  // bias partial sums over (b,t) rows; sources per bias gate
+  const size_t es = dtype_size(dtype), ND = (size_t)N * D;
+  const void* src[4];
+  long ld[4];
+  for (int g = 0; g < c.GT; ++g) {
+    if (function == FRNN_GRU) {
+      if (g == 0) { src[g] = w.dgx; ld[g] = (long)ND; }
+      else { src[g] = (const char*)dWx + (size_t)(g - 1) * ND * es; ld[g] = (long)(c.GW * ND); }
+    } else {
+      src[g] = (const char*)dWx + (size_t)g * ND * es; ld[g] = (long)(c.GW * ND);
+    }
+  }
+  e = launch_bias_partial(dtype, src, ld, c.GT, N, D, (long)B * T, w.bsplits, w.dbp, st);
+  if (e) return hip_fail(e, "bias partial sums");
+  return weight_grads(function, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, w.bsplits, dR, db, st);
+}
+
+}  // extern "C"

@@ -1,0 +1,147 @@
+// Shared definitions for the gfx950 FlashRNN kernels: ids, cell descriptors, storage-type
+// traits (MFMA fragment shapes, tagged exchange words) and small device helpers.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+
+#include "../../include/flashrnn_hip.h"
+
+namespace frnn {
+
+typedef __bf16 bf16_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned long long u64;
+
+// ---------------------------------------------------------------------------------------
+// Cell descriptors.  Gate-slot rule of the reference (flashrnn/flashrnn/flashrnn.py:148-158):
+// R fills the first GR of the GI interacting slots, Wx the last GW, b covers all GT.
+// NC = values cached per element for the backward pass (private layout, see DESIGN).
+// ---------------------------------------------------------------------------------------
+template <int F> struct Cell;
+template <> struct Cell<FRNN_LSTM>  { static constexpr int GR = 4, GW = 4, GT = 4, S = 2, NC = 4; };
+template <> struct Cell<FRNN_SLSTM> { static constexpr int GR = 4, GW = 4, GT = 4, S = 4, NC = 5; };
+template <> struct Cell<FRNN_GRU>   { static constexpr int GR = 3, GW = 3, GT = 4, S = 1, NC = 4; };
+template <> struct Cell<FRNN_ELMAN> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 0; };
+
+struct CellDims { int GR, GW, GT, S, NC; };
+inline CellDims cell_dims(int f) {
+  switch (f) {
+    case FRNN_LSTM:  return {4, 4, 4, 2, 4};
+    case FRNN_SLSTM: return {4, 4, 4, 4, 5};
+    case FRNN_GRU:   return {3, 3, 4, 1, 4};
+    case FRNN_ELMAN: return {1, 1, 1, 1, 0};
+  }
+  return {0, 0, 0, 0, 0};
+}
+inline int dtype_size(int dt) { return dt == FRNN_BF16 ? 2 : 4; }
+
+// ---------------------------------------------------------------------------------------
+// Storage-type traits.
+//  KM   : K extent of one MFMA (bf16: v_mfma_f32_16x16x32_bf16, f32: v_mfma_f32_16x16x4_f32)
+//  Frag : per-lane A/B operand of one MFMA
+//  EPW  : elements carried by one 64-bit tagged exchange word
+// Fragment order of a [16 rows x K] operand (row = batch for the streamed operand):
+//  bf16: element (row, k) -> ((k/32)*64 + ((k%32)/8)*16 + row)*8 + k%8
+//  f32 : element (row, k) -> (k/4)*64 + (k%4)*16 + row
+// so that lane l of k-step ks reads one contiguous Frag at (ks*64 + l).
+// ---------------------------------------------------------------------------------------
+template <typename T> struct ST;
+template <> struct ST<bf16_t> {
+  static constexpr int KM = 32, EPW = 2, ID = FRNN_BF16;
+  static constexpr bool FAST = true;
+  typedef bf16x8 Frag;
+  typedef uint2 Vec4;  // 4 packed elements
+  static __device__ __forceinline__ int frag_elem(int row, int k) {
+    return (((k >> 5) * 64 + ((k & 31) >> 3) * 16 + row) << 3) + (k & 7);
+  }
+  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct ST<float> {
+  static constexpr int KM = 4, EPW = 1, ID = FRNN_F32;
+  static constexpr bool FAST = false;
+  typedef float Frag;
+  typedef float4 Vec4;
+  static __device__ __forceinline__ int frag_elem(int row, int k) {
+    return (k >> 2) * 64 + (k & 3) * 16 + row;
+  }
+  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
+  }
+};
+
+__device__ __forceinline__ float bf2f(unsigned short u) { return __uint_as_float(((unsigned)u) << 16); }
+__device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest even; NaN stays NaN
+  unsigned u = __float_as_uint(f);
+  if ((u & 0x7fffffffu) > 0x7f800000u) return (unsigned short)((u >> 16) | 0x40);
+  u += 0x7fffu + ((u >> 16) & 1u);
+  return (unsigned short)(u >> 16);
+}
+
+// 4 consecutive elements <-> 4 floats
+__device__ __forceinline__ void unpack4(uint2 v, float* o) {
+  o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+  o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+__device__ __forceinline__ void unpack4(float4 v, float* o) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
+__device__ __forceinline__ void pack4(const float* i, uint2& v) {
+  v.x = (unsigned)f2bf(i[0]) | ((unsigned)f2bf(i[1]) << 16);
+  v.y = (unsigned)f2bf(i[2]) | ((unsigned)f2bf(i[3]) << 16);
+}
+__device__ __forceinline__ void pack4(const float* i, float4& v) { v = make_float4(i[0], i[1], i[2], i[3]); }
+
+// value as it will be seen after a round trip through the storage type
+__device__ __forceinline__ float round_st(float x, bf16_t*) { return bf2f(f2bf(x)); }
+__device__ __forceinline__ float round_st(float x, float*) { return x; }
+
+// ---------------------------------------------------------------------------------------
+// Tagged exchange words ("data + step tag in one store"): a reader that sees the tag of the
+// step it waits for has the data of that step; no separate flag, no fence.  32-bit stores
+// are single-copy atomic, so each tagged element is validated on its own.
+//  bf16: 64-bit word = two (tag16 << 16 | bf16) halves;  f32: (tag32 << 32 | f32 bits).
+// Tag of step t is never 0, so zero-filled memory never validates.
+// ---------------------------------------------------------------------------------------
+__device__ __forceinline__ unsigned tag16(int t) { return (unsigned)(t % 65535) + 1u; }
+__device__ __forceinline__ u64 ll_pack(bf16_t*, float a, float b, int t) {
+  unsigned tg = tag16(t) << 16;
+  return (u64)(tg | f2bf(a)) | ((u64)(tg | f2bf(b)) << 32);
+}
+__device__ __forceinline__ u64 ll_pack(float*, float a, int t) {
+  return (u64)__float_as_uint(a) | ((u64)(unsigned)(t + 1) << 32);
+}
+__device__ __forceinline__ bool ll_ok(bf16_t*, u64 w, int t) {
+  unsigned tg = tag16(t);
+  return ((unsigned)(w >> 16) & 0xffffu) == tg && (unsigned)(w >> 48) == tg;
+}
+__device__ __forceinline__ bool ll_ok(float*, u64 w, int t) { return (unsigned)(w >> 32) == (unsigned)(t + 1); }
+// payload as the 32 bits that go to LDS (bf16: two elements; f32: one)
+__device__ __forceinline__ unsigned ll_payload(bf16_t*, u64 w) {
+  return ((unsigned)w & 0xffffu) | (((unsigned)(w >> 32) & 0xffffu) << 16);
+}
+__device__ __forceinline__ unsigned ll_payload(float*, u64 w) { return (unsigned)w; }
+
+__device__ __forceinline__ u64 ll_load(const u64* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void ll_store(u64* p, u64 v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
+// status word values written by a kernel whose bounded wait ran out
+enum { STATUS_OK = 0, STATUS_WAIT_EXPIRED = 1 };
+
+// Workgroup -> (group, slice) mapping.  Workgroups are dispatched round-robin over the 8
+// XCDs, so the KW workgroups of one (head, batch-tile) group take ids that are congruent
+// mod 8 and share one XCD's L2.  grid = 8 * KW * ceil(groups / 8).
+__device__ __forceinline__ bool decode_block(int groups, int KW, int& grp, int& slice) {
+  const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
+  grp = (q / KW) * 8 + xcd;
+  slice = q % KW;
+  return grp < groups;
+}
+inline int grid_for(int groups, int KW) { return 8 * KW * ((groups + 7) / 8); }
+
+}  // namespace frnn

@@ -1,0 +1,219 @@
+// Weight-gradient side of the backward pass, shared by the fused and the alternating backend:
+//   * transpose of R for the reverse contraction      (reference: Python-side permute+contiguous,
+//     flashrnn/flashrnn/flashrnn.py:746 and :874)
+//   * dR[g,n,d,p] = sum_{b,t} dG_g[b,t,n,d] * h_{t-1}[b,n,p]  as one split-K MFMA GEMM over all
+//     compute units after the scan                    (reference: cuBLAS gemmsb with k = B*T,
+//     flashrnn/flashrnn/fused/flashrnn_fused_backward.cu:1049-1055)
+//   * final reduction of the split-K partial sums and of the per-batch-tile bias sums
+//     (reference: gradientBiasAggregationKernel, flashrnn_fused_backward.cu:626-665).
+// Both GEMM operands are stored with the contraction index (b,t) as the slow index, so tiles are
+// transposed on their way into LDS (bf16; the fp32 MFMA takes them as they are).
+#include "frnn_grad.h"
+
+namespace frnn {
+
+// ---------------------------------------------------------------------------------------------
+template <typename T>
+__global__ void __launch_bounds__(256) transpose_r_kernel(const T* __restrict__ R, T* __restrict__ Rt, int N, int D, int GR) {
+  __shared__ T tile[32][33];
+  const int g = blockIdx.z / N, n = blockIdx.z % N;
+  const int d0 = blockIdx.y * 32, p0 = blockIdx.x * 32;
+  const int tx = threadIdx.x & 31, ty = threadIdx.x >> 5;
+  const T* src = R + ((size_t)(g * N + n) * D) * D;
+  for (int r = ty; r < 32; r += 8) tile[r][tx] = src[(size_t)(d0 + r) * D + p0 + tx];  // [d][p]
+  __syncthreads();
+  T* dst = Rt + (size_t)n * D * ((size_t)GR * D);
+  for (int r = ty; r < 32; r += 8) dst[(size_t)(p0 + r) * ((size_t)GR * D) + (size_t)g * D + d0 + tx] = tile[tx][r];
+}
+
+int launch_transpose_r(int dtype, const void* R, void* Rt, int N, int D, int GR, hipStream_t st) {
+  const dim3 grid(D / 32, D / 32, GR * N);
+  if (dtype == FRNN_BF16)
+    hipLaunchKernelGGL(transpose_r_kernel<unsigned short>, grid, dim3(256), 0, st, (const unsigned short*)R, (unsigned short*)Rt, N, D, GR);
+  else
+    hipLaunchKernelGGL(transpose_r_kernel<float>, grid, dim3(256), 0, st, (const float*)R, (float*)Rt, N, D, GR);
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------
+// dR GEMM.  Workgroup tile TM (units d of one gate) x TM (previous units p), 4 waves in 2 x 2,
+// 32 rows (b,t) per LDS stage; grid (tiles, N, splits).
+// ---------------------------------------------------------------------------------------------
+template <typename T, int TM> struct GemmStage;
+
+template <int TM> struct GemmStage<bf16_t, TM> {
+  static constexpr int LD = 40;  // 32 rows + pad, 80-byte row stride keeps 16-byte alignment
+  bf16_t a[TM][LD], b[TM][LD];   // transposed: [unit][row]
+};
+template <int TM> struct GemmStage<float, TM> {
+  static constexpr int LD = TM + 4;
+  float a[32][LD], b[32][LD];    // as stored: [row][unit]
+};
+
+template <typename T, int TM>
+__global__ void __launch_bounds__(256) grad_gemm_kernel(const GradGemmArgs a) {
+  typedef ST<T> X;
+  constexpr int EV = TM / 8;           // elements per thread per staged row
+  constexpr int WT = TM / 32;          // MFMA tiles per wave per dimension
+  __shared__ __attribute__((aligned(16))) GemmStage<T, TM> sm;
+
+  const int tiles_p = a.D / TM, tiles_d = a.D / TM;
+  int tile = blockIdx.x;
+  const int pt = tile % tiles_p; tile /= tiles_p;
+  const int dt = tile % tiles_d;
+  const int g = tile / tiles_d;
+  const int n = blockIdx.y, split = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int wm = w >> 1, wn = w & 1;
+  const int r16 = lane & 15, q4 = lane >> 4;
+  const int D = a.D, N = a.N, Tn = a.T;
+  const long rows = (long)a.B * Tn;
+  const long r_begin = (long)split * a.rows_per_split;
+  const long r_end = min(rows, r_begin + a.rows_per_split);
+  const size_t ND = (size_t)N * D;
+
+  const T* __restrict__ G = static_cast<const T*>(a.gsrc[g]) + (size_t)n * D + dt * TM;
+  const long gld = a.gld[g];
+  const T* __restrict__ H = static_cast<const T*>(a.states_h) + (size_t)n * D + pt * TM;
+  const T* __restrict__ H0 = static_cast<const T*>(a.s0_h) + (size_t)n * D + pt * TM;
+
+  const int rr = tid / (TM / EV), cc = (tid % (TM / EV)) * EV;
+
+  f32x4 acc[WT][WT];
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
+
+  T ga[EV], hb[EV];
+  auto fetch = [&](long r0) __attribute__((always_inline)) {
+    const long r = r0 + rr;
+    if (r < r_end) {
+      const long b = r / Tn, t = r - b * Tn;
+      const T* gp = G + (size_t)r * gld + cc;
+      const T* hp = (t > 0) ? H + (size_t)(r - 1) * ND + cc : H0 + (size_t)b * ND + cc;
+#pragma unroll
+      for (int e = 0; e < EV; ++e) { ga[e] = gp[e]; hb[e] = hp[e]; }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EV; ++e) { ga[e] = (T)0.0f; hb[e] = (T)0.0f; }
+    }
+  };
+
+  fetch(r_begin);
+  for (long r0 = r_begin; r0 < r_end; r0 += 32) {
+    __syncthreads();  // previous stage fully consumed
+    if constexpr (sizeof(T) == 2) {
+#pragma unroll
+      for (int e = 0; e < EV; ++e) { sm.a[cc + e][rr] = ga[e]; sm.b[cc + e][rr] = hb[e]; }
+    } else {
+#pragma unroll
+      for (int e = 0; e < EV; ++e) { sm.a[rr][cc + e] = ga[e]; sm.b[rr][cc + e] = hb[e]; }
+    }
+    __syncthreads();
+    if (r0 + 32 < r_end) fetch(r0 + 32);
+    if constexpr (sizeof(T) == 2) {
+      bf16x8 af[WT], bfr[WT];
+#pragma unroll
+      for (int i = 0; i < WT; ++i) {
+        af[i] = *reinterpret_cast<const bf16x8*>(&sm.a[wm * (TM / 2) + i * 16 + r16][q4 * 8]);
+        bfr[i] = *reinterpret_cast<const bf16x8*>(&sm.b[wn * (TM / 2) + i * 16 + r16][q4 * 8]);
+      }
+#pragma unroll
+      for (int i = 0; i < WT; ++i)
+#pragma unroll
+        for (int j = 0; j < WT; ++j) acc[i][j] = X::mfma(af[i], bfr[j], acc[i][j]);
+    } else {
+#pragma unroll
+      for (int k4 = 0; k4 < 8; ++k4) {
+        float af[WT], bfr[WT];
+#pragma unroll
+        for (int i = 0; i < WT; ++i) {
+          af[i] = sm.a[k4 * 4 + q4][wm * (TM / 2) + i * 16 + r16];
+          bfr[i] = sm.b[k4 * 4 + q4][wn * (TM / 2) + i * 16 + r16];
+        }
+#pragma unroll
+        for (int i = 0; i < WT; ++i)
+#pragma unroll
+          for (int j = 0; j < WT; ++j) acc[i][j] = X::mfma(af[i], bfr[j], acc[i][j]);
+      }
+    }
+  }
+
+  float* out = a.part + ((((size_t)split * a.GR + g) * N + n) * D) * D;
+#pragma unroll
+  for (int i = 0; i < WT; ++i)
+#pragma unroll
+    for (int j = 0; j < WT; ++j) {
+      const int d = dt * TM + wm * (TM / 2) + i * 16 + q4 * 4;
+      const int p = pt * TM + wn * (TM / 2) + j * 16 + r16;
+#pragma unroll
+      for (int e = 0; e < 4; ++e) out[(size_t)(d + e) * D + p] = acc[i][j][e];
+    }
+}
+
+int grad_gemm_splits(int B, int T, int N, int D, int GR) {
+  const int TM = (D % 64 == 0) ? 64 : 32;
+  const long tiles = (long)GR * (D / TM) * (D / TM) * N;
+  const long chunks = ((long)B * T + 31) / 32;
+  long s = (1024 + tiles - 1) / tiles;
+  if (s > 16) s = 16;
+  if (s > chunks) s = chunks;
+  if (s < 1) s = 1;
+  return (int)s;
+}
+
+int launch_grad_gemm(int dtype, GradGemmArgs a, int splits, hipStream_t st) {
+  const int TM = (a.D % 64 == 0) ? 64 : 32;
+  const long chunks = ((long)a.B * a.T + 31) / 32;
+  a.rows_per_split = (int)(((chunks + splits - 1) / splits) * 32);
+  const dim3 grid(a.GR * (a.D / TM) * (a.D / TM), a.N, splits);
+  if (dtype == FRNN_BF16) {
+    if (TM == 64) hipLaunchKernelGGL((grad_gemm_kernel<bf16_t, 64>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((grad_gemm_kernel<bf16_t, 32>), grid, dim3(256), 0, st, a);
+  } else {
+    if (TM == 64) hipLaunchKernelGGL((grad_gemm_kernel<float, 64>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((grad_gemm_kernel<float, 32>), grid, dim3(256), 0, st, a);
+  }
+  return (int)hipGetLastError();
+}
+
+// ---------------------------------------------------------------------------------------------
+// out[i] = sum_s part[s][i]: i < n_r for the dR partials (splits_r of them), then i - n_r < n_b
+// for the bias partials (splits_b of them).
+// ---------------------------------------------------------------------------------------------
+__global__ void __launch_bounds__(256) grad_reduce_kernel(const float* __restrict__ part_r, int splits_r, size_t n_r, float* __restrict__ dR,
+                                                          const float* __restrict__ part_b, int splits_b, size_t n_b, float* __restrict__ db) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < n_r) {
+    float s = 0.f;
+    for (int k = 0; k < splits_r; ++k) s += part_r[(size_t)k * n_r + i];
+    dR[i] = s;
+  } else if (i - n_r < n_b) {
+    const size_t j = i - n_r;
+    float s = 0.f;
+    for (int k = 0; k < splits_b; ++k) s += part_b[(size_t)k * n_b + j];
+    db[j] = s;
+  }
+}
+
+int launch_grad_reduce(const float* part_r, int splits_r, size_t n_r, float* dR,
+                       const float* part_b, int splits_b, size_t n_b, float* db, hipStream_t st) {
+  const size_t total = n_r + n_b;
+  hipLaunchKernelGGL(grad_reduce_kernel, dim3((unsigned)((total + 255) / 256)), dim3(256), 0, st,
+                     part_r, splits_r, n_r, dR, part_b, splits_b, n_b, db);
+  return (int)hipGetLastError();
+}
+
+__global__ void __launch_bounds__(256) fill_zero_kernel(unsigned* p, size_t words) {
+  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  if (i < words) p[i] = 0u;
+}
+int launch_fill_zero(void* p, size_t bytes, hipStream_t st) {
+  const size_t words = (bytes + 3) / 4;
+  if (words == 0) return 0;
+  hipLaunchKernelGGL(fill_zero_kernel, dim3((unsigned)((words + 255) / 256)), dim3(256), 0, st, (unsigned*)p, words);
+  return (int)hipGetLastError();
+}
+
+}  // namespace frnn

@@ -1,0 +1,53 @@
+// Declarations shared between the per-(function, dtype) kernel translation units and the API.
+#pragma once
+#include "frnn_common.h"
+#include "frnn_plan.h"
+
+namespace frnn {
+
+struct FwdArgs;
+struct BwdArgs;
+
+// Each is defined in exactly one translation unit (fused_fwd_tu.hip / fused_bwd_tu.hip compiled
+// with -DFRNN_F=<function> -DFRNN_DT=<dtype>).  Return: hipError_t, or FRNN_E_UNSUPPORTED if the
+// plan is not compiled in.
+template <int F, int DT> int fused_fwd_launch(const Plan& p, const FwdArgs& a, hipStream_t st);
+template <int F, int DT> int fused_bwd_launch(const Plan& p, const BwdArgs& a, hipStream_t st);
+
+// plan table lookup: gate rows per unit (4/3/1), dtype, D, variant -> plan; false if none
+bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out);
+
+}  // namespace frnn
+
+#if defined(FRNN_F) && defined(FRNN_DT)
+#if FRNN_DT == 0
+#define FRNN_TU_T frnn::bf16_t
+#else
+#define FRNN_TU_T float
+#endif
+#if FRNN_F == 0 || FRNN_F == 1
+#if FRNN_DT == 0
+#define FRNN_TU_PLANS FRNN_PLANS_GR4_BF16
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16
+#else
+#define FRNN_TU_PLANS FRNN_PLANS_GR4_F32
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_F32
+#endif
+#elif FRNN_F == 2
+#if FRNN_DT == 0
+#define FRNN_TU_PLANS FRNN_PLANS_GR3_BF16
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR3_BF16
+#else
+#define FRNN_TU_PLANS FRNN_PLANS_GR3_F32
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR3_F32
+#endif
+#else
+#if FRNN_DT == 0
+#define FRNN_TU_PLANS FRNN_PLANS_GR1_BF16
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR1_BF16
+#else
+#define FRNN_TU_PLANS FRNN_PLANS_GR1_F32
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR1_F32
+#endif
+#endif
+#endif

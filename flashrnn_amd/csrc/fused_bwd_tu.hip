@@ -1,0 +1,27 @@
+// One translation unit per (function, storage type): instantiates the fused backward kernel for
+// every tiling in the plan table.  Build with -DFRNN_F=<0..3> -DFRNN_DT=<0|1>.
+#include "frnn_fused_bwd.h"
+#include "frnn_launch.h"
+
+namespace frnn {
+
+template <>
+int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream_t st) {
+  const dim3 grid(grid_for(a.groups, p.kw));
+  const size_t lds = (size_t)2 * 16 * Cell<FRNN_F>::GR * (p.D / p.kw) * sizeof(FRNN_TU_T);
+#define FRNN_CASE(Dv, VAR, W, U, K)                                                                     \
+  if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                            \
+    auto kern = fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K>;                                        \
+    if (lds > 65536) {                                                                                   \
+      hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
+      if (e != hipSuccess) return (int)e;                                                                \
+    }                                                                                                    \
+    hipLaunchKernelGGL(kern, grid, dim3(W * 64), lds, st, a);                                            \
+    return (int)hipGetLastError();                                                                       \
+  }
+  FRNN_TU_BWD_PLANS(FRNN_CASE)
+#undef FRNN_CASE
+  return FRNN_E_UNSUPPORTED;
+}
+
+}  // namespace frnn

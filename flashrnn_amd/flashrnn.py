@@ -1,0 +1,230 @@
+"""Functional API and autograd shim.
+
+Mirrors the reference's operator interface (flashrnn/flashrnn/flashrnn.py):
+  * ``flashrnn(Wx, R, b, states=None, function=, config=, backend=, dtype=)``   :1114-1135
+  * ``FlashRNNConfig`` and ``rnn_function_registry``                           :49-71, :124-337
+  * the autograd.Function shims ``FlashRNNFunctionFused`` / ``FlashRNNFunction`` :679-889
+with backends ``hip_fused`` (for the reference's ``cuda_fused``) and ``hip`` (for ``cuda``).
+
+What the shim does NOT do, because the kernels make it unnecessary: permute inputs to internal
+layouts (:1130-1133), make them contiguous copies (:1053), pad the batch (:699-717), transpose R
+for the backward pass (:746) or slice dWx (:789-796).
+"""
+from __future__ import annotations
+
+import os
+from dataclasses import dataclass
+from typing import Optional
+
+import torch
+
+from . import _lib
+
+# function -> (num_gates_r, num_gates_w, num_gates_i, num_gates_t, num_states); flashrnn.py:49-71
+rnn_function_registry = {
+    "slstm": {"gates_states": (4, 4, 4, 4, 4), "constants": {}, "simple_agg": True},
+    "lstm": {"gates_states": (4, 4, 4, 4, 2), "constants": {}, "simple_agg": True},
+    "gru": {"gates_states": (3, 3, 4, 4, 1), "constants": {}, "simple_agg": False},
+    "elman": {"gates_states": (1, 1, 1, 1, 1), "constants": {}, "simple_agg": True},
+}
+
+DTYPE_DICT = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+BACKENDS = ("hip_fused", "hip")
+
+
+@dataclass
+class FlashRNNConfig:
+    """The fields of the reference's FlashRNNConfig (flashrnn.py:124-231) that describe the
+    problem; tiling, internal layouts and per-tensor dtypes have no counterpart here."""
+
+    backend: str = "hip_fused"
+    function: str = "lstm"
+    dtype: str = "bfloat16"
+    head_dim: int = -1
+    num_heads: int = -1
+    hidden_dim: int = -1
+    batch_size: int = 8
+    gradient_recurrent_cut: bool = False
+    gradient_recurrent_clipval: Optional[float] = None
+    forward_clipval: Optional[float] = None
+    num_states: int = 0
+    num_gates_r: int = 0
+    num_gates_w: int = 0
+    num_gates_i: int = 0
+    num_gates_t: int = 0
+    simple_agg: bool = True
+
+    def __post_init__(self):
+        if self.function not in rnn_function_registry:
+            raise ValueError(f"RNN function {self.function} not in registry")
+        if self.backend not in BACKENDS:
+            raise ValueError(
+                f"Unknown backend {self.backend}: this package provides {BACKENDS}; the pure-PyTorch "
+                "'vanilla' loop is the test oracle and is not part of the package")
+        if self.dtype not in DTYPE_DICT:
+            raise ValueError(f"dtype {self.dtype} not supported (bfloat16, float32)")
+        if self.gradient_recurrent_cut or self.gradient_recurrent_clipval is not None \
+                or self.forward_clipval is not None:
+            raise NotImplementedError("gradient cut / clip options are not implemented")
+        (self.num_gates_r, self.num_gates_w, self.num_gates_i, self.num_gates_t,
+         self.num_states) = rnn_function_registry[self.function]["gates_states"]
+        self.simple_agg = rnn_function_registry[self.function]["simple_agg"]
+        if self.num_heads <= 0 and self.head_dim <= 0:
+            self.num_heads = 1
+        if self.num_heads <= 0:
+            self.num_heads = self.hidden_dim // self.head_dim
+        elif self.head_dim <= 0:
+            self.head_dim = self.hidden_dim // self.num_heads
+        if self.hidden_dim <= 0:
+            self.hidden_dim = self.num_heads * self.head_dim
+
+
+def _entry(backend: str, name: str):
+    prefix = "frnn_fused_" if backend == "hip_fused" else "frnn_alt_"
+    return getattr(_lib.load_library(), prefix + name)
+
+
+def _raise(code: int, what: str):
+    msg = f"{what}: {_lib.last_error()} (code {code})"
+    if code == _lib.E_UNSUPPORTED:
+        raise ValueError(msg)  # the reference raises ValueError when no tiling exists
+    raise RuntimeError(msg)
+
+
+_last_workspace = {}
+
+
+def last_status(kind: str = "forward") -> int:
+    """Status word of the most recent fused call of this kind (synchronises): 0 ok, 1 = a bounded
+    wait between workgroups ran out and the outputs were filled with NaN."""
+    ws = _last_workspace.get(kind)
+    return 0 if ws is None else int(ws[:4].view(torch.int32).item())
+
+
+def fused_plan(function: str, dtype: str, B: int, N: int, D: int, backward: bool = False):
+    """(waves per workgroup, unit tiles per wave, workgroups per head, workgroups doing work)."""
+    import ctypes
+
+    out = [ctypes.c_int() for _ in range(4)]
+    rc = _lib.load_library().frnn_fused_plan(_lib.FUNCTION_IDS[function], _lib.DTYPE_IDS[dtype], B, N, D,
+                                            int(backward), *[ctypes.byref(o) for o in out])
+    if rc != 0:
+        _raise(rc, "fused_plan")
+    return tuple(o.value for o in out)
+
+
+class _FlashRNNFunction(torch.autograd.Function):
+    """forward(Wx [B,T,G_w,N,D], R [G_r,N,D,D], b [G_t,N,D], s0 [S,B,1,N,D]) -> states [S,B,T,N,D]."""
+
+    @staticmethod
+    def forward(ctx, Wx, R, b, s0, cfg: FlashRNNConfig, training: bool):
+        if not Wx.is_cuda:
+            raise RuntimeError("flashrnn_amd runs on a GPU only (got a CPU tensor); there is no CPU fallback")
+        kdt = DTYPE_DICT[cfg.dtype]
+        f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
+        B, T, Gw, N, D = Wx.shape
+        S = cfg.num_states
+        # cast to the kernel type as the reference's custom_fwd(cast_inputs=...) does (:690-695)
+        Wx_k = Wx.detach().to(kdt).contiguous()
+        R_k = R.detach().to(kdt).contiguous()
+        b_k = b.detach().to(kdt).contiguous()
+        s0_k = s0.detach().to(kdt).reshape(S, B, N, D).contiguous()
+        with torch.cuda.device(Wx.device):
+            rc = _entry(cfg.backend, "supported")(f_id, d_id, B, N, D)
+            if rc != 0:
+                _raise(rc, f"{cfg.backend} backend")
+            states = torch.empty((S, B, T, N, D), dtype=kdt, device=Wx.device)
+            cache_bytes = _entry(cfg.backend, "cache_bytes")(f_id, d_id, B, T, N, D) if training else 0
+            cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx.device)
+            ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 0)
+            ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx.device)
+            stream = torch.cuda.current_stream().cuda_stream
+            rc = _entry(cfg.backend, "forward")(
+                f_id, d_id, int(training), B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(),
+                s0_k.data_ptr(), states.data_ptr(), cache.data_ptr() if training else None,
+                ws.data_ptr(), ws.numel(), stream)
+            if rc != 0:
+                _raise(rc, f"{cfg.backend} forward")
+        _last_workspace["forward"] = ws
+        ctx.cfg, ctx.training = cfg, training
+        ctx.dims = (B, T, N, D)
+        ctx.save_for_backward(R_k, b_k, s0_k, states, cache)
+        return states
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dstates):
+        if not ctx.training:
+            raise RuntimeError("FlashRNN backward can only be called in training mode")
+        cfg = ctx.cfg
+        R_k, b_k, s0_k, states, cache = ctx.saved_tensors
+        kdt = DTYPE_DICT[cfg.dtype]
+        f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
+        B, T, N, D = ctx.dims
+        S, Gw, Gr, Gt = cfg.num_states, cfg.num_gates_w, cfg.num_gates_r, cfg.num_gates_t
+        dev = states.device
+        ds = dstates.to(kdt).contiguous()
+        with torch.cuda.device(dev):
+            dWx = torch.empty((B, T, Gw, N, D), dtype=kdt, device=dev)
+            ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
+            dR = torch.empty((Gr, N, D, D), dtype=torch.float32, device=dev)
+            db = torch.empty((Gt, N, D), dtype=torch.float32, device=dev)
+            ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 1)
+            ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+            stream = torch.cuda.current_stream().cuda_stream
+            rc = _entry(cfg.backend, "backward")(
+                f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
+                cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
+                ws.data_ptr(), ws.numel(), stream)
+            if rc != 0:
+                _raise(rc, f"{cfg.backend} backward")
+        _last_workspace["backward"] = ws
+        # dR / db stay fp32: autograd casts them to the dtype of the leaf they belong to, so fp32
+        # master weights receive unrounded gradients
+        return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None
+
+
+def _get_config(Wx, R, b, function, backend, dtype) -> FlashRNNConfig:
+    return FlashRNNConfig(head_dim=Wx.shape[4], num_heads=Wx.shape[3], batch_size=Wx.shape[0],
+                          function=function, backend=backend,
+                          dtype=dtype if dtype is not None else "bfloat16")
+
+
+def _zero_state(config: FlashRNNConfig, Wx: torch.Tensor) -> torch.Tensor:
+    """[S,B,1,N,D] zeros like the reference's _zero_state (flashrnn.py:927-954)."""
+    B, _, _, N, D = Wx.shape
+    return torch.zeros((config.num_states, B, 1, N, D), dtype=Wx.dtype, device=Wx.device)
+
+
+def flashrnn(
+    Wx: torch.Tensor,  # [B, T, G_w, N, D]
+    R: torch.Tensor,  # [G_r, N, D, D]   (gate, head, output unit, previous unit)
+    b: torch.Tensor,  # [G_t, N, D]
+    states: Optional[torch.Tensor] = None,  # [S, B, 1, N, D]
+    function: str = "lstm",
+    config: Optional[FlashRNNConfig] = None,
+    backend: str = "hip_fused",
+    dtype: str = "bfloat16",
+):
+    """Same call as the reference's ``flashrnn`` (flashrnn.py:1114-1135).
+
+    Returns ``(all_states [S,B,T,N,D], last_states [S,B,1,N,D])`` in the kernel dtype ``dtype``.
+    Differentiable w.r.t. Wx, R, b and states.  Raises ValueError if the chosen backend has no
+    kernel for the head dimension (as the reference does when no tiling exists)."""
+    if config is None:
+        config = _get_config(Wx, R, b, function, backend, dtype)
+    Gr, Gw, _, Gt, S = rnn_function_registry[config.function]["gates_states"]
+    if Wx.dim() != 5 or Wx.shape[2] != Gw:
+        raise ValueError(f"Wx must be [B,T,{Gw},N,D], got {tuple(Wx.shape)}")
+    B, T, _, N, D = Wx.shape
+    if tuple(R.shape) != (Gr, N, D, D):
+        raise ValueError(f"R must be [{Gr},{N},{D},{D}], got {tuple(R.shape)}")
+    if tuple(b.shape) != (Gt, N, D):
+        raise ValueError(f"b must be [{Gt},{N},{D}], got {tuple(b.shape)}")
+    if states is None:
+        states = _zero_state(config, Wx)
+    if tuple(states.shape) != (S, B, 1, N, D):
+        raise ValueError(f"states must be [{S},{B},1,{N},{D}], got {tuple(states.shape)}")
+    training = torch.is_grad_enabled() and any(x.requires_grad for x in (Wx, R, b, states))
+    out = _FlashRNNFunction.apply(Wx, R, b, states, config, training)
+    return out, out[:, :, -1:]

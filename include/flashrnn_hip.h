@@ -1,0 +1,126 @@
+/* C ABI of libflashrnn_hip.so: the MI355X (gfx950) recurrent hot path of FlashRNN.
+ *
+ * Each entry point replaces one method of the reference's per-configuration pybind objects
+ *   FlashRNNFuncFused {forward, backward}   flashrnn/flashrnn/fused/flashrnn.cc:55-346
+ *   FlashRNNFunc      {forward, backward}   flashrnn/flashrnn/alternating/flashrnn.cc:39-313
+ * and, below them, ForwardPass::Run / BackwardPass::Run
+ *   flashrnn/flashrnn/fused/flashrnn.h:118-150, flashrnn/flashrnn/alternating/flashrnn.h:48-369.
+ *
+ * Differences in contract (all on purpose):
+ *  - one library for every (function, dtype, head dim): the configuration is passed at run
+ *    time, nothing is JIT-compiled (reference: one nvcc build per config, cuda_init.py:95-168);
+ *  - tensors are read and written in the PUBLIC layouts of flashrnn() (flashrnn.py:165-173):
+ *      Wx [B,T,G_w,N,D]   R [G_r,N,D,D] (out unit, previous unit)   b [G_t,N,D]
+ *      s0 [S,B,N,D]       states [S,B,T,N,D]       dstates [S,B,T,N,D]
+ *    so the caller makes no permuted copies (reference: flashrnn.py:1130-1133, :1053);
+ *  - the batch is padded to the MFMA tile inside the kernels; B is the true batch size
+ *    (reference pads in Python, flashrnn.py:699-717);
+ *  - the library allocates nothing: outputs, the gate cache and a workspace are the caller's,
+ *    sized by the *_bytes queries; every call runs on the stream it is given and is
+ *    asynchronous; there are no device-wide synchronisations
+ *    (reference: cudaDeviceSynchronize in flashrnn_fused_backward.cu:1001);
+ *  - dR and db are returned in fp32 whatever the storage type (reference: storage type).
+ *
+ * All pointers are device pointers, 16-byte aligned, tensors contiguous.  Element type is
+ * bf16 (FRNN_BF16) or fp32 (FRNN_F32) for Wx, R, b, s0, states, dstates, dWx, ds0.
+ *
+ * Return value: 0 ok; negative = argument error found on the host before any launch
+ * (FRNN_E_*; text in frnn_last_error()); positive = hipError_t of a failed launch.
+ */
+#ifndef FLASHRNN_HIP_H
+#define FLASHRNN_HIP_H
+
+#include <stddef.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+/* function ids: gate/state counts as in flashrnn.py:49-71 */
+enum { FRNN_LSTM = 0, FRNN_SLSTM = 1, FRNN_GRU = 2, FRNN_ELMAN = 3 };
+enum { FRNN_BF16 = 0, FRNN_F32 = 1 };
+
+enum {
+  FRNN_OK = 0,
+  FRNN_E_ARG = -1,         /* unknown function / dtype, non-positive size */
+  FRNN_E_UNSUPPORTED = -2, /* no kernel for this (function, dtype, D); use the other backend */
+  FRNN_E_NULL = -3,        /* a required pointer is null */
+  FRNN_E_ALIGN = -4,       /* a pointer is not 16-byte aligned */
+  FRNN_E_WORKSPACE = -5,   /* workspace smaller than frnn_*_workspace_bytes() */
+  FRNN_E_DEVICE = -6       /* current device is not usable (query failed, too few CUs) */
+};
+
+/* Thread-local text of the last error returned on this thread ("" if none). */
+const char* frnn_last_error(void);
+const char* frnn_version(void);
+
+/* (G_r, G_w, G_t, S) of a function and the number of values per element the gate cache
+ * holds; 0 ok / FRNN_E_ARG.  Mirrors rnn_function_registry, flashrnn.py:49-71. */
+int frnn_function_dims(int function, int* G_r, int* G_w, int* G_t, int* S, int* cache_vals);
+
+/* ---- fused backend ("hip_fused"): replaces FlashRNNFuncFused, fused/flashrnn.cc:55-346 ---- */
+
+/* 0 if a fused kernel exists for (function, dtype, D) and B,N fit the device, else FRNN_E_*.
+ * Replaces the reference's "does a tiling exist" search (flashrnn.py:429-589). */
+int frnn_fused_supported(int function, int dtype, int B, int N, int D);
+
+/* The launch plan: waves per workgroup, 16-unit tiles per wave, workgroups per head and the
+ * number of workgroups that do work (= compute units used).  backward = 0/1. */
+int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
+                    int* waves, int* tiles_per_wave, int* wgs_per_head, int* active_wgs);
+
+/* Bytes of the private gate cache written by a training forward and read by backward
+ * (reference: gate_cache_r / gate_cache_i, fused/flashrnn.cc:97-112). */
+size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int D);
+
+/* Bytes of workspace for forward (backward = 0) or backward (backward = 1).  The first
+ * 4 bytes of the workspace hold a status word after the call: 0 ok, 1 = a bounded wait
+ * between workgroups ran out (the outputs are then filled with NaN from that step on). */
+size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward);
+
+/* Forward over the whole sequence.  Replaces FlashRNNFuncFused::forward (fused/flashrnn.cc:68-144)
+ * + ForwardPass::Run (fused/flashrnn_fused_forward.cu:772-975).
+ *   training != 0: also fills `cache` (frnn_fused_cache_bytes); else cache may be null.
+ *   states [S,B,T,N,D] receives s_1..s_T (s0 is NOT copied in front, unlike the reference's
+ *   [S,T+1,B,N,D] buffer). */
+int frnn_fused_forward(int function, int dtype, int training, int B, int T, int N, int D,
+                       const void* Wx, const void* R, const void* b, const void* s0,
+                       void* states, void* cache, void* workspace, size_t workspace_bytes,
+                       void* stream);
+
+/* Backward.  Replaces FlashRNNFuncFused::backward (fused/flashrnn.cc:146-246) +
+ * BackwardPass::Run (fused/flashrnn_fused_backward.cu:768-1086) including its post-loop
+ * dR GEMM (:1049-1055) and bias reduction (:626-665).
+ *   dstates [S,B,T,N,D]: cotangent of every output state.
+ *   outputs: dWx [B,T,G_w,N,D], ds0 [S,B,N,D] (storage type); dR [G_r,N,D,D], db [G_t,N,D] (fp32). */
+int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
+                        const void* R, const void* b, const void* s0, const void* states,
+                        const void* cache, const void* dstates,
+                        void* dWx, void* ds0, float* dR, float* db,
+                        void* workspace, size_t workspace_bytes, void* stream);
+
+/* ---- alternating backend ("hip"): replaces FlashRNNFunc, alternating/flashrnn.cc:39-313 ---- */
+
+int frnn_alt_supported(int function, int dtype, int B, int N, int D);
+size_t frnn_alt_cache_bytes(int function, int dtype, int B, int T, int N, int D);
+size_t frnn_alt_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward);
+
+/* Per time step: one MFMA GEMM kernel (R h_{t-1} for all heads) then one pointwise kernel.
+ * Replaces ForwardPass::Run / IterateInternal, alternating/flashrnn_forward.cu:150-267. */
+int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N, int D,
+                     const void* Wx, const void* R, const void* b, const void* s0,
+                     void* states, void* cache, void* workspace, size_t workspace_bytes,
+                     void* stream);
+
+/* Per reverse step: pointwise adjoint kernel then MFMA GEMM (R^T dg); then dR GEMM and bias
+ * reduction.  Replaces BackwardPass::Run, alternating/flashrnn_backward.cu:267-431. */
+int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
+                      const void* R, const void* b, const void* s0, const void* states,
+                      const void* cache, const void* dstates,
+                      void* dWx, void* ds0, float* dR, float* db,
+                      void* workspace, size_t workspace_bytes, void* stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif /* FLASHRNN_HIP_H */
