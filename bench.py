@@ -1,0 +1,199 @@
+#!/usr/bin/env python3
+"""Benchmark of the recurrent hot path on one MI355X.
+
+    python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--backend hip_fused]
+
+A step is one forward + backward pass of ``flashrnn()`` over one batch of synthetic input that is
+already resident in HBM.  Prints ONE JSON line: tokens/s (B*T per second) of the whole job, the
+roofline figures of the dominant kernel (measured with HIP events on the launch stream inside the
+timed region), the same workload on the alternating backend, and the CPU oracle timed on the host.
+"""
+import argparse
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+# name -> workload; seeds fixed per config.  C2 is the configuration the metric is quoted on.
+WORKLOADS = {
+    "C1": dict(function="lstm", dtype="float32", B=4, T=256, N=1, D=64, init="zeros", grad_on="all", bwd=False, seed=1001),
+    "C2": dict(function="lstm", dtype="bfloat16", B=8, T=1024, N=3, D=256, init="randn", grad_on="all", bwd=True, seed=1002),
+    "C3": dict(function="gru", dtype="bfloat16", B=16, T=2048, N=4, D=128, init="zeros", grad_on="all", bwd=True, seed=1003),
+    "C4": dict(function="slstm", dtype="bfloat16", B=16, T=4096, N=4, D=192, init="zeros", grad_on="h", bwd=True, seed=1004,
+               forget_bias_linspace=True),
+    "C5": dict(function="elman", dtype="bfloat16", B=32, T=1024, N=1, D=1024, init="zeros", grad_on="all", bwd=True, seed=1005),
+}
+GATES_R = {"lstm": 4, "slstm": 4, "gru": 3, "elman": 1}
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, published
+
+
+def describe(w):
+    return (f"{w['function']} {w['dtype']} B{w['B']} T{w['T']} N{w['N']} D{w['D']} "
+            f"{'fwd+bwd' if w['bwd'] else 'fwd'}")
+
+
+def make_gpu_inputs(w, device):
+    import torch
+    from oracle import make_inputs
+
+    rt = torch.bfloat16 if w["dtype"] == "bfloat16" else None
+    inp = make_inputs(w["function"], w["B"], w["T"], w["N"], w["D"], w["seed"], init=w["init"], round_to=rt,
+                      grad_on=w["grad_on"], forget_bias_linspace=w.get("forget_bias_linspace", False))
+    kdt = torch.bfloat16 if w["dtype"] == "bfloat16" else torch.float32
+    dev = {k: v.to(device=device, dtype=kdt) for k, v in inp.items()}
+    return inp, dev
+
+
+def _launches_per_step(w, backend):
+    """Profile entries one step produces (see the prof_begin calls of the C library)."""
+    if backend == "hip_fused":
+        return 2 + (5 if w["bwd"] else 0)
+    return 1 + (5 if w["bwd"] else 0)
+
+
+def run_gpu(w, backend, steps, warmup, device):
+    """Returns (ms_per_step, {kernel name: (avg ms, launches per step)})."""
+    import torch
+    from flashrnn_amd import flashrnn, load_library
+
+    lib = load_library()
+    _, dev = make_gpu_inputs(w, device)
+    leaves = [dev[k].requires_grad_(w["bwd"]) for k in ("Wx", "R", "b", "states")]
+    dst = dev["dstates"]
+
+    def step():
+        out, _ = flashrnn(*leaves, function=w["function"], backend=backend, dtype=w["dtype"])
+        if w["bwd"]:
+            torch.autograd.grad(out, leaves, grad_outputs=dst)
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    # HIP events around every kernel launch, recorded on the launch stream inside the timed
+    # region; the library keeps the most recent 64 launches, read after the region ends
+    lib.frnn_profile_enable(1)
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    per_kernel = {}
+    held = lib.frnn_profile_count()
+    for i in range(held):
+        per_kernel.setdefault(lib.frnn_profile_name(i).decode(), []).append(lib.frnn_profile_ms(i))
+    lib.frnn_profile_enable(0)
+    calls = max(1, min(steps, held // max(1, _launches_per_step(w, backend))))
+    kern = {k: (sum(v) / len(v), max(1, round(len(v) / calls))) for k, v in per_kernel.items()}
+    return (t1 - t0) * 1e3 / steps, kern
+
+
+def run_cpu_baseline(w, budget_s=12.0):
+    """The CPU oracle (a port of the reference's vanilla backend) on the host cores, fp32."""
+    import torch
+    from oracle import flashrnn_oracle, make_inputs
+
+    torch.set_num_threads(os.cpu_count() or 1)
+    rt = torch.bfloat16 if w["dtype"] == "bfloat16" else None
+    inp = make_inputs(w["function"], w["B"], w["T"], w["N"], w["D"], w["seed"], init=w["init"], round_to=rt,
+                      grad_on=w["grad_on"], forget_bias_linspace=w.get("forget_bias_linspace", False))
+
+    def one():
+        leaves = [inp[k].clone().requires_grad_(w["bwd"]) for k in ("Wx", "R", "b", "states")]
+        out, _ = flashrnn_oracle(*leaves, function=w["function"], slstm_per_element_first_step=True)
+        if w["bwd"]:
+            torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"])
+
+    t0 = time.perf_counter()
+    one()  # warm-up, also tells us how many repetitions fit the budget
+    first = time.perf_counter() - t0
+    reps = max(1, min(5, int(budget_s / max(first, 1e-3))))
+    times = []
+    for _ in range(reps):
+        t0 = time.perf_counter()
+        one()
+        times.append(time.perf_counter() - t0)
+    med = sorted(times)[len(times) // 2]
+    return dict(value=w["B"] * w["T"] / med, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"full workload ({describe(w)}), fp32 torch CPU, median of {reps} after 1 warm-up",
+                ms=med * 1e3)
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=20)
+    ap.add_argument("--warmup", type=int, default=5)
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--backend", default=None, choices=["hip_fused", "hip"])
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-alt", action="store_true", help="skip the other-backend comparison leg")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: the recurrent path has no multi-GPU leg in this build "
+              "(heads and batch rows shard without per-step communication); run with --gpus 1", file=sys.stderr)
+        sys.exit(2)
+
+    import torch
+
+    if not torch.cuda.is_available():
+        print("bench.py needs a GPU (flashrnn_amd has no CPU path)", file=sys.stderr)
+        sys.exit(2)
+    device = torch.device("cuda:0")
+    w = WORKLOADS[args.workload]
+    backend = args.backend or ("hip" if args.workload == "C5" else "hip_fused")
+    tokens = w["B"] * w["T"]
+
+    ms, kern = run_gpu(w, backend, args.steps, args.warmup, device)
+
+    # dominant kernel and its roofline: 2*N*G_r*D^2 flops per token in the forward scan and the
+    # same in the reverse scan (dh = R^T dg) and in the dR GEMM
+    flops_scan = 2.0 * w["N"] * GATES_R[w["function"]] * w["D"] ** 2 * tokens
+    algo = {"fused_fwd_kernel": flops_scan, "fused_bwd_kernel": flops_scan, "grad_gemm_kernel": flops_scan,
+            "alt_forward_steps": flops_scan, "alt_backward_steps": flops_scan}
+    cand = {k: v for k, v in kern.items() if k in algo}
+    dom = max(cand, key=lambda k: cand[k][0] * cand[k][1])
+    dom_ms = cand[dom][0]
+    peak = PEAK_TFLOPS[w["dtype"]]
+    achieved = algo[dom] / cand[dom][1] / (dom_ms * 1e-3) / 1e12
+    roofline = dict(kernel=dom, bound="mfma", achieved=achieved, peak=peak, unit="TFLOP/s", frac=achieved / peak,
+                    traffic=None, avg_launch_ms=dom_ms, launches_per_step=cand[dom][1],
+                    us_per_time_step=dom_ms * 1e3 / w["T"])
+    try:
+        from flashrnn_amd import fused_plan
+
+        if backend == "hip_fused":
+            wv, utw, kw, active = fused_plan(w["function"], w["dtype"], w["B"], w["N"], w["D"], dom == "fused_bwd_kernel")
+            roofline.update(compute_units_used=active, wgs_per_head=kw,
+                            frac_of_used_cus=achieved / (peak * active / 256.0))
+    except Exception:  # plan query is informational only
+        pass
+
+    out = {
+        "metric": "tokens/s fwd+bwd, LSTM bf16 B8 T1024 N3 D256; MFMA util vs peak" if args.workload == "C2"
+                  else f"tokens/s {describe(w)}",
+        "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16" if w["dtype"] == "bfloat16" else "f32", "data": "synthetic",
+        "config": {"workload": f"{args.workload}: {describe(w)}", "backend": backend, "seed": w["seed"],
+                   "timed": "flashrnn() + torch.autograd.grad through the C ABI, inputs resident in HBM"},
+        "roofline": roofline,
+        "kernels_ms": {k: {"avg_ms": v[0], "per_step": v[1]} for k, v in kern.items()},
+    }
+    if not args.no_alt and w["bwd"]:
+        other = "hip" if backend == "hip_fused" else "hip_fused"
+        try:
+            ms_o, _ = run_gpu(w, other, max(3, args.steps // 4), 2, device)
+            out["other_backend"] = {"backend": other, "ms_per_step": ms_o, "tokens_per_s": tokens / (ms_o * 1e-3),
+                                    "speedup_of_" + backend: ms_o / ms}
+        except ValueError as e:  # no kernel of the other backend for this head dim
+            out["other_backend"] = {"backend": other, "error": str(e)}
+    if not args.no_cpu:
+        out["cpu_baseline"] = run_cpu_baseline(w)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()

@@ -19,6 +19,11 @@ _P6 = [c_int] * 6
 _SIGNATURES = {
     "frnn_last_error": (c_char_p, []),
     "frnn_version": (c_char_p, []),
+    "frnn_profile_enable": (None, [c_int]),
+    "frnn_profile_reset": (None, []),
+    "frnn_profile_count": (c_int, []),
+    "frnn_profile_name": (c_char_p, [c_int]),
+    "frnn_profile_ms": (ctypes.c_float, [c_int]),
     "frnn_function_dims": (c_int, [c_int] + [POINTER(c_int)] * 5),
     "frnn_fused_supported": (c_int, [c_int] * 5),
     "frnn_fused_plan": (c_int, [c_int] * 6 + [POINTER(c_int)] * 4),

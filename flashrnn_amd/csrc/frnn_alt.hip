@@ -90,13 +90,15 @@ __global__ void __launch_bounds__(256) alt_pw_fwd_kernel(const AltPwArgs a) {
   const T* bias = static_cast<const T*>(a.b);
   const T* s0 = static_cast<const T*>(a.s0);
   T* states = static_cast<T*>(a.states);
-  float ry[GR], wx[GW], bb[GT], s[S], cc[NC > 0 ? NC : 1];
+  float ry[GR], wx[GW], bb[GT - GR + 1], s[S], cc[NC > 0 ? NC : 1];
 #pragma unroll
   for (int g = 0; g < GR; ++g) ry[g] = a.ry[((size_t)b * N + n) * GR * D + (size_t)g * D + d];
 #pragma unroll
   for (int g = 0; g < GW; ++g) wx[g] = ld(Wx + (((size_t)b * Tn + t) * GW + g) * ND + (size_t)n * D + d);
 #pragma unroll
-  for (int g = 0; g < GT; ++g) bb[g] = ld(bias + (size_t)(g * N + n) * D + d);
+  for (int g = 0; g < GR; ++g) ry[g] += ld(bias + (size_t)(g * N + n) * D + d);
+#pragma unroll
+  for (int g = GR; g < GT; ++g) bb[g - GR] = ld(bias + (size_t)(g * N + n) * D + d);
 #pragma unroll
   for (int k = 0; k < S; ++k)
     s[k] = t > 0 ? ld(states + (((size_t)k * B + b) * Tn + t - 1) * ND + (size_t)n * D + d)

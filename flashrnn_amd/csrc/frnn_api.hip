@@ -29,6 +29,35 @@ static int hip_fail(int e, const char* what) {
   return e;
 }
 
+// ---- optional per-launch timing with HIP events on the caller's stream ---------------------------
+// Off by default.  When on, every kernel launch (or launch loop) of a call is bracketed by two
+// events; frnn_profile_ms() waits for them.  Meant for benchmarks: one thread, one stream.
+struct ProfRec { const char* name; hipEvent_t a, b; };
+static const int kProfMax = 64;  // ring: the most recent kProfMax launches are kept
+static ProfRec g_prof[kProfMax];
+static long g_prof_n = 0;
+static int g_prof_on = 0, g_prof_events = 0;
+static void prof_begin(const char* name, hipStream_t st) {
+  if (!g_prof_on) return;
+  const int i = (int)(g_prof_n % kProfMax);
+  if (g_prof_events <= i) {
+    if (hipEventCreate(&g_prof[i].a) != hipSuccess || hipEventCreate(&g_prof[i].b) != hipSuccess) { g_prof_on = 0; return; }
+    g_prof_events = i + 1;
+  }
+  g_prof[i].name = name;
+  hipEventRecord(g_prof[i].a, st);
+}
+static void prof_end(hipStream_t st) {
+  if (!g_prof_on) return;
+  hipEventRecord(g_prof[(int)(g_prof_n % kProfMax)].b, st);
+  ++g_prof_n;
+}
+static int prof_slot(int i) {  // i-th oldest entry still held -> ring slot, or -1
+  const long held = g_prof_n < kProfMax ? g_prof_n : kProfMax;
+  if (i < 0 || i >= held) return -1;
+  return (int)((g_prof_n - held + i) % kProfMax);
+}
+
 // ---- plan table -------------------------------------------------------------------------------
 #define FRNN_ROW(Dv, VAR, W, U, K) {Dv, VAR, W, U, K},
 static const Plan kFwd4B[] = {FRNN_PLANS_GR4_BF16(FRNN_ROW)};
@@ -99,6 +128,16 @@ static int check_problem(int function, int dtype, int B, int T, int N, int D) {
   if ((long)B * T >= (1L << 31)) return fail(FRNN_E_ARG, "B*T too large");
   return 0;
 }
+// the fused kernels address each tensor with 32-bit byte offsets
+static int check_fused_sizes(int function, int dtype, int B, int T, int N, int D) {
+  const CellDims c = cell_dims(function);
+  const size_t es = dtype_size(dtype), btnd = (size_t)B * T * N * D;
+  const size_t gmax = (size_t)(c.GW > c.S ? c.GW : c.S);
+  const size_t cache = (size_t)T * N * ((B + 15) / 16) * 16 * D * c.NC * es;
+  if (btnd * gmax * es >= ((size_t)1 << 31) || cache >= ((size_t)1 << 31))
+    return fail(FRNN_E_ARG, "a tensor of this problem reaches 2 GiB; split the batch (fused kernels use 32-bit offsets)");
+  return 0;
+}
 static int check_ptr(const void* p, const char* name) {
   if (!p) return fail(FRNN_E_NULL, "%s is null", name);
   if (((uintptr_t)p) & 15) return fail(FRNN_E_ALIGN, "%s is not 16-byte aligned", name);
@@ -114,7 +153,7 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   w.status = (int*)bp.take(256);
   const size_t groups = (size_t)N * ((B + 15) / 16);
   const size_t llw = (size_t)16 * D / (dtype == FRNN_BF16 ? 2 : 1);
-  w.ll = (u64*)bp.take(p.kw > 1 ? groups * 2 * llw * 8 : 0);
+  w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
   w.zero_bytes = bp.off;  // status + exchange slots must start at zero for every call
   w.total = bp.off;
   return w;
@@ -127,7 +166,7 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   FusedBwdWs w;
   w.status = (int*)bp.take(256);
   const size_t bt = (B + 15) / 16, groups = (size_t)N * bt;
-  w.ll = (u64*)bp.take(p.kw > 1 ? groups * 2 * bwd_inbox_words(D, p.kw) * 8 : 0);
+  w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * bwd_inbox_words(D, p.kw) * 8 : 0);
   w.zero_bytes = bp.off;
   w.Rt = bp.take((size_t)N * D * c.GR * D * es);
   w.dgx = bp.take(function == FRNN_GRU ? (size_t)B * T * N * D * es : 0);
@@ -165,9 +204,13 @@ static int weight_grads(int function, int dtype, int B, int T, int N, int D, con
   }
   g.states_h = states; g.s0_h = s0; g.part = part;
   g.B = B; g.T = T; g.N = N; g.D = D; g.GR = c.GR;
+  prof_begin("grad_gemm_kernel", st);
   int e = launch_grad_gemm(dtype, g, splits, st);
+  prof_end(st);
   if (e) return hip_fail(e, "dR gemm");
+  prof_begin("grad_reduce_kernel", st);
   e = launch_grad_reduce(part, splits, (size_t)c.GR * N * D * D, dR, dbp, db_splits, (size_t)c.GT * ND, db, st);
+  prof_end(st);
   if (e) return hip_fail(e, "gradient reduction");
   return 0;
 }
@@ -180,6 +223,19 @@ extern "C" {
 
 const char* frnn_last_error(void) { return g_err; }
 const char* frnn_version(void) { return "flashrnn_hip 0.1 (gfx950)"; }
+
+void frnn_profile_enable(int on) { g_prof_on = on ? 1 : 0; g_prof_n = 0; }
+void frnn_profile_reset(void) { g_prof_n = 0; }
+int frnn_profile_count(void) { return (int)(g_prof_n < kProfMax ? g_prof_n : kProfMax); }
+const char* frnn_profile_name(int i) { const int k = prof_slot(i); return k < 0 ? "" : g_prof[k].name; }
+float frnn_profile_ms(int i) {
+  const int k = prof_slot(i);
+  if (k < 0) return -1.0f;
+  float ms = -1.0f;
+  if (hipEventSynchronize(g_prof[k].b) != hipSuccess) return -1.0f;
+  if (hipEventElapsedTime(&ms, g_prof[k].a, g_prof[k].b) != hipSuccess) return -1.0f;
+  return ms;
+}
 
 int frnn_function_dims(int function, int* G_r, int* G_w, int* G_t, int* S, int* cache_vals) {
   if (function < 0 || function > 3) return fail(FRNN_E_ARG, "unknown function id %d", function);
@@ -239,13 +295,17 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
   Plan p;
   if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  e = check_fused_sizes(function, dtype, B, T, N, D);
+  if (e) return e;
   CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
   const bool need_cache = training && cell_dims(function).NC > 0;
   if (need_cache) CHECK_PTR(cache)
   const FusedFwdWs w = carve_fused_fwd(workspace, dtype, B, N, D, p);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
+  prof_begin("fill_zero_kernel", st);
   e = launch_fill_zero(workspace, w.zero_bytes, st);
+  prof_end(st);
   if (e) return hip_fail(e, "workspace clear");
   const int groups = N * ((B + 15) / 16);
   int per_launch = groups;
@@ -261,12 +321,14 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
+    prof_begin("fused_fwd_kernel", st);
     switch (function) {
       case FRNN_LSTM:  e = fused_fwd_dispatch<FRNN_LSTM>(dtype, p, a, st); break;
       case FRNN_SLSTM: e = fused_fwd_dispatch<FRNN_SLSTM>(dtype, p, a, st); break;
       case FRNN_GRU:   e = fused_fwd_dispatch<FRNN_GRU>(dtype, p, a, st); break;
       default:         e = fused_fwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
     }
+    prof_end(st);
     if (e) return hip_fail(e, "fused forward launch");
   }
   return 0;
@@ -285,15 +347,21 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
   Plan p;
   if (!find_plan(c.GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  e = check_fused_sizes(function, dtype, B, T, N, D);
+  if (e) return e;
   CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
   CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
   if (c.NC > 0) CHECK_PTR(cache)
   const FusedBwdWs w = carve_fused_bwd(workspace, function, dtype, B, T, N, D, p);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
+  prof_begin("fill_zero_kernel", st);
   e = launch_fill_zero(workspace, w.zero_bytes, st);
+  prof_end(st);
   if (e) return hip_fail(e, "workspace clear");
+  prof_begin("transpose_r_kernel", st);
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
+  prof_end(st);
   if (e) return hip_fail(e, "R transpose");
   const int bt = (B + 15) / 16, groups = N * bt;
   int per_launch = groups;
@@ -309,12 +377,14 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
+    prof_begin("fused_bwd_kernel", st);
     switch (function) {
       case FRNN_LSTM:  e = fused_bwd_dispatch<FRNN_LSTM>(dtype, p, a, st); break;
       case FRNN_SLSTM: e = fused_bwd_dispatch<FRNN_SLSTM>(dtype, p, a, st); break;
       case FRNN_GRU:   e = fused_bwd_dispatch<FRNN_GRU>(dtype, p, a, st); break;
       default:         e = fused_bwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
     }
+    prof_end(st);
     if (e) return hip_fail(e, "fused backward launch");
   }
   return weight_grads(function, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, bt, dR, db, st);
@@ -379,7 +449,9 @@ int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N,
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0};
   AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.ry};
+  prof_begin("alt_forward_steps", (hipStream_t)stream);
   e = alt_forward(p, bf, (hipStream_t)stream);
+  prof_end((hipStream_t)stream);
   return e ? hip_fail(e, "alternating forward launch") : 0;
 }
 
@@ -404,7 +476,9 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
   if (e) return hip_fail(e, "R transpose");
   AltProblem p{function, dtype, B, T, N, D, 1};
   AltBwdBuffers bf{w.Rt, s0, states, cache, dstates, dWx, w.dgx, ds0, w.dg, w.dsr, w.dh};
+  prof_begin("alt_backward_steps", st);
   e = alt_backward_scan(p, bf, st);
+  prof_end(st);
   if (e) return hip_fail(e, "alternating backward launch");
   // bias partial sums over (b,t) rows; sources per bias gate
   const size_t es = dtype_size(dtype), ND = (size_t)N * D;
@@ -418,7 +492,9 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
       src[g] = (const char*)dWx + (size_t)g * ND * es; ld[g] = (long)(c.GW * ND);
     }
   }
+  prof_begin("alt_bias_kernel", st);
   e = launch_bias_partial(dtype, src, ld, c.GT, N, D, (long)B * T, w.bsplits, w.dbp, st);
+  prof_end(st);
   if (e) return hip_fail(e, "bias partial sums");
   return weight_grads(function, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, w.bsplits, dR, db, st);
 }

@@ -81,21 +81,72 @@ __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest e
   return (unsigned short)(u >> 16);
 }
 
-// 4 consecutive elements <-> 4 floats
+// ---------------------------------------------------------------------------------------
+// E consecutive elements of the storage type as NDW dwords (bf16: two per dword, f32: one).
+// ---------------------------------------------------------------------------------------
+template <int N> struct Dw { unsigned v[N]; };
+template <typename T, int E> struct NDW { static constexpr int value = E * (int)sizeof(T) / 4; };
+
+typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
+typedef float f32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {  // v_cvt_pk_bf16_f32, round to nearest even
+  const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
+  return __builtin_bit_cast(unsigned, h);
+}
+template <int E> __device__ __forceinline__ void unpack(const Dw<E / 2>& d, float* o, bf16_t*) {
+#pragma unroll
+  for (int k = 0; k < E / 2; ++k) { o[2 * k] = __uint_as_float(d.v[k] << 16); o[2 * k + 1] = __uint_as_float(d.v[k] & 0xffff0000u); }
+}
+template <int E> __device__ __forceinline__ void unpack(const Dw<E>& d, float* o, float*) {
+#pragma unroll
+  for (int k = 0; k < E; ++k) o[k] = __uint_as_float(d.v[k]);
+}
+template <int E> __device__ __forceinline__ Dw<E / 2> pack(const float* i, bf16_t*) {
+  Dw<E / 2> d;
+#pragma unroll
+  for (int k = 0; k < E / 2; ++k) d.v[k] = pack_bf16x2(i[2 * k], i[2 * k + 1]);
+  return d;
+}
+template <int E> __device__ __forceinline__ Dw<E> pack(const float* i, float*) {
+  Dw<E> d;
+#pragma unroll
+  for (int k = 0; k < E; ++k) d.v[k] = __float_as_uint(i[k]);
+  return d;
+}
+
+// ---------------------------------------------------------------------------------------
+// Raw buffer access: one descriptor per tensor in SGPRs, 32-bit byte offsets.  An offset at or
+// beyond the tensor's size makes a load return 0 and drops a store, so padded batch rows need
+// no branch; kInvalidOff keeps such a lane out of range for any scalar offset below 2 GiB,
+// which is why tensors handed to the fused kernels must be smaller than 2 GiB.
+// ---------------------------------------------------------------------------------------
+typedef __amdgpu_buffer_rsrc_t rsrc_t;
+constexpr unsigned kInvalidOff = 0x80000000u;
+__device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
+  return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(bytes > 0x7fffffffu ? 0x7fffffffu : bytes), 0x00020000);
+}
+template <int N> __device__ __forceinline__ Dw<N> buf_load(rsrc_t r, unsigned voff, unsigned soff) {
+  Dw<N> d;
+  if constexpr (N == 1) { d.v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0); }
+  else if constexpr (N == 2) { const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0); d.v[0] = t.x; d.v[1] = t.y; }
+  else { static_assert(N == 4, "1, 2 or 4 dwords"); const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); d.v[0] = t.x; d.v[1] = t.y; d.v[2] = t.z; d.v[3] = t.w; }
+  return d;
+}
+template <int N> __device__ __forceinline__ void buf_store(const Dw<N>& d, rsrc_t r, unsigned voff, unsigned soff) {
+  if constexpr (N == 1) { __builtin_amdgcn_raw_buffer_store_b32(d.v[0], r, voff, soff, 0); }
+  else if constexpr (N == 2) { __builtin_amdgcn_raw_buffer_store_b64(u32x2{d.v[0], d.v[1]}, r, voff, soff, 0); }
+  else { static_assert(N == 4, "1, 2 or 4 dwords"); __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[0], d.v[1], d.v[2], d.v[3]}, r, voff, soff, 0); }
+}
+
+// 4 consecutive elements <-> 4 floats (vector form, used outside the time loops)
 __device__ __forceinline__ void unpack4(uint2 v, float* o) {
   o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
   o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
 }
 __device__ __forceinline__ void unpack4(float4 v, float* o) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
-__device__ __forceinline__ void pack4(const float* i, uint2& v) {
-  v.x = (unsigned)f2bf(i[0]) | ((unsigned)f2bf(i[1]) << 16);
-  v.y = (unsigned)f2bf(i[2]) | ((unsigned)f2bf(i[3]) << 16);
-}
-__device__ __forceinline__ void pack4(const float* i, float4& v) { v = make_float4(i[0], i[1], i[2], i[3]); }
-
-// value as it will be seen after a round trip through the storage type
-__device__ __forceinline__ float round_st(float x, bf16_t*) { return bf2f(f2bf(x)); }
-__device__ __forceinline__ float round_st(float x, float*) { return x; }
 
 // ---------------------------------------------------------------------------------------
 // Tagged exchange words ("data + step tag in one store"): a reader that sees the tag of the
@@ -106,8 +157,8 @@ __device__ __forceinline__ float round_st(float x, float*) { return x; }
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned tag16(int t) { return (unsigned)(t % 65535) + 1u; }
 __device__ __forceinline__ u64 ll_pack(bf16_t*, float a, float b, int t) {
-  unsigned tg = tag16(t) << 16;
-  return (u64)(tg | f2bf(a)) | ((u64)(tg | f2bf(b)) << 32);
+  const unsigned tg = tag16(t) << 16, ab = pack_bf16x2(a, b);
+  return (u64)(tg | (ab & 0xffffu)) | ((u64)(tg | (ab >> 16)) << 32);
 }
 __device__ __forceinline__ u64 ll_pack(float*, float a, int t) {
   return (u64)__float_as_uint(a) | ((u64)(unsigned)(t + 1) << 32);

@@ -1,38 +1,66 @@
-// Moving the per-step vector (h_{t-1} forward, dg_t backward) to every wave that needs it
-// as an MFMA operand.
+// Moving the per-step vector to every wave that needs it as an MFMA operand, and the lane
+// ownership of the MFMA result.
 //
-// Within one workgroup the vector lives in LDS in MFMA fragment order, so a lane's operand
-// for k-step ks is one contiguous read at (ks*64 + lane).  Between the KW workgroups of one
-// head it travels through a small global buffer of tagged words: the producer's store carries
-// data and step tag together, the consumer polls the words it needs until the tag matches and
-// copies the payload to LDS.  That costs one L2 round trip instead of the store -> fence ->
-// flag -> poll -> fence -> load chain of a flag barrier.  Two slots alternate by step parity:
-// a workgroup can only write step t+2 after it has read all of step t+1, which every workgroup
-// wrote only after reading step t, so slot (t & 1) is never overwritten while still in use.
+// Within one workgroup the vector (h_{t-1} forward, the own dg_t backward) lives in LDS in MFMA
+// fragment order, so a lane's operand for k-step ks is one contiguous read at (ks*64 + lane).
+// Between the KW workgroups of one head data travels through small global buffers of tagged
+// words: the producer's store carries data and step tag together, the consumer polls the words
+// it needs until the tag matches.  That costs one trip through the coherent memory path instead
+// of the store -> fence -> flag -> poll -> fence -> load chain of a flag barrier.  Two slots
+// alternate by step parity: a workgroup can only write step t+2 after it has read all of step
+// t+1, which every workgroup wrote only after reading step t, so slot (t & 1) is never
+// overwritten while still in use.  Accesses are agent scope: workgroup-scope loads are served
+// from the per-CU L1 and never see another compute unit's store (measured), and agent scope
+// costs the same ~0.45 us per hop whether or not the two workgroups share an XCD.
+//
+// Ownership.  The 16x16 MFMA result gives lane l the 4 rows 4*(l/16)..+3 of column l%16, i.e.
+// (with A = weight rows, B = streamed vector) 4 consecutive units of batch row l%16.
+//   FULL: a lane keeps its 4 elements.
+//   HALF (batch <= 8): columns 8..15 are padding, so lanes 8..15 of every 16-lane row take
+//   elements 2,3 of the lane 8 below them (one DPP move each) and every lane does the gate
+//   math of 2 elements instead of 4.
 #pragma once
 #include "frnn_common.h"
 
 namespace frnn {
 
-// LDS writes of 4 consecutive elements (row, k0..k0+3), k0 % 4 == 0, in fragment order
-__device__ __forceinline__ void lds_write4(bf16_t* buf, int row, int k0, const float* v) {
-  uint2 p; pack4(v, p);
-  *reinterpret_cast<uint2*>(buf + ST<bf16_t>::frag_elem(row, k0)) = p;
+template <bool HALF> struct Own {
+  static constexpr int E = HALF ? 2 : 4;  // elements per lane per 16-unit tile
+  static __device__ __forceinline__ int row(int r16) { return HALF ? (r16 & 7) : r16; }              // batch row in the tile
+  static __device__ __forceinline__ int sub(int r16, int q4) { return q4 * 4 + (HALF ? 2 * (r16 >> 3) : 0); }  // first unit in the tile
+};
+
+// HALF: lanes 0..7 of a row keep `lo`, lanes 8..15 receive `hi` of the lane 8 below (row_shr:8)
+__device__ __forceinline__ float half_pick(float lo, float hi) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, lo), __builtin_bit_cast(int, hi),
+                                                              0x118, 0xF, 0xC, false));
 }
-__device__ __forceinline__ void lds_write4(float* buf, int row, int k0, const float* v) {
-#pragma unroll
-  for (int i = 0; i < 4; ++i) buf[ST<float>::frag_elem(row, k0 + i)] = v[i];
+template <bool HALF> __device__ __forceinline__ void own_elems(const f32x4& acc, float* out) {
+  if constexpr (HALF) { out[0] = half_pick(acc[0], acc[2]); out[1] = half_pick(acc[1], acc[3]); }
+  else { out[0] = acc[0]; out[1] = acc[1]; out[2] = acc[2]; out[3] = acc[3]; }
 }
 
-// tagged global stores of 4 consecutive elements (row, k0..k0+3) for step t
-__device__ __forceinline__ void ll_write4(bf16_t*, u64* slot, int row, int k0, const float* v, int t) {
-  const int q = ST<bf16_t>::frag_elem(row, k0) >> 1;
-  ll_store(slot + q, ll_pack((bf16_t*)0, v[0], v[1], t));
-  ll_store(slot + q + 1, ll_pack((bf16_t*)0, v[2], v[3], t));
+// LDS writes of E consecutive elements (row, k0..k0+E-1) in fragment order; k0 % E == 0
+template <int E> __device__ __forceinline__ void lds_write(bf16_t* buf, int row, int k0, const float* v) {
+  const Dw<E / 2> p = pack<E>(v, (bf16_t*)0);
+  unsigned* dst = reinterpret_cast<unsigned*>(buf + ST<bf16_t>::frag_elem(row, k0));
+  if constexpr (E == 4) *reinterpret_cast<uint2*>(dst) = make_uint2(p.v[0], p.v[1]);
+  else dst[0] = p.v[0];
 }
-__device__ __forceinline__ void ll_write4(float*, u64* slot, int row, int k0, const float* v, int t) {
+template <int E> __device__ __forceinline__ void lds_write(float* buf, int row, int k0, const float* v) {
 #pragma unroll
-  for (int i = 0; i < 4; ++i) ll_store(slot + ST<float>::frag_elem(row, k0 + i), ll_pack((float*)0, v[i], t));
+  for (int i = 0; i < E; ++i) buf[ST<float>::frag_elem(row, k0 + i)] = v[i];
+}
+
+// tagged global stores of E consecutive elements (row, k0..) for step t
+template <int E> __device__ __forceinline__ void ll_write(bf16_t*, u64* slot, int row, int k0, const float* v, int t) {
+  const int q = ST<bf16_t>::frag_elem(row, k0) >> 1;
+#pragma unroll
+  for (int k = 0; k < E / 2; ++k) ll_store(slot + q + k, ll_pack((bf16_t*)0, v[2 * k], v[2 * k + 1], t));
+}
+template <int E> __device__ __forceinline__ void ll_write(float*, u64* slot, int row, int k0, const float* v, int t) {
+#pragma unroll
+  for (int i = 0; i < E; ++i) ll_store(slot + ST<float>::frag_elem(row, k0 + i), ll_pack((float*)0, v[i], t));
 }
 
 // The words thread `tid` of NT polls, for a [rows_valid x KDIM] vector; -1 = none.
@@ -81,6 +109,14 @@ __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, 
       if (q[i] >= 0) reinterpret_cast<unsigned*>(lds_dst)[q[i]] = ll_payload((T*)0, v[i]);
   }
   return fail;
+}
+
+// Workgroup barrier that also tells every wave whether any lane passed `fail`; `flag` is one LDS
+// word that starts at 0 and is only ever set.  Costs one LDS read more than a plain barrier.
+__device__ __forceinline__ bool barrier_or(bool fail, volatile int* flag) {
+  if (fail) *flag = 1;
+  __syncthreads();
+  return *flag != 0;
 }
 
 }  // namespace frnn

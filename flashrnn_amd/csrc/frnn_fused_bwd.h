@@ -39,20 +39,20 @@ struct BwdArgs {
   int spin_limit;
 };
 
-// 64-bit words of one inbox slot of one group: [dst wg][wave][tile][src wg][lane][4]
+// 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][lane][4]
 constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) * 256; }
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_at(const T* p);
 template <> __device__ __forceinline__ bf16x8 load_frag_at<bf16_t>(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 template <> __device__ __forceinline__ float load_frag_at<float>(const float* p) { return *p; }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW>
+template <int F, typename T, int D, int WAVES, int UTW, int KW, bool HALF>
 __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
-  typedef typename X::Vec4 Vec4;
   typedef typename X::Frag Frag;
+  typedef Own<HALF> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
   constexpr int NT = WAVES * 64, UT_WG = WAVES * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
@@ -64,10 +64,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   constexpr int NCA = NC > 0 ? NC : 1;
   constexpr int RC = KW == 1 ? 1 : ((KW - 1) < 3 ? (KW - 1) : 3);  // remote sources polled together
   constexpr size_t INW = bwd_inbox_words(D, KW);
+  constexpr int E = O::E, ND_ = NDW<T, E>::value;
+  constexpr unsigned ES = sizeof(T);
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);
   T* const gbuf1 = gbuf0 + 16 * KDL;
+  int* const dead_flag = reinterpret_cast<int*>(gbuf1 + 16 * KDL);
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -76,20 +79,30 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const int n = grp % N, bt = grp / N;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
-  const int bg = bt * 16 + r16;
+  const int brow = O::row(r16), esub = O::sub(r16, q4);
+  const int bg = bt * 16 + brow;
   const bool bvalid = bg < B;
   const T* __restrict__ Rt = static_cast<const T*>(a.Rt);
-  const T* __restrict__ s0 = static_cast<const T*>(a.s0);
-  const T* __restrict__ states = static_cast<const T*>(a.states);
-  const T* __restrict__ cache = static_cast<const T*>(a.cache);
-  const T* __restrict__ dstates = static_cast<const T*>(a.dstates);
-  T* __restrict__ dWx = static_cast<T*>(a.dWx);
-  T* __restrict__ dgx = static_cast<T*>(a.dgx);
-  const size_t ND = (size_t)N * D;
+  const unsigned ND = (unsigned)N * D;
+
+  const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
+  const rsrc_t rS0 = make_rsrc(a.s0, (size_t)S * B * ND * ES);
+  const rsrc_t rDs = make_rsrc(a.dstates, (size_t)S * B * Tn * ND * ES);
+  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * a.groups_total * 16 * D * NC * ES);
+  const rsrc_t rDw = make_rsrc(a.dWx, (size_t)B * Tn * GW * ND * ES);
+  const rsrc_t rDx = make_rsrc(a.dgx, (size_t)B * Tn * ND * ES);
 
   int ub[UTW];
+  unsigned wx_v[UTW], st_v[UTW], s0_v[UTW], ca_v[UTW];
 #pragma unroll
-  for (int u = 0; u < UTW; ++u) ub[u] = (slice * UT_WG + w * UTW + u) * 16;
+  for (int u = 0; u < UTW; ++u) {
+    ub[u] = (slice * UT_WG + w * UTW + u) * 16;
+    const unsigned d0 = n * D + ub[u] + esub;
+    wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
+    st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
+    s0_v[u] = bvalid ? ((unsigned)bg * ND + d0) * ES : kInvalidOff;
+    ca_v[u] = bvalid ? ((unsigned)(ub[u] >> 4) * NC * 256 + brow * 16 + esub) * ES : kInvalidOff;
+  }
 
   // rtf[r][u][ks]: rows p of the tiles at this wave's position in workgroup (slice + r) % KW,
   // columns = the own gate rows, local index kk = g*DL + (d - slice*DL)
@@ -108,106 +121,90 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     }
   }
 
-  float ds[UTW][4][S];
-  float dbacc[UTW][4][GT];
+  // zero both LDS buffers once (rows 8..15 are never written in HALF mode) and the flag
+  for (int idx = tid; idx < (2 * 16 * KDL * (int)sizeof(T)) / 4 + 1; idx += NT) reinterpret_cast<unsigned*>(smem_raw)[idx] = 0u;
+
+  float ds[UTW][E][S];
+  float dbacc[UTW][E][GT];
 #pragma unroll
   for (int u = 0; u < UTW; ++u)
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
+    for (int e = 0; e < E; ++e) {
 #pragma unroll
-      for (int k = 0; k < S; ++k) ds[u][i][k] = 0.f;
+      for (int k = 0; k < S; ++k) ds[u][e][k] = 0.f;
 #pragma unroll
-      for (int g = 0; g < GT; ++g) dbacc[u][i][g] = 0.f;
+      for (int g = 0; g < GT; ++g) dbacc[u][e][g] = 0.f;
     }
 
-  u64* const inbox = a.ll + (size_t)grp * 2 * INW;
+  // per group: area 0, area 1 (by step parity) and a third that swallows padded lanes' stores
+  u64* const inbox = a.ll + (size_t)grp * 3 * INW;
 
-  struct Pre { Vec4 cache[UTW][NCA], sp[UTW][S], sn[UTW][S], dso[UTW][S]; };
+  struct Pre { Dw<ND_> cache[UTW][NCA], sp[UTW][S], sn[UTW][S], dso[UTW][S]; };
   Pre pa, pb;
   auto load_pre = [&](Pre& p, int t) __attribute__((always_inline)) {
+    const bool first = t == 0;
+    const rsrc_t rPrev = first ? rS0 : rSt;
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-      const int d0 = ub[u] + q4 * 4;
-      const size_t cb = ((((size_t)t * a.groups_total + grp) * (D / 16) + (ub[u] >> 4)) * NC) * 256 + r16 * 16 + q4 * 4;
 #pragma unroll
-      for (int c = 0; c < NC; ++c) p.cache[u][c] = *reinterpret_cast<const Vec4*>(cache + cb + (size_t)c * 256);
+      for (int c = 0; c < NC; ++c)
+        p.cache[u][c] = buf_load<ND_>(rCa, ca_v[u], ((((unsigned)t * a.groups_total + grp) * (D / 16)) * NC + c) * 256 * ES);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
-        if (bvalid) {
-          const size_t so = (((size_t)k * B + bg) * Tn + t) * ND + (size_t)n * D + d0;
-          p.sn[u][k] = *reinterpret_cast<const Vec4*>(states + so);
-          p.dso[u][k] = *reinterpret_cast<const Vec4*>(dstates + so);
-          p.sp[u][k] = t > 0 ? *reinterpret_cast<const Vec4*>(states + so - ND)
-                             : *reinterpret_cast<const Vec4*>(s0 + ((size_t)k * B + bg) * ND + (size_t)n * D + d0);
-        } else {
-          p.sn[u][k] = Vec4{}; p.dso[u][k] = Vec4{}; p.sp[u][k] = Vec4{};
-        }
+        const unsigned so = ((unsigned)k * B * Tn + t) * ND * ES;
+        p.sn[u][k] = buf_load<ND_>(rSt, st_v[u], so);
+        p.dso[u][k] = buf_load<ND_>(rDs, st_v[u], so);
+        p.sp[u][k] = buf_load<ND_>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * B * ND * ES : so - ND * ES);
       }
     }
   };
   load_pre(pa, Tn - 1);
+  __syncthreads();
 
   bool dead = false, fail = false;
   // one reverse step: consumes `pc` (operands of step t), prefetches those of step t-1 into `pn`
   auto step = [&](const int t, Pre& pc, Pre& pn) __attribute__((always_inline)) {
     T* const gb = (t & 1) ? gbuf1 : gbuf0;
+    load_pre(pn, max(t - 1, 0));
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-      const int d0 = ub[u] + q4 * 4;
-      float cv[NCA][4], spv[S][4], snv[S][4], dsov[S][4];
+      float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
 #pragma unroll
-      for (int c = 0; c < NC; ++c) unpack4(pc.cache[u][c], cv[c]);
+      for (int c = 0; c < NC; ++c) unpack<E>(pc.cache[u][c], cv[c], (T*)0);
 #pragma unroll
-      for (int k = 0; k < S; ++k) { unpack4(pc.sp[u][k], spv[k]); unpack4(pc.sn[u][k], snv[k]); unpack4(pc.dso[u][k], dsov[k]); }
-      float dgr[GR][4], dgw[GW][4];
+      for (int k = 0; k < S; ++k) {
+        unpack<E>(pc.sp[u][k], spv[k], (T*)0); unpack<E>(pc.sn[u][k], snv[k], (T*)0); unpack<E>(pc.dso[u][k], dsov[k], (T*)0);
+      }
+      float dgr[GR][E], dgw[GW][E];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int e = 0; e < E; ++e) {
         float cc[NCA], sp[S], sn[S], dso[S], gr[GR], gw[GW], gb_[GT];
 #pragma unroll
-        for (int c = 0; c < NC; ++c) cc[c] = cv[c][i];
+        for (int c = 0; c < NC; ++c) cc[c] = cv[c][e];
 #pragma unroll
-        for (int k = 0; k < S; ++k) { sp[k] = spv[k][i]; sn[k] = snv[k][i]; dso[k] = dsov[k][i]; }
-        CM::bwd(cc, sp, sn, dso, ds[u][i], gr, gw, gb_);
-        if (!bvalid) {  // padded batch rows contribute nothing
+        for (int k = 0; k < S; ++k) { sp[k] = spv[k][e]; sn[k] = snv[k][e]; dso[k] = dsov[k][e]; }
+        CM::bwd(cc, sp, sn, dso, ds[u][e], gr, gw, gb_);
+        // padded batch rows contribute nothing (selects, not branches)
 #pragma unroll
-          for (int g = 0; g < GR; ++g) gr[g] = 0.f;
+        for (int g = 0; g < GR; ++g) dgr[g][e] = bvalid ? gr[g] : 0.f;
 #pragma unroll
-          for (int g = 0; g < GW; ++g) gw[g] = 0.f;
+        for (int g = 0; g < GW; ++g) dgw[g][e] = bvalid ? gw[g] : 0.f;
 #pragma unroll
-          for (int g = 0; g < GT; ++g) gb_[g] = 0.f;
+        for (int g = 0; g < GT; ++g) dbacc[u][e][g] += bvalid ? gb_[g] : 0.f;
 #pragma unroll
-          for (int k = 0; k < S; ++k) ds[u][i][k] = 0.f;
-        }
-#pragma unroll
-        for (int g = 0; g < GR; ++g) dgr[g][i] = gr[g];
-#pragma unroll
-        for (int g = 0; g < GW; ++g) dgw[g][i] = gw[g];
-#pragma unroll
-        for (int g = 0; g < GT; ++g) dbacc[u][i][g] += gb_[g];
-      }
-      if (bvalid) {
-#pragma unroll
-        for (int g = 0; g < GW; ++g) {
-          Vec4 p; pack4(dgw[g], p);
-          *reinterpret_cast<Vec4*>(dWx + (((size_t)bg * Tn + t) * GW + g) * ND + (size_t)n * D + d0) = p;
-        }
-        if (F == FRNN_GRU) {
-          Vec4 p; pack4(dgr[0], p);
-          *reinterpret_cast<Vec4*>(dgx + ((size_t)bg * Tn + t) * ND + (size_t)n * D + d0) = p;
-        }
+        for (int k = 0; k < S; ++k) ds[u][e][k] = bvalid ? ds[u][e][k] : 0.f;
       }
 #pragma unroll
-      for (int g = 0; g < GR; ++g) lds_write4(gb, r16, g * DL + (d0 - slice * DL), dgr[g]);
+      for (int g = 0; g < GW; ++g)
+        buf_store<ND_>(pack<E>(dgw[g], (T*)0), rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
+      if (F == FRNN_GRU) buf_store<ND_>(pack<E>(dgr[0], (T*)0), rDx, st_v[u], (unsigned)t * ND * ES);
+#pragma unroll
+      for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
     }
     // the barrier also spreads a failed wait of the previous step to the whole workgroup
-    if (__syncthreads_or(fail)) { dead = true; return; }
-    if (t > 0) load_pre(pn, t - 1);
+    if (barrier_or(fail, dead_flag)) { dead = true; return; }
 
     f32x4 acc[KW][UTW];
-#pragma unroll
-    for (int r = 0; r < KW; ++r)
-#pragma unroll
-      for (int u = 0; u < UTW; ++u) acc[r][u] = f32x4{0.f, 0.f, 0.f, 0.f};
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -215,42 +212,37 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
       for (int r = 0; r < KW; ++r)
 #pragma unroll
-        for (int u = 0; u < UTW; ++u) acc[r][u] = X::mfma(rtf[r][u][ks], g, acc[r][u]);
+        for (int u = 0; u < UTW; ++u) acc[r][u] = X::mfma(rtf[r][u][ks], g, ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[r][u]);
     }
 #pragma unroll
-    for (int u = 0; u < UTW; ++u)
+    for (int u = 0; u < UTW; ++u) {
+      float own[E];
+      own_elems<HALF>(acc[0][u], own);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) ds[u][i][0] += acc[0][u][i];
+      for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
+    }
 
-    if constexpr (KW > 1) if (bvalid) {
-      u64* const slot = inbox + (size_t)(t & 1) * INW;
+    if constexpr (KW > 1) {
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
+      u64* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
 #pragma unroll
       for (int r = 1; r < KW; ++r) {
         const int x = (slice + r) % KW;
 #pragma unroll
         for (int u = 0; u < UTW; ++u) {
-          u64* dst = slot + ((((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 64 + lane) * 4;
+          float part[E];
+          own_elems<HALF>(acc[r][u], part);
+          u64* dst = sslot + ((((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 64 + lane) * 4;
 #pragma unroll
-          for (int i = 0; i < 4; ++i) ll_store(dst + i, ll_pack((float*)0, acc[r][u][i], t));
+          for (int e = 0; e < E; ++e) ll_store(dst + e, ll_pack((float*)0, part[e], t));
         }
       }
       // receive: KW-1 partial sums of the own tiles, RC sources at a time
-      const u64* const mine = slot + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + (size_t)lane * 4;
+      const u64* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + (size_t)lane * 4;
+      if (bvalid) {
 #pragma unroll
-      for (int r0 = 1; r0 < KW; r0 += RC) {
-        u64 v[RC][UTW][4];
-#pragma unroll
-        for (int rr = 0; rr < RC; ++rr)
-          if (r0 + rr < KW) {
-            const int src = (slice + r0 + rr) % KW;
-#pragma unroll
-            for (int u = 0; u < UTW; ++u)
-#pragma unroll
-              for (int i = 0; i < 4; ++i) v[rr][u][i] = ll_load(mine + ((size_t)u * KW + src) * 256 + i);
-          }
-        for (int spins = 0; !fail;) {
-          bool ok = true;
+        for (int r0 = 1; r0 < KW; r0 += RC) {
+          u64 v[RC][UTW][E];
 #pragma unroll
           for (int rr = 0; rr < RC; ++rr)
             if (r0 + rr < KW) {
@@ -258,22 +250,34 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
               for (int u = 0; u < UTW; ++u)
 #pragma unroll
-                for (int i = 0; i < 4; ++i)
-                  if (!ll_ok((float*)0, v[rr][u][i], t)) { ok = false; v[rr][u][i] = ll_load(mine + ((size_t)u * KW + src) * 256 + i); }
+                for (int e = 0; e < E; ++e) v[rr][u][e] = ll_load(mine + ((size_t)u * KW + src) * 256 + e);
             }
-          if (ok) break;
-          if (++spins > a.spin_limit) fail = true;
-          else if ((spins & 255) == 0 &&
-                   __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) fail = true;
-        }
+          for (int spins = 0; !fail;) {
+            bool ok = true;
 #pragma unroll
-        for (int rr = 0; rr < RC; ++rr)
-          if (r0 + rr < KW) {
+            for (int rr = 0; rr < RC; ++rr)
+              if (r0 + rr < KW) {
+                const int src = (slice + r0 + rr) % KW;
 #pragma unroll
-            for (int u = 0; u < UTW; ++u)
+                for (int u = 0; u < UTW; ++u)
 #pragma unroll
-              for (int i = 0; i < 4; ++i) ds[u][i][0] += __uint_as_float((unsigned)v[rr][u][i]);
+                  for (int e = 0; e < E; ++e)
+                    if (!ll_ok((float*)0, v[rr][u][e], t)) { ok = false; v[rr][u][e] = ll_load(mine + ((size_t)u * KW + src) * 256 + e); }
+              }
+            if (ok) break;
+            if (++spins > a.spin_limit) fail = true;
+            else if ((spins & 255) == 0 &&
+                     __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) fail = true;
           }
+#pragma unroll
+          for (int rr = 0; rr < RC; ++rr)
+            if (r0 + rr < KW) {
+#pragma unroll
+              for (int u = 0; u < UTW; ++u)
+#pragma unroll
+                for (int e = 0; e < E; ++e) ds[u][e][0] += __uint_as_float((unsigned)v[rr][u][e]);
+            }
+        }
       }
     }
   };
@@ -285,40 +289,37 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     step(t - 1, pb, pa);
   }
   if (!dead && t == 0) step(0, pa, pb);
-  if (!dead && __syncthreads_or(fail)) dead = true;
+  if (!dead && barrier_or(fail, dead_flag)) dead = true;
 
   if (dead) {
     if (tid == 0) __hip_atomic_store(a.status, (int)STATUS_WAIT_EXPIRED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
-      for (int i = 0; i < 4; ++i)
+      for (int e = 0; e < E; ++e)
 #pragma unroll
-        for (int k = 0; k < S; ++k) ds[u][i][k] = __uint_as_float(0x7fc00000u);
+        for (int k = 0; k < S; ++k) ds[u][e][k] = __uint_as_float(0x7fc00000u);
   }
 
   // ---- cotangent of the initial state, bias partial sums ----------------------------------
-  T* __restrict__ ds0 = static_cast<T*>(a.ds0);
+  const rsrc_t rD0 = make_rsrc(a.ds0, (size_t)S * B * ND * ES);
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
-    const int d0 = ub[u] + q4 * 4;
-    if (bvalid) {
 #pragma unroll
-      for (int k = 0; k < S; ++k) {
-        float v[4];
+    for (int k = 0; k < S; ++k) {
+      float v[E];
 #pragma unroll
-        for (int i = 0; i < 4; ++i) v[i] = ds[u][i][k];
-        Vec4 p; pack4(v, p);
-        *reinterpret_cast<Vec4*>(ds0 + ((size_t)k * B + bg) * ND + (size_t)n * D + d0) = p;
-      }
+      for (int e = 0; e < E; ++e) v[e] = ds[u][e][k];
+      buf_store<ND_>(pack<E>(v, (T*)0), rD0, s0_v[u], (unsigned)k * B * ND * ES);
     }
 #pragma unroll
     for (int g = 0; g < GT; ++g)
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
-        float v = dead ? __uint_as_float(0x7fc00000u) : dbacc[u][i][g];
-        v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4); v += __shfl_xor(v, 8);
-        if (r16 == 0) a.dbp[(((size_t)bt * GT + g) * N + n) * D + d0 + i] = v;
+      for (int e = 0; e < E; ++e) {
+        float v = dead ? __uint_as_float(0x7fc00000u) : dbacc[u][e][g];
+        v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4);
+        if (!HALF) v += __shfl_xor(v, 8);
+        if (brow == 0) a.dbp[(((size_t)bt * GT + g) * N + n) * D + ub[u] + esub + e] = v;
       }
   }
 }

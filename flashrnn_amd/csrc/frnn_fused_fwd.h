@@ -13,6 +13,10 @@
 //   -> gates, new states in fp32 registers; states / gate cache stored straight in the public
 //      / private layouts; the new h goes to the other LDS buffer (KW == 1) or to the tagged
 //      global exchange (KW > 1).
+// Nothing inside a step branches on the lane: padded batch rows are handled by out-of-range
+// buffer offsets, so the compiler can count outstanding memory operations exactly and the Wx
+// prefetch and the output stores never stall the recurrence.  The bias is the C operand of the
+// first MFMA of each gate.
 #pragma once
 #include "frnn_exchange.h"
 #include "frnn_pointwise.h"
@@ -36,21 +40,26 @@ template <> __device__ __forceinline__ float load_frag<float>(const float* row, 
   return row[ks * 4 + kq];
 }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW>
+template <int F, typename T, int D, int WAVES, int UTW, int KW, bool HALF>
 __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
   typedef typename X::Vec4 Vec4;
   typedef typename X::Frag Frag;
+  typedef Own<HALF> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
   constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
   constexpr int LLW = 16 * D / X::EPW;  // 64-bit words per exchange slot
   constexpr int NP = (LLW + NT - 1) / NT;
   constexpr int NCA = NC > 0 ? NC : 1;
+  constexpr int GX = GT - GR > 0 ? GT - GR : 1;
+  constexpr int E = O::E, ND_ = NDW<T, E>::value;
+  constexpr unsigned ES = sizeof(T);
 
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
+  __shared__ int dead_flag;
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -59,20 +68,30 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   const int n = grp % N, bt = grp / N;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
-  const int bg = bt * 16 + r16;  // batch row of this lane's output column
+  const int brow = O::row(r16), esub = O::sub(r16, q4);
+  const int bg = bt * 16 + brow;  // batch row this lane does the gate math for
   const bool bvalid = bg < B;
   const int rows_valid = min(16, B - bt * 16);
-  const T* __restrict__ Wx = static_cast<const T*>(a.Wx);
   const T* __restrict__ R = static_cast<const T*>(a.R);
   const T* __restrict__ bias_g = static_cast<const T*>(a.b);
   const T* __restrict__ s0 = static_cast<const T*>(a.s0);
-  T* __restrict__ states = static_cast<T*>(a.states);
-  T* __restrict__ cache = static_cast<T*>(a.cache);
-  const size_t ND = (size_t)N * D;
+  const unsigned ND = (unsigned)N * D;
+  if (tid == 0) dead_flag = 0;
+
+  const rsrc_t rWx = make_rsrc(a.Wx, (size_t)B * Tn * GW * ND * ES);
+  const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
+  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * a.groups_total * 16 * D * NC * ES);
 
   int ub[UTW];
+  unsigned wx_v[UTW], st_v[UTW], ca_v[UTW];  // per-lane byte offsets; out of range for padded rows
 #pragma unroll
-  for (int u = 0; u < UTW; ++u) ub[u] = (slice * UT_WG + w * UTW + u) * 16;
+  for (int u = 0; u < UTW; ++u) {
+    ub[u] = (slice * UT_WG + w * UTW + u) * 16;
+    const unsigned d0 = n * D + ub[u] + esub;
+    wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
+    st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
+    ca_v[u] = (bvalid && a.training) ? ((unsigned)(ub[u] >> 4) * NC * 256 + brow * 16 + esub) * ES : kInvalidOff;
+  }
 
   // ---- resident operands ----------------------------------------------------------------
   Frag rf[UTW][GR][KS];
@@ -84,75 +103,69 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) rf[u][g][ks] = load_frag<T>(row, ks, q4);
     }
-  float bias[UTW][4][GT];
-  float s[UTW][4][S];
+  f32x4 biasc[UTW][GR];   // bias of the recurrent gate slots, in MFMA C layout
+  float bx[UTW][E][GX];   // bias of the gate slots without recurrent input
+  float s[UTW][E][S];
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
-    const int d0 = ub[u] + q4 * 4;
 #pragma unroll
-    for (int g = 0; g < GT; ++g) {
+    for (int g = 0; g < GR; ++g) {
       float v[4];
-      unpack4(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + d0), v);
-#pragma unroll
-      for (int i = 0; i < 4; ++i) bias[u][i][g] = v[i];
+      unpack4(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
+      biasc[u][g] = f32x4{v[0], v[1], v[2], v[3]};
     }
 #pragma unroll
-    for (int k = 0; k < S; ++k) {
-      float v[4] = {0.f, 0.f, 0.f, 0.f};
-      if (bvalid) unpack4(*reinterpret_cast<const Vec4*>(s0 + ((size_t)k * B + bg) * ND + (size_t)n * D + d0), v);
+    for (int e = 0; e < E; ++e) {
 #pragma unroll
-      for (int i = 0; i < 4; ++i) s[u][i][k] = v[i];
+      for (int g = GR; g < GT; ++g) bx[u][e][g - GR] = (float)bias_g[(size_t)(g * N + n) * D + ub[u] + esub + e];
+#pragma unroll
+      for (int k = 0; k < S; ++k)
+        s[u][e][k] = bvalid ? (float)s0[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e] : 0.f;
     }
   }
 
-  // ---- h_0 of the whole head -> LDS buffer 0 (rows beyond B: zeros, and they stay zero or
-  //      private to their own MFMA column, so they never reach a valid row) ----------------
+  // ---- h_0 of the whole head -> LDS (rows beyond B are zero and stay zero or private to their
+  //      own MFMA column, so they never reach a valid row) --------------------------------------
   for (int idx = tid; idx < 16 * D / 4; idx += NT) {
     const int row = idx / (D / 4), k0 = (idx % (D / 4)) * 4;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     if (bt * 16 + row < B) unpack4(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * 16 + row) * ND + (size_t)n * D + k0), v);
-    lds_write4(hbuf[0], row, k0, v);
-    if (KW > 1) lds_write4(hbuf[1], row, k0, v);  // padded rows of buffer 1 must be finite too
+    lds_write<4>(hbuf[0], row, k0, v);
+    if (KW > 1 || HALF) {  // rows that are never rewritten must be finite in both buffers
+      if (bt * 16 + row >= B) lds_write<4>(hbuf[1], row, k0, v);
+    }
   }
 
   int qpoll[NP];
   if (KW > 1) ll_plan<T, NP, NT>(tid, rows_valid, D, qpoll);
-  u64* const llbase = a.ll + (size_t)grp * 2 * LLW;
+  // per group: slot 0, slot 1, and a third area that swallows the stores of padded lanes
+  u64* const llbase = a.ll + (size_t)grp * 3 * LLW;
 
-  Vec4 wxA[UTW][GW], wxB[UTW][GW];
-  auto load_wx = [&](Vec4 (&dst)[UTW][GW], int t) __attribute__((always_inline)) {
+  Dw<ND_> wxA[UTW][GW], wxB[UTW][GW];
+  auto load_wx = [&](Dw<ND_> (&dst)[UTW][GW], int t) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
-      for (int g = 0; g < GW; ++g) {
-        if (bvalid)
-          dst[u][g] = *reinterpret_cast<const Vec4*>(Wx + (((size_t)bg * Tn + t) * GW + g) * ND + (size_t)n * D + ub[u] + q4 * 4);
-        else
-          dst[u][g] = Vec4{};
-      }
+      for (int g = 0; g < GW; ++g) dst[u][g] = buf_load<ND_>(rWx, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
   };
   load_wx(wxA, 0);
   __syncthreads();
 
   bool dead = false;
   // one time step: consumes `wc` (Wx of step t), prefetches Wx of step t+1 into `wn`
-  auto step = [&](const int t, Vec4 (&wc)[UTW][GW], Vec4 (&wn)[UTW][GW]) __attribute__((always_inline)) {
+  auto step = [&](const int t, Dw<ND_> (&wc)[UTW][GW], Dw<ND_> (&wn)[UTW][GW]) __attribute__((always_inline)) {
     const int cur = t & 1;
     if (t > 0) {
       if (KW > 1) {
         const bool fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit);
-        if (__syncthreads_or(fail)) { dead = true; return; }
+        if (barrier_or(fail, &dead_flag)) { dead = true; return; }
       } else {
         __syncthreads();
       }
     }
-    if (t + 1 < Tn) load_wx(wn, t + 1);
+    load_wx(wn, min(t + 1, Tn - 1));
 
     f32x4 acc[UTW][GR];
-#pragma unroll
-    for (int u = 0; u < UTW; ++u)
-#pragma unroll
-      for (int g = 0; g < GR; ++g) acc[u][g] = f32x4{0.f, 0.f, 0.f, 0.f};
     const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane;
 #pragma unroll
     for (int ks = 0; ks < KS; ++ks) {
@@ -160,50 +173,41 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int u = 0; u < UTW; ++u)
 #pragma unroll
-        for (int g = 0; g < GR; ++g) acc[u][g] = X::mfma(rf[u][g][ks], h, acc[u][g]);
+        for (int g = 0; g < GR; ++g) acc[u][g] = X::mfma(rf[u][g][ks], h, ks == 0 ? biasc[u][g] : acc[u][g]);
     }
 
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-      const int d0 = ub[u] + q4 * 4;
-      float wxv[GW][4];
+      float ryv[GR][E], wxv[GW][E];
 #pragma unroll
-      for (int g = 0; g < GW; ++g) unpack4(wc[u][g], wxv[g]);
-      float cv[NCA][4];
-      float so[S][4];
+      for (int g = 0; g < GR; ++g) own_elems<HALF>(acc[u][g], ryv[g]);
 #pragma unroll
-      for (int i = 0; i < 4; ++i) {
+      for (int g = 0; g < GW; ++g) unpack<E>(wc[u][g], wxv[g], (T*)0);
+      float cv[NCA][E];
+      float so[S][E];
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
         float ry[GR], wx[GW], cc[NCA];
 #pragma unroll
-        for (int g = 0; g < GR; ++g) ry[g] = acc[u][g][i];
+        for (int g = 0; g < GR; ++g) ry[g] = ryv[g][e];
 #pragma unroll
-        for (int g = 0; g < GW; ++g) wx[g] = wxv[g][i];
-        CM::fwd(ry, wx, bias[u][i], s[u][i], cc);
+        for (int g = 0; g < GW; ++g) wx[g] = wxv[g][e];
+        CM::fwd(ry, wx, bx[u][e], s[u][e], cc);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) cv[c][i] = cc[c];
+        for (int c = 0; c < NC; ++c) cv[c][e] = cc[c];
 #pragma unroll
-        for (int k = 0; k < S; ++k) so[k][i] = s[u][i][k];
+        for (int k = 0; k < S; ++k) so[k][e] = s[u][e][k];
       }
-      if (bvalid) {
 #pragma unroll
-        for (int k = 0; k < S; ++k) {
-          Vec4 p; pack4(so[k], p);
-          *reinterpret_cast<Vec4*>(states + (((size_t)k * B + bg) * Tn + t) * ND + (size_t)n * D + d0) = p;
-        }
-      }
-      if (a.training && NC > 0) {
-        // private layout [t][group][unit tile][value][16 rows][16 units]: 512 B runs per wave
-        const size_t cb = ((((size_t)t * a.groups_total + grp) * (D / 16) + (ub[u] >> 4)) * NC) * 256 + r16 * 16 + q4 * 4;
+      for (int k = 0; k < S; ++k)
+        buf_store<ND_>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
+      // private cache layout [t][group][unit tile][value][16 rows][16 units]
 #pragma unroll
-        for (int c = 0; c < NC; ++c) {
-          Vec4 p; pack4(cv[c], p);
-          *reinterpret_cast<Vec4*>(cache + cb + (size_t)c * 256) = p;
-        }
-      }
-      if (t + 1 < Tn) {
-        if (KW == 1) lds_write4(hbuf[cur ^ 1], r16, d0, so[0]);
-        else if (bvalid) ll_write4((T*)0, llbase + (size_t)(t & 1) * LLW, r16, d0, so[0], t);
-      }
+      for (int c = 0; c < NC; ++c)
+        buf_store<ND_>(pack<E>(cv[c], (T*)0), rCa, ca_v[u],
+                       ((((unsigned)t * a.groups_total + grp) * (D / 16)) * NC + c) * 256 * ES);
+      if (KW == 1) lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
+      else ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
     }
   };
 
@@ -219,16 +223,12 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     // bounded wait ran out: report, and make the damage visible (NaN in every h of this
     // workgroup's units; the step that failed is not known exactly, so all steps are marked)
     if (tid == 0) __hip_atomic_store(a.status, (int)STATUS_WAIT_EXPIRED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-    if (bvalid) {
-      float nanv[4];
+    float nanv[E];
 #pragma unroll
-      for (int i = 0; i < 4; ++i) nanv[i] = __uint_as_float(0x7fc00000u);
-      Vec4 p; pack4(nanv, p);
-      for (int tt = 0; tt < Tn; ++tt)
+    for (int e = 0; e < E; ++e) nanv[e] = __uint_as_float(0x7fc00000u);
+    for (int tt = 0; tt < Tn; ++tt)
 #pragma unroll
-        for (int u = 0; u < UTW; ++u)
-          *reinterpret_cast<Vec4*>(states + ((size_t)bg * Tn + tt) * ND + (size_t)n * D + ub[u] + q4 * 4) = p;
-    }
+      for (int u = 0; u < UTW; ++u) buf_store<ND_>(pack<E>(nanv, (T*)0), rSt, st_v[u], (unsigned)tt * ND * ES);
   }
 }
 

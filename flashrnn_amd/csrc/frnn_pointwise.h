@@ -30,7 +30,9 @@ template <bool FAST> struct Math {
   }
 };
 
-// fwd:  ry[GR] recurrent pre-activations, wx[GW], bias[GT], s[S] in/out, cache[NC] out
+// fwd:  ry[GR] recurrent pre-activations WITH the bias of their gate slot already added (the
+//       fused kernels fold it into the MFMA accumulator), wx[GW], bx = biases of the gate slots
+//       that have no recurrent input (gru: the n gate), s[S] in/out, cache[NC] out
 // bwd:  cache[NC], sp[S] = s_{t-1}, sn[S] = s_t, dso[S] upstream cotangent of s_t,
 //       ds[S] in: running cotangent arriving from step t+1; out: cotangent for s_{t-1}
 //       WITHOUT the recurrent term R^T dgr (the caller adds it to ds[0]);
@@ -40,10 +42,10 @@ template <int F, bool FAST> struct CellMath;
 template <bool FAST> struct CellMath<FRNN_LSTM, FAST> {
   typedef Math<FAST> M;
   static __device__ __forceinline__ void fwd(const float* ry, const float* wx, const float* b, float* s, float* cache) {
-    const float i = M::sigmoid(wx[0] + ry[0] + b[0]);
-    const float f = M::sigmoid(wx[1] + ry[1] + b[1]);
-    const float z = M::tanh(wx[2] + ry[2] + b[2]);
-    const float o = M::sigmoid(wx[3] + ry[3] + b[3]);
+    const float i = M::sigmoid(wx[0] + ry[0]);
+    const float f = M::sigmoid(wx[1] + ry[1]);
+    const float z = M::tanh(wx[2] + ry[2]);
+    const float o = M::sigmoid(wx[3] + ry[3]);
     const float c = f * s[1] + i * z;
     s[1] = c;
     s[0] = o * M::tanh(c);
@@ -69,10 +71,10 @@ template <bool FAST> struct CellMath<FRNN_LSTM, FAST> {
 template <bool FAST> struct CellMath<FRNN_SLSTM, FAST> {
   typedef Math<FAST> M;
   static __device__ __forceinline__ void fwd(const float* ry, const float* wx, const float* b, float* s, float* cache) {
-    const float ir = wx[0] + ry[0] + b[0];
-    const float fr = wx[1] + ry[1] + b[1];
-    const float z = M::tanh(wx[2] + ry[2] + b[2]);
-    const float o = M::sigmoid(wx[3] + ry[3] + b[3]);
+    const float ir = wx[0] + ry[0];
+    const float fr = wx[1] + ry[1];
+    const float z = M::tanh(wx[2] + ry[2]);
+    const float o = M::sigmoid(wx[3] + ry[3]);
     const float lfm = M::logsigmoid(fr) + s[3];
     // first step of a fresh sequence: n == 0 (per element, as the native reference kernels,
     // flashrnn/flashrnn/fused/slstm_fused_pointwise.cuh:54-62)
@@ -107,10 +109,10 @@ template <bool FAST> struct CellMath<FRNN_GRU, FAST> {
   typedef Math<FAST> M;
   // R gates [g, r, z]; Wx gates [r, z, n]; bias gates [g, r, z, n]
   static __device__ __forceinline__ void fwd(const float* ry, const float* wx, const float* b, float* s, float* cache) {
-    const float g = ry[0] + b[0];
-    const float r = M::sigmoid(wx[0] + ry[1] + b[1]);
-    const float z = M::sigmoid(wx[1] + ry[2] + b[2]);
-    const float nr = wx[2] + b[3];
+    const float g = ry[0];
+    const float r = M::sigmoid(wx[0] + ry[1]);
+    const float z = M::sigmoid(wx[1] + ry[2]);
+    const float nr = wx[2] + b[0];
     s[0] = z * s[0] + (1.0f - z) * M::tanh(nr + r * g);
     cache[0] = g; cache[1] = r; cache[2] = z; cache[3] = nr;
   }
@@ -133,7 +135,7 @@ template <bool FAST> struct CellMath<FRNN_GRU, FAST> {
 template <bool FAST> struct CellMath<FRNN_ELMAN, FAST> {
   typedef Math<FAST> M;
   static __device__ __forceinline__ void fwd(const float* ry, const float* wx, const float* b, float* s, float*) {
-    s[0] = M::tanh(wx[0] + ry[0] + b[0]);
+    s[0] = M::tanh(wx[0] + ry[0]);
   }
   static __device__ __forceinline__ void bwd(const float*, const float*, const float* sn, const float* dso,
                                              float* ds, float* dgr, float* dgw, float* dgb) {

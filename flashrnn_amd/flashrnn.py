@@ -145,7 +145,8 @@ class _FlashRNNFunction(torch.autograd.Function):
                 ws.data_ptr(), ws.numel(), stream)
             if rc != 0:
                 _raise(rc, f"{cfg.backend} forward")
-        _last_workspace["forward"] = ws
+        if cfg.backend == "hip_fused":
+            _last_workspace["forward"] = ws
         ctx.cfg, ctx.training = cfg, training
         ctx.dims = (B, T, N, D)
         ctx.save_for_backward(R_k, b_k, s0_k, states, cache)
@@ -178,7 +179,8 @@ class _FlashRNNFunction(torch.autograd.Function):
                 ws.data_ptr(), ws.numel(), stream)
             if rc != 0:
                 _raise(rc, f"{cfg.backend} backward")
-        _last_workspace["backward"] = ws
+        if cfg.backend == "hip_fused":
+            _last_workspace["backward"] = ws
         # dR / db stay fp32: autograd casts them to the dtype of the leaf they belong to, so fp32
         # master weights receive unrounded gradients
         return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None

@@ -54,6 +54,17 @@ enum {
 const char* frnn_last_error(void);
 const char* frnn_version(void);
 
+/* Optional per-launch timing with HIP events on the caller's stream (off by default; for
+ * benchmarks: one thread, one stream).  No counterpart in the reference, which prints occupancy
+ * and register use at build time instead (cuda_init.py:144-147).  frnn_profile_enable(1) starts
+ * recording; each entry is one kernel launch (or the per-step launch loop of the alternating
+ * backend); frnn_profile_ms(i) waits for entry i and returns its duration in milliseconds. */
+void frnn_profile_enable(int on);
+void frnn_profile_reset(void);
+int frnn_profile_count(void);
+const char* frnn_profile_name(int i);
+float frnn_profile_ms(int i);
+
 /* (G_r, G_w, G_t, S) of a function and the number of values per element the gate cache
  * holds; 0 ok / FRNN_E_ARG.  Mirrors rnn_function_registry, flashrnn.py:49-71. */
 int frnn_function_dims(int function, int* G_r, int* G_w, int* G_t, int* S, int* cache_vals);
