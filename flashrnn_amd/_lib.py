@@ -41,7 +41,8 @@ EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 
 
 def library_path() -> str:
-    return os.path.join(_HERE, "libflashrnn_hip.so")
+    """The in-tree library; FLASHRNN_HIP_LIBRARY overrides it (e.g. an instrumented build)."""
+    return os.environ.get("FLASHRNN_HIP_LIBRARY") or os.path.join(_HERE, "libflashrnn_hip.so")
 
 
 def build_library(jobs: int = 8, force: bool = False) -> str:

@@ -155,6 +155,9 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   const size_t llw = (size_t)16 * D / (dtype == FRNN_BF16 ? 2 : 1);
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
   w.zero_bytes = bp.off;  // status + exchange slots must start at zero for every call
+#ifdef FRNN_TRACE
+  bp.take(1 << 20);
+#endif
   w.total = bp.off;
   return w;
 }
@@ -319,6 +322,11 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
   a.B = B; a.T = T; a.N = N; a.groups_total = groups;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  a.poll_delay = env_int("FRNN_POLL_DELAY", 0);
+  a.trace = nullptr;
+#ifdef FRNN_TRACE
+  a.trace = (long long*)((char*)workspace + w.zero_bytes);
+#endif
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
     prof_begin("fused_fwd_kernel", st);
@@ -375,6 +383,7 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
   a.ll = w.ll; a.status = w.status;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", 8);  // ~0.25 us: measured best on MI355X
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
     prof_begin("fused_bwd_kernel", st);

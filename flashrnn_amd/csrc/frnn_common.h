@@ -181,6 +181,9 @@ __device__ __forceinline__ void ll_store(u64* p, u64 v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 
+// largest divisor of n that is <= 8: k-steps whose LDS fragments are fetched together
+constexpr int chunk_of(int n) { for (int c = 8; c > 1; --c) if (n % c == 0) return c; return 1; }
+
 // status word values written by a kernel whose bounded wait ran out
 enum { STATUS_OK = 0, STATUS_WAIT_EXPIRED = 1 };
 

@@ -83,40 +83,74 @@ __device__ __forceinline__ void ll_plan(int tid, int rows_valid, int kdim, int* 
   }
 }
 
-// Poll until every planned word carries the tag of step t, then copy payloads to LDS.
-// Returns true if the bounded wait ran out (or another workgroup already reported that).
+// Poll NW tagged words (addresses base + off[i]; every lane polls NW words, lanes or entries
+// with nothing to wait for pass need[i] = false and may point anywhere valid) until all carry the
+// tag of step t.  PD probes of the whole set are kept in flight, so a word that becomes visible is
+// seen within 1/PD of a memory round trip; loads are unconditional and the exit test is a wave
+// vote, so the waits between probes are exact counts, not drains.  Returns true if the bounded
+// wait ran out (or another workgroup already reported that).
+template <typename TAG, int NW, int PD>
+__device__ __forceinline__ bool poll_words(const u64* base, const int* off, const bool* need, int t, u64* out,
+                                           int* status, int spin_limit, int first_delay) {
+  // the producers finish their step at about the same time as this wave: a probe sent at once
+  // reaches memory before their stores and costs a whole extra round trip
+  for (int i = 0; i < first_delay; ++i) __builtin_amdgcn_s_sleep(1);
+  u64 v[PD][NW];
+#pragma unroll
+  for (int p = 0; p < PD; ++p)
+#pragma unroll
+    for (int i = 0; i < NW; ++i) v[p][i] = ll_load(base + off[i]);
+  for (int spins = 0;; ++spins) {
+#pragma unroll
+    for (int p = 0; p < PD; ++p) {
+      bool ok = true;
+#pragma unroll
+      for (int i = 0; i < NW; ++i) ok = ok && (!need[i] || ll_ok((TAG*)0, v[p][i], t));
+      if (__all(ok)) {
+#pragma unroll
+        for (int i = 0; i < NW; ++i) out[i] = v[p][i];
+        return false;
+      }
+#pragma unroll
+      for (int i = 0; i < NW; ++i) v[p][i] = ll_load(base + off[i]);
+    }
+    if (spins > spin_limit) return true;
+    if ((spins & 63) == 63 &&
+        __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
+  }
+}
+constexpr int probe_depth(int) { return 1; }  // more probes in flight only add congestion (measured)
+
+// Forward gather: poll the planned words of slot, then copy their payloads to LDS.
 template <typename T, int NP>
 __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, T* lds_dst,
-                                          int* status, int spin_limit) {
-  u64 v[NP];
-#pragma unroll
-  for (int i = 0; i < NP; ++i)
-    if (q[i] >= 0) v[i] = ll_load(slot + q[i]);
+                                          int* status, int spin_limit, int first_delay) {
+  constexpr int CH = NP < 16 ? NP : 16;  // words polled together
+  static_assert(NP % CH == 0, "poll list must split into whole chunks");
   bool fail = false;
-  for (int spins = 0;;) {
-    bool ok = true;
 #pragma unroll
-    for (int i = 0; i < NP; ++i)
-      if (q[i] >= 0 && !ll_ok((T*)0, v[i], t)) { ok = false; v[i] = ll_load(slot + q[i]); }
-    if (ok) break;
-    if (++spins > spin_limit) { fail = true; break; }
-    if ((spins & 255) == 0 &&
-        __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) { fail = true; break; }
-  }
-  if (!fail) {
+  for (int c0 = 0; c0 < NP; c0 += CH) {
+    int off[CH]; bool need[CH]; u64 v[CH];
 #pragma unroll
-    for (int i = 0; i < NP; ++i)
-      if (q[i] >= 0) reinterpret_cast<unsigned*>(lds_dst)[q[i]] = ll_payload((T*)0, v[i]);
+    for (int i = 0; i < CH; ++i) { need[i] = q[c0 + i] >= 0; off[i] = need[i] ? q[c0 + i] : 0; }
+    fail = fail || poll_words<T, CH, probe_depth(CH)>(slot, off, need, t, v, status, spin_limit, c0 == 0 ? first_delay : 0);
+    if (!fail) {
+#pragma unroll
+      for (int i = 0; i < CH; ++i)
+        if (need[i]) reinterpret_cast<unsigned*>(lds_dst)[off[i]] = ll_payload((T*)0, v[i]);
+    }
   }
   return fail;
 }
 
 // Workgroup barrier that also tells every wave whether any lane passed `fail`; `flag` is one LDS
 // word that starts at 0 and is only ever set.  Costs one LDS read more than a plain barrier.
+// The result is read back through readfirstlane so that the compiler knows it is wave-uniform
+// and keeps the time-step counter (and every address derived from it) in scalar registers.
 __device__ __forceinline__ bool barrier_or(bool fail, volatile int* flag) {
   if (fail) *flag = 1;
   __syncthreads();
-  return *flag != 0;
+  return __builtin_amdgcn_readfirstlane(*flag) != 0;
 }
 
 }  // namespace frnn

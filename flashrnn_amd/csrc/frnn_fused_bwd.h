@@ -24,6 +24,10 @@
 #include "frnn_fused_fwd.h"
 #include "frnn_pointwise.h"
 
+#ifndef FRNN_BWD_PD
+#define FRNN_BWD_PD 1
+#endif
+
 namespace frnn {
 
 struct BwdArgs {
@@ -36,7 +40,7 @@ struct BwdArgs {
   u64* ll; int* status;
   int B, T, N;
   int grp0, groups, groups_total;
-  int spin_limit;
+  int spin_limit, poll_delay;
 };
 
 // 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][lane][4]
@@ -206,13 +210,26 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 
     f32x4 acc[KW][UTW];
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;
+    constexpr int KC = chunk_of(KS);
+    static_assert(KS % KC == 0, "k-steps must split into whole chunks");
+    Frag gq[2][KC];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const Frag g = gf[ks * 64];
+    for (int k = 0; k < KC; ++k) gq[0][k] = gf[k * 64];
 #pragma unroll
-      for (int r = 0; r < KW; ++r)
+    for (int kc = 0; kc < KS / KC; ++kc) {
+      if (kc + 1 < KS / KC) {
 #pragma unroll
-        for (int u = 0; u < UTW; ++u) acc[r][u] = X::mfma(rtf[r][u][ks], g, ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[r][u]);
+        for (int k = 0; k < KC; ++k) gq[(kc + 1) & 1][k] = gf[((kc + 1) * KC + k) * 64];
+      }
+#pragma unroll
+      for (int k = 0; k < KC; ++k) {
+        const int ks = kc * KC + k;
+#pragma unroll
+        for (int r = 0; r < KW; ++r)
+#pragma unroll
+          for (int u = 0; u < UTW; ++u)
+            acc[r][u] = X::mfma(rtf[r][u][ks], gq[kc & 1][k], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : acc[r][u]);
+      }
     }
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
@@ -239,45 +256,30 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
       // receive: KW-1 partial sums of the own tiles, RC sources at a time
       const u64* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + (size_t)lane * 4;
-      if (bvalid) {
 #pragma unroll
-        for (int r0 = 1; r0 < KW; r0 += RC) {
-          u64 v[RC][UTW][E];
+      for (int r0 = 1; r0 < KW; r0 += RC) {
+        constexpr int NWR = RC * UTW * E;
+        int off[NWR]; bool need[NWR]; u64 v[NWR];
 #pragma unroll
-          for (int rr = 0; rr < RC; ++rr)
-            if (r0 + rr < KW) {
-              const int src = (slice + r0 + rr) % KW;
+        for (int rr = 0; rr < RC; ++rr) {
+          const int src = (slice + (r0 + rr < KW ? r0 + rr : 1)) % KW;
 #pragma unroll
-              for (int u = 0; u < UTW; ++u)
+          for (int u = 0; u < UTW; ++u)
 #pragma unroll
-                for (int e = 0; e < E; ++e) v[rr][u][e] = ll_load(mine + ((size_t)u * KW + src) * 256 + e);
-            }
-          for (int spins = 0; !fail;) {
-            bool ok = true;
-#pragma unroll
-            for (int rr = 0; rr < RC; ++rr)
-              if (r0 + rr < KW) {
-                const int src = (slice + r0 + rr) % KW;
-#pragma unroll
-                for (int u = 0; u < UTW; ++u)
-#pragma unroll
-                  for (int e = 0; e < E; ++e)
-                    if (!ll_ok((float*)0, v[rr][u][e], t)) { ok = false; v[rr][u][e] = ll_load(mine + ((size_t)u * KW + src) * 256 + e); }
-              }
-            if (ok) break;
-            if (++spins > a.spin_limit) fail = true;
-            else if ((spins & 255) == 0 &&
-                     __hip_atomic_load(a.status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) fail = true;
-          }
-#pragma unroll
-          for (int rr = 0; rr < RC; ++rr)
-            if (r0 + rr < KW) {
-#pragma unroll
-              for (int u = 0; u < UTW; ++u)
-#pragma unroll
-                for (int e = 0; e < E; ++e) ds[u][e][0] += __uint_as_float((unsigned)v[rr][u][e]);
+            for (int e = 0; e < E; ++e) {
+              off[(rr * UTW + u) * E + e] = (u * KW + src) * 256 + e;
+              need[(rr * UTW + u) * E + e] = bvalid && (r0 + rr < KW);
             }
         }
+        if (!fail) fail = poll_words<float, NWR, FRNN_BWD_PD>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
+#pragma unroll
+        for (int rr = 0; rr < RC; ++rr)
+          if (r0 + rr < KW) {
+#pragma unroll
+            for (int u = 0; u < UTW; ++u)
+#pragma unroll
+              for (int e = 0; e < E; ++e) ds[u][e][0] += __uint_as_float((unsigned)v[(rr * UTW + u) * E + e]);
+          }
       }
     }
   };

@@ -29,8 +29,15 @@ struct FwdArgs {
   u64* ll; int* status;
   int B, T, N;
   int grp0, groups, groups_total;  // this launch handles groups [grp0, grp0 + groups)
-  int training, spin_limit;
+  int training, spin_limit, poll_delay;
+  long long* trace;  // phase cycle sums per workgroup; only written by -DFRNN_TRACE builds
 };
+
+#ifdef FRNN_TRACE
+#define FRNN_STAMP(var) __builtin_amdgcn_sched_barrier(0); const long long var = clock64(); __builtin_amdgcn_sched_barrier(0)
+#else
+#define FRNN_STAMP(var)
+#endif
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag(const T* row, int ks, int kq);
 template <> __device__ __forceinline__ bf16x8 load_frag<bf16_t>(const bf16_t* row, int ks, int kq) {
@@ -151,31 +158,59 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   load_wx(wxA, 0);
   __syncthreads();
 
+#ifdef FRNN_TRACE
+  long long tr[3] = {0, 0, 0};
+  const long long tr_begin = clock64();
+#endif
   bool dead = false;
   // one time step: consumes `wc` (Wx of step t), prefetches Wx of step t+1 into `wn`
   auto step = [&](const int t, Dw<ND_> (&wc)[UTW][GW], Dw<ND_> (&wn)[UTW][GW]) __attribute__((always_inline)) {
     const int cur = t & 1;
+    FRNN_STAMP(c0);
     if (t > 0) {
       if (KW > 1) {
-        const bool fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit);
+        const bool fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
         if (barrier_or(fail, &dead_flag)) { dead = true; return; }
       } else {
         __syncthreads();
       }
     }
+    FRNN_STAMP(c1);
     load_wx(wn, min(t + 1, Tn - 1));
 
+    // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once
     f32x4 acc[UTW][GR];
     const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane;
+    constexpr int KC = chunk_of(KS);
+    static_assert(KS % KC == 0, "k-steps must split into whole chunks");
+    Frag hq[2][KC];
 #pragma unroll
-    for (int ks = 0; ks < KS; ++ks) {
-      const Frag h = hf[ks * 64];
+    for (int k = 0; k < KC; ++k) hq[0][k] = hf[k * 64];
+#pragma unroll
+    for (int kc = 0; kc < KS / KC; ++kc) {
+      if (kc + 1 < KS / KC) {
+#pragma unroll
+        for (int k = 0; k < KC; ++k) hq[(kc + 1) & 1][k] = hf[((kc + 1) * KC + k) * 64];
+      }
+#pragma unroll
+      for (int k = 0; k < KC; ++k) {
+        const int ks = kc * KC + k;
+#pragma unroll
+        for (int u = 0; u < UTW; ++u)
+#pragma unroll
+          for (int g = 0; g < GR; ++g) acc[u][g] = X::mfma(rf[u][g][ks], hq[kc & 1][k], ks == 0 ? biasc[u][g] : acc[u][g]);
+      }
+    }
+
+#ifdef FRNN_TRACE
+    { float sink = 0.f;
 #pragma unroll
       for (int u = 0; u < UTW; ++u)
 #pragma unroll
-        for (int g = 0; g < GR; ++g) acc[u][g] = X::mfma(rf[u][g][ks], h, ks == 0 ? biasc[u][g] : acc[u][g]);
-    }
-
+        for (int g = 0; g < GR; ++g) sink += acc[u][g][0];
+      asm volatile("" ::"v"(sink)); }
+#endif
+    FRNN_STAMP(c2);
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float ryv[GR][E], wxv[GW][E];
@@ -198,6 +233,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
         for (int k = 0; k < S; ++k) so[k][e] = s[u][e][k];
       }
+      // the new h first: it is what the next step (of every workgroup of the head) waits for
+      if (KW == 1) lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
+      else ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
@@ -206,9 +244,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       for (int c = 0; c < NC; ++c)
         buf_store<ND_>(pack<E>(cv[c], (T*)0), rCa, ca_v[u],
                        ((((unsigned)t * a.groups_total + grp) * (D / 16)) * NC + c) * 256 * ES);
-      if (KW == 1) lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
-      else ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
     }
+#ifdef FRNN_TRACE
+    FRNN_STAMP(c3);
+    tr[0] += c1 - c0; tr[1] += c2 - c1; tr[2] += c3 - c2;
+#endif
   };
 
   int t = 0;
@@ -219,6 +259,12 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   }
   if (!dead && t < Tn) step(t, wxA, wxB);
 
+#ifdef FRNN_TRACE
+  if (lane == 0 && a.trace) {
+    long long* o = a.trace + ((size_t)blockIdx.x * WAVES + w) * 4;
+    o[0] = tr[0]; o[1] = tr[1]; o[2] = tr[2]; o[3] = clock64() - tr_begin;
+  }
+#endif
   if (dead) {
     // bounded wait ran out: report, and make the damage visible (NaN in every h of this
     // workgroup's units; the step that failed is not known exactly, so all steps are marked)
