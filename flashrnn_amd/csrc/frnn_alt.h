@@ -11,7 +11,8 @@ struct AltProblem { int function, dtype, B, T, N, D, training; };
 struct AltFwdBuffers {
   const void* Wx; const void* R; const void* b; const void* s0;
   void* states; void* cache;
-  float* ry;  // [B][N][G_r*D]
+  float* ry;   // [B][N][G_r*D]
+  float* sfp;  // [S][B][N][D]
 };
 
 struct AltBwdBuffers {

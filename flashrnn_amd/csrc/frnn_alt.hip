@@ -73,6 +73,9 @@ __device__ __forceinline__ void st_(float* p, float v) { *p = v; }
 struct AltPwArgs {
   const void* Wx; const void* b; const void* s0; void* states; void* cache;
   const float* ry;  // [B][N][G_r*D]
+  float* sfp;       // [S][B][N][D] fp32 copy of the running state: the states tensor is the
+                    // storage-type output, the recurrence itself is carried unrounded (only the h
+                    // that feeds the GEMM is read back in the storage type), as in the fused path
   int B, T, N, D, t, training;
 };
 
@@ -99,13 +102,16 @@ __global__ void __launch_bounds__(256) alt_pw_fwd_kernel(const AltPwArgs a) {
   for (int g = 0; g < GR; ++g) ry[g] += ld(bias + (size_t)(g * N + n) * D + d);
 #pragma unroll
   for (int g = GR; g < GT; ++g) bb[g - GR] = ld(bias + (size_t)(g * N + n) * D + d);
+  const size_t BND = (size_t)B * ND;
 #pragma unroll
   for (int k = 0; k < S; ++k)
-    s[k] = t > 0 ? ld(states + (((size_t)k * B + b) * Tn + t - 1) * ND + (size_t)n * D + d)
-                 : ld(s0 + ((size_t)k * B + b) * ND + (size_t)n * D + d);
+    s[k] = t > 0 ? a.sfp[(size_t)k * BND + idx] : ld(s0 + ((size_t)k * B + b) * ND + (size_t)n * D + d);
   CM::fwd(ry, wx, bb, s, cc);
 #pragma unroll
-  for (int k = 0; k < S; ++k) st_(states + (((size_t)k * B + b) * Tn + t) * ND + (size_t)n * D + d, s[k]);
+  for (int k = 0; k < S; ++k) {
+    st_(states + (((size_t)k * B + b) * Tn + t) * ND + (size_t)n * D + d, s[k]);
+    a.sfp[(size_t)k * BND + idx] = s[k];
+  }
   if (a.training && NC > 0) {
     T* cache = static_cast<T*>(a.cache) + (((size_t)t * B + b) * N + n) * NC * D + d;
 #pragma unroll
@@ -205,7 +211,7 @@ static int alt_forward_t(const AltProblem& p, const AltFwdBuffers& bf, hipStream
     g.out = bf.ry; g.B = p.B; g.N = p.N; g.D = p.D; g.M = GR * p.D; g.K = p.D;
     int e = launch_alt_gemm(ST<T>::ID, g, st);
     if (e) return e;
-    AltPwArgs a{bf.Wx, bf.b, bf.s0, bf.states, bf.cache, bf.ry, p.B, p.T, p.N, p.D, t, p.training};
+    AltPwArgs a{bf.Wx, bf.b, bf.s0, bf.states, bf.cache, bf.ry, bf.sfp, p.B, p.T, p.N, p.D, t, p.training};
     hipLaunchKernelGGL((alt_pw_fwd_kernel<F, T>), dim3(pw_blocks), dim3(256), 0, st, a);
     e = (int)hipGetLastError();
     if (e) return e;

@@ -413,7 +413,7 @@ size_t frnn_alt_cache_bytes(int function, int dtype, int B, int T, int N, int D)
 }
 
 namespace {
-struct AltWs { float* ry; void* Rt; void* dgx; void* dg; float* dsr; float* dh; float* dbp; int bsplits; float* part; int splits; size_t total; };
+struct AltWs { float* ry; float* sfp; void* Rt; void* dgx; void* dg; float* dsr; float* dh; float* dbp; int bsplits; float* part; int splits; size_t total; };
 AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, int backward) {
   const CellDims c = cell_dims(function);
   const size_t es = dtype_size(dtype), ND = (size_t)N * D, BND = (size_t)B * ND;
@@ -422,6 +422,7 @@ AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, i
   memset(&w, 0, sizeof(w));
   if (!backward) {
     w.ry = (float*)bp.take(BND * c.GR * 4);
+    w.sfp = (float*)bp.take(BND * c.S * 4);
   } else {
     w.Rt = bp.take(ND * c.GR * D * es);
     w.dgx = bp.take(function == FRNN_GRU ? (size_t)T * BND * es : 0);
@@ -457,7 +458,7 @@ int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N,
   const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 0);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0};
-  AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.ry};
+  AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.ry, w.sfp};
   prof_begin("alt_forward_steps", (hipStream_t)stream);
   e = alt_forward(p, bf, (hipStream_t)stream);
   prof_end((hipStream_t)stream);

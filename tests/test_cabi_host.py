@@ -1,0 +1,155 @@
+"""Host-side checks that need no GPU: the C-ABI library loads, exports every symbol the header
+declares, and rejects bad arguments with the documented codes before any launch."""
+import ctypes
+import os
+import re
+
+import pytest
+import torch
+
+from flashrnn_amd import FlashRNNConfig, flashrnn, load_library
+from flashrnn_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+HEADER = os.path.join(ROOT, "include", "flashrnn_hip.h")
+FAKE = ctypes.c_void_p(0x1000)  # non-null, 16-byte aligned; never dereferenced: every call below fails earlier
+
+
+@pytest.fixture(scope="module")
+def lib():
+    return load_library()
+
+
+def _declared_symbols():
+    text = open(HEADER).read()
+    text = re.sub(r"/\*.*?\*/", "", text, flags=re.S)
+    return sorted(set(re.findall(r"\b(frnn_\w+)\s*\(", text)))
+
+
+def test_library_exports_every_declared_symbol(lib):
+    names = _declared_symbols()
+    assert len(names) >= 14
+    for n in names:
+        assert hasattr(lib, n), n
+    assert set(names) == set(_lib.EXPORTED_SYMBOLS)
+    assert b"gfx950" in lib.frnn_version()
+
+
+def test_function_dims_mirror_the_registry(lib):
+    from flashrnn_amd import rnn_function_registry
+
+    for name, fid in _lib.FUNCTION_IDS.items():
+        vals = [ctypes.c_int() for _ in range(5)]
+        assert lib.frnn_function_dims(fid, *[ctypes.byref(v) for v in vals]) == 0
+        gr, gw, gi, gt, s = rnn_function_registry[name]["gates_states"]
+        assert [v.value for v in vals[:4]] == [gr, gw, gt, s]
+    assert lib.frnn_function_dims(9, None, None, None, None, None) == _lib.E_ARG
+
+
+def test_supported_table(lib):
+    L, S, G, E = (_lib.FUNCTION_IDS[k] for k in ("lstm", "slstm", "gru", "elman"))
+    for f in (L, S, G, E):
+        for D in (32, 64, 128, 192, 256, 512):
+            assert lib.frnn_fused_supported(f, 0, 8, 3, D) == 0, (f, D)
+    assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0
+    assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == _lib.E_UNSUPPORTED  # too large to keep on chip
+    assert lib.frnn_fused_supported(L, 1, 8, 1, 512) == _lib.E_UNSUPPORTED   # fp32 R is twice the size
+    assert lib.frnn_fused_supported(L, 0, 8, 1, 48) == _lib.E_UNSUPPORTED
+    assert b"head dim" in lib.frnn_last_error()
+    assert lib.frnn_alt_supported(L, 0, 8, 1, 1024) == 0
+    assert lib.frnn_alt_supported(L, 0, 8, 1, 48) == _lib.E_UNSUPPORTED
+    assert lib.frnn_fused_supported(7, 0, 8, 1, 64) == _lib.E_ARG
+    assert lib.frnn_fused_supported(L, 5, 8, 1, 64) == _lib.E_ARG
+    assert lib.frnn_fused_supported(L, 0, 0, 1, 64) == _lib.E_ARG
+
+
+def test_plan_and_sizes(lib):
+    L = _lib.FUNCTION_IDS["lstm"]
+    out = [ctypes.c_int() for _ in range(4)]
+    assert lib.frnn_fused_plan(L, 0, 8, 3, 256, 0, *[ctypes.byref(o) for o in out]) == 0
+    waves, utw, kw, active = (o.value for o in out)
+    assert 16 * waves * utw * kw == 256 and active == 3 * kw
+    # gate cache: T * N * padded batch * D * values * bytes
+    assert lib.frnn_fused_cache_bytes(L, 0, 8, 1024, 3, 256) == 1024 * 3 * 16 * 256 * 4 * 2
+    assert lib.frnn_alt_cache_bytes(L, 0, 8, 1024, 3, 256) == 1024 * 3 * 8 * 256 * 4 * 2
+    assert lib.frnn_fused_cache_bytes(_lib.FUNCTION_IDS["elman"], 0, 8, 16, 3, 256) == 0
+    assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 256, 0) >= 256
+    assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 256, 1) > lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 256, 0)
+    assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 1024, 0) == 0  # unsupported
+
+
+def _fwd(lib, entry, function=0, dtype=0, B=8, T=4, N=1, D=64, Wx=FAKE, R=FAKE, b=FAKE, s0=FAKE, states=FAKE,
+         cache=FAKE, ws=FAKE, ws_bytes=0, training=1):
+    return getattr(lib, entry)(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, ws, ws_bytes, None)
+
+
+@pytest.mark.parametrize("entry", ["frnn_fused_forward", "frnn_alt_forward"])
+def test_forward_rejects_bad_arguments_before_launch(lib, entry):
+    assert _fwd(lib, entry, function=4) == _lib.E_ARG
+    assert _fwd(lib, entry, dtype=3) == _lib.E_ARG
+    assert _fwd(lib, entry, T=0) == _lib.E_ARG
+    assert _fwd(lib, entry, D=40) == _lib.E_UNSUPPORTED
+    assert _fwd(lib, entry, Wx=None) == _lib.E_NULL
+    assert b"Wx" in lib.frnn_last_error()
+    assert _fwd(lib, entry, cache=None) == _lib.E_NULL          # training needs the cache
+    assert _fwd(lib, entry, R=ctypes.c_void_p(0x1004)) == _lib.E_ALIGN
+    assert _fwd(lib, entry, ws_bytes=16) == _lib.E_WORKSPACE    # smaller than *_workspace_bytes
+    assert b"workspace" in lib.frnn_last_error()
+
+
+@pytest.mark.parametrize("entry", ["frnn_fused_backward", "frnn_alt_backward"])
+def test_backward_rejects_bad_arguments_before_launch(lib, entry):
+    fn = getattr(lib, entry)
+
+    def call(function=0, dtype=0, B=8, T=4, N=1, D=64, ptrs=None, ws_bytes=0):
+        p = [FAKE] * 11 if ptrs is None else ptrs
+        return fn(function, dtype, B, T, N, D, *p, ws_bytes, None)
+
+    assert call(function=-1) == _lib.E_ARG
+    assert call(D=24) == _lib.E_UNSUPPORTED
+    for i in (0, 2, 3, 5, 6, 7, 8, 9, 10):  # R, s0, states, dstates, dWx, ds0, dR, db, workspace
+        p = [FAKE] * 11
+        p[i] = None
+        assert call(ptrs=p) == _lib.E_NULL, i
+    p = [FAKE] * 11
+    p[8] = ctypes.c_void_p(0x1008)
+    assert call(ptrs=p) == _lib.E_ALIGN
+    assert call(ws_bytes=64) == _lib.E_WORKSPACE
+
+
+def test_fused_refuses_tensors_of_2_gib(lib):
+    # 32-bit byte offsets inside the fused kernels: B*T*N*D*G_w*2 bytes must stay below 2 GiB
+    assert _fwd(lib, "frnn_fused_forward", B=64, T=16384, N=4, D=256) == _lib.E_ARG
+    assert b"2 GiB" in lib.frnn_last_error()
+
+
+def test_python_api_argument_errors():
+    with pytest.raises(ValueError):
+        FlashRNNConfig(backend="vanilla")  # the torch loop is the test oracle, not a backend
+    with pytest.raises(ValueError):
+        FlashRNNConfig(function="rnn")
+    with pytest.raises(ValueError):
+        FlashRNNConfig(dtype="float16")
+    with pytest.raises(NotImplementedError):
+        FlashRNNConfig(gradient_recurrent_cut=True)
+    cfg = FlashRNNConfig(function="gru", head_dim=64, num_heads=3)
+    assert (cfg.num_gates_r, cfg.num_gates_w, cfg.num_gates_t, cfg.num_states, cfg.hidden_dim) == (3, 3, 4, 1, 192)
+    Wx = torch.zeros(2, 3, 4, 1, 32)
+    R = torch.zeros(4, 1, 32, 32)
+    b = torch.zeros(4, 1, 32)
+    with pytest.raises(ValueError):
+        flashrnn(Wx, R[:3], b, function="lstm")
+    with pytest.raises(ValueError):
+        flashrnn(Wx, R, b, states=torch.zeros(2, 2, 1, 1, 16), function="lstm")
+    with pytest.raises(ValueError):
+        flashrnn(Wx[:, :, :3], R, b, function="lstm")
+    # no CPU path: a CPU tensor is refused, loudly
+    with pytest.raises(RuntimeError, match="GPU only"):
+        flashrnn(Wx, R, b, function="lstm")
+
+
+def test_missing_library_is_an_error(monkeypatch, tmp_path):
+    monkeypatch.setenv("FLASHRNN_HIP_LIBRARY", str(tmp_path / "nope.so"))
+    monkeypatch.setattr(_lib, "_LIB", None)
+    with pytest.raises(RuntimeError, match="missing"):
+        _lib.load_library()

@@ -1,0 +1,107 @@
+"""Parity of the HIP path (through the C ABI) with the CPU oracle on the same seeded inputs."""
+import pytest
+import torch
+
+from parity import check_case
+
+pytestmark = pytest.mark.gpu
+
+FUSED_SMALL = [
+    # function, B, T, N, D, dtype
+    ("lstm", 4, 8, 1, 64, "float32"),
+    ("lstm", 3, 5, 2, 32, "bfloat16"),
+    ("lstm", 1, 1, 1, 32, "bfloat16"),       # single step, single row
+    ("lstm", 9, 3, 2, 64, "bfloat16"),       # ragged batch: one row over the half tile
+    ("lstm", 20, 6, 2, 128, "bfloat16"),     # two batch tiles, second ragged
+    ("lstm", 8, 16, 3, 256, "bfloat16"),     # 4 workgroups per head, half-tile ownership
+    ("lstm", 16, 9, 1, 256, "bfloat16"),     # 4 workgroups per head, full tile
+    ("lstm", 33, 4, 1, 256, "bfloat16"),     # 3 batch tiles x 4 workgroups
+    ("lstm", 16, 5, 1, 512, "bfloat16"),     # 8 workgroups per head
+    ("lstm", 4, 6, 1, 256, "float32"),       # fp32, 4 workgroups per head
+    ("lstm", 5, 7, 2, 128, "float32"),
+    ("gru", 5, 9, 2, 64, "bfloat16"),
+    ("gru", 16, 8, 4, 128, "bfloat16"),
+    ("gru", 7, 5, 1, 256, "bfloat16"),
+    ("gru", 3, 6, 2, 32, "float32"),
+    ("gru", 16, 4, 1, 192, "bfloat16"),
+    ("elman", 16, 7, 2, 128, "bfloat16"),
+    ("elman", 32, 6, 1, 512, "bfloat16"),
+    ("elman", 16, 4, 1, 1024, "bfloat16"),   # 16 workgroups per head
+    ("elman", 6, 9, 3, 64, "float32"),
+    ("slstm", 8, 6, 2, 64, "bfloat16"),
+    ("slstm", 16, 12, 2, 192, "bfloat16"),   # D not a power of two, 3 workgroups per head
+    ("slstm", 5, 8, 1, 192, "float32"),
+    ("slstm", 12, 5, 2, 256, "bfloat16"),
+]
+
+
+@pytest.mark.parametrize("function,B,T,N,D,dtype", FUSED_SMALL)
+@pytest.mark.parametrize("init", ["zeros", "randn"])
+def test_fused_matches_oracle(gpu, function, B, T, N, D, dtype, init):
+    print(f"case fused {function} B{B} T{T} N{N} D{D} {dtype} init={init}", flush=True)
+    check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=7, init=init)
+
+
+ALT_SMALL = [
+    ("lstm", 4, 8, 1, 64, "float32"),
+    ("lstm", 3, 5, 2, 32, "bfloat16"),
+    ("lstm", 20, 4, 2, 128, "bfloat16"),
+    ("gru", 5, 9, 2, 64, "bfloat16"),
+    ("gru", 17, 3, 1, 96, "float32"),
+    ("slstm", 8, 6, 2, 64, "bfloat16"),
+    ("slstm", 3, 4, 1, 192, "float32"),
+    ("elman", 32, 8, 1, 1024, "bfloat16"),
+    ("elman", 2, 5, 2, 32, "float32"),
+]
+
+
+@pytest.mark.parametrize("function,B,T,N,D,dtype", ALT_SMALL)
+def test_alternating_matches_oracle(gpu, function, B, T, N, D, dtype):
+    print(f"case alt {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
+    check_case(gpu, function, B, T, N, D, dtype, "hip", seed=11, init="randn")
+
+
+def test_forward_only_no_grad(gpu):
+    """Inference call: no cache is written, backward is refused."""
+    print("case forward only", flush=True)
+    check_case(gpu, "lstm", 6, 9, 2, 64, "bfloat16", "hip_fused", backward=False)
+    check_case(gpu, "gru", 6, 9, 2, 64, "bfloat16", "hip", backward=False)
+
+
+# ---- the benchmark configurations --------------------------------------------------------------
+def test_config1_lstm_fp32_forward(gpu):
+    print("case C1", flush=True)
+    check_case(gpu, "lstm", 4, 256, 1, 64, "float32", "hip_fused", seed=1001, init="zeros", backward=False)
+    check_case(gpu, "lstm", 4, 256, 1, 64, "float32", "hip", seed=1001, init="zeros", backward=False)
+
+
+def test_config2_lstm_bf16_full_size(gpu):
+    print("case C2 full", flush=True)
+    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", "hip_fused", seed=1002, init="randn")
+
+
+def test_config2_alternating_full_size(gpu):
+    print("case C2 alt full", flush=True)
+    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", "hip", seed=1002, init="randn")
+
+
+def test_config3_gru_bf16_quarter_length(gpu):
+    print("case C3 T=512", flush=True)
+    check_case(gpu, "gru", 16, 512, 4, 128, "bfloat16", "hip_fused", seed=1003, init="zeros")
+
+
+def test_config4_slstm_bf16_eighth_length(gpu):
+    print("case C4 T=512", flush=True)
+    check_case(gpu, "slstm", 16, 512, 4, 192, "bfloat16", "hip_fused", seed=1004, init="zeros",
+               forget_bias_linspace=True)
+
+
+def test_config5_elman_alternating_quarter_length(gpu):
+    print("case C5 T=256", flush=True)
+    check_case(gpu, "elman", 32, 256, 1, 1024, "bfloat16", "hip", seed=1005, init="zeros")
+
+
+@pytest.mark.parametrize("N,D", [(24, 32), (12, 64), (6, 128), (3, 256), (1, 512)])
+def test_head_dim_sweep_points(gpu, N, D):
+    print(f"case sweep N{N} D{D}", flush=True)
+    check_case(gpu, "lstm", 16, 64, N, D, "bfloat16", "hip_fused", seed=1006, init="zeros")
