@@ -43,7 +43,7 @@ struct BwdArgs {
   int spin_limit, poll_delay;
 };
 
-// 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][lane][4]
+// 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][element 4][lane 64]
 constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) * 256; }
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_at(const T* p);
@@ -249,13 +249,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         for (int u = 0; u < UTW; ++u) {
           float part[E];
           own_elems<HALF>(acc[r][u], part);
-          u64* dst = sslot + ((((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 64 + lane) * 4;
+          u64* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
 #pragma unroll
-          for (int e = 0; e < E; ++e) ll_store(dst + e, ll_pack((float*)0, part[e], t));
+          for (int e = 0; e < E; ++e) ll_store(dst + e * 64, ll_pack((float*)0, part[e], t));
         }
       }
       // receive: KW-1 partial sums of the own tiles, RC sources at a time
-      const u64* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + (size_t)lane * 4;
+      const u64* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
 #pragma unroll
       for (int r0 = 1; r0 < KW; r0 += RC) {
         constexpr int NWR = RC * UTW * E;
@@ -267,7 +267,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
           for (int u = 0; u < UTW; ++u)
 #pragma unroll
             for (int e = 0; e < E; ++e) {
-              off[(rr * UTW + u) * E + e] = (u * KW + src) * 256 + e;
+              off[(rr * UTW + u) * E + e] = (u * KW + src) * 256 + e * 64;
               need[(rr * UTW + u) * E + e] = bvalid && (r0 + rr < KW);
             }
         }
