@@ -28,6 +28,13 @@ WORKLOADS = {
 }
 GATES_R = {"lstm": 4, "slstm": 4, "gru": 3, "elman": 1}
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, published
+# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, KiB -> bytes, copy-kernel factor 1.00) measured with
+# two `rocprofv3 --pmc` runs of this script; summary and commands in
+# profiles/fused_kernels_lstm_bf16_B8_T1024_N3_D256_hbm_traffic.txt.  Workloads not profiled: null.
+TRAFFIC_BYTES = {
+    ("C2", "fused_fwd_kernel"): (37711.0 + 98304.0) * 1024,
+    ("C2", "fused_bwd_kernel"): (121552.7 + 196644.0) * 1024,
+}
 
 
 def describe(w):
@@ -90,7 +97,7 @@ def run_gpu(w, backend, steps, warmup, device):
     return (t1 - t0) * 1e3 / steps, kern
 
 
-def run_cpu_baseline(w, budget_s=12.0):
+def run_cpu_baseline(w, budget_s=20.0):
     """The CPU oracle (a port of the reference's vanilla backend) on the host cores, fp32."""
     import torch
     from oracle import flashrnn_oracle, make_inputs
@@ -159,7 +166,7 @@ def main():
     peak = PEAK_TFLOPS[w["dtype"]]
     achieved = algo[dom] / cand[dom][1] / (dom_ms * 1e-3) / 1e12
     roofline = dict(kernel=dom, bound="mfma", achieved=achieved, peak=peak, unit="TFLOP/s", frac=achieved / peak,
-                    traffic=None, avg_launch_ms=dom_ms, launches_per_step=cand[dom][1],
+                    traffic=TRAFFIC_BYTES.get((args.workload, dom)), avg_launch_ms=dom_ms, launches_per_step=cand[dom][1],
                     us_per_time_step=dom_ms * 1e3 / w["T"])
     try:
         from flashrnn_amd import fused_plan
