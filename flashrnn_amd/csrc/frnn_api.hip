@@ -116,6 +116,16 @@ static int device_cus() {
   return cached[dev];
 }
 
+// Batch rows per group.  8-row tiles halve the gate math per lane (the larger cost of a step) at
+// the price of twice the workgroups and copies of R, so they are used while every workgroup of the
+// call still gets a compute unit of its own.
+static int tile_rows_for(int B, int N, int kw) {
+  const int forced = env_int("FRNN_TILE_ROWS", 0);
+  if (forced == 8 || forced == 16) return B <= 8 ? 8 : forced;
+  if (B <= 8) return 8;
+  return (long)N * ((B + 7) / 8) * kw <= device_cus() ? 8 : 16;
+}
+
 struct Bump {
   unsigned char* base; size_t off;
   void* take(size_t bytes) { void* p = base ? base + off : nullptr; off += (bytes + 255) & ~(size_t)255; return p; }
@@ -133,7 +143,7 @@ static int check_fused_sizes(int function, int dtype, int B, int T, int N, int D
   const CellDims c = cell_dims(function);
   const size_t es = dtype_size(dtype), btnd = (size_t)B * T * N * D;
   const size_t gmax = (size_t)(c.GW > c.S ? c.GW : c.S);
-  const size_t cache = (size_t)T * N * ((B + 15) / 16) * 16 * D * c.NC * es;
+  const size_t cache = (size_t)T * N * ((B + 15) / 16) * 16 * D * c.NC * es;  // rows padded to 16
   if (btnd * gmax * es >= ((size_t)1 << 31) || cache >= ((size_t)1 << 31))
     return fail(FRNN_E_ARG, "a tensor of this problem reaches 2 GiB; split the batch (fused kernels use 32-bit offsets)");
   return 0;
@@ -151,7 +161,8 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   Bump bp{(unsigned char*)ws, 0};
   FusedFwdWs w;
   w.status = (int*)bp.take(256);
-  const size_t groups = (size_t)N * ((B + 15) / 16);
+  const int tr = tile_rows_for(B, N, p.kw);
+  const size_t groups = (size_t)N * ((B + tr - 1) / tr);
   const size_t llw = (size_t)16 * D / (dtype == FRNN_BF16 ? 2 : 1);
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
   w.zero_bytes = bp.off;  // status + exchange slots must start at zero for every call
@@ -168,7 +179,8 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   Bump bp{(unsigned char*)ws, 0};
   FusedBwdWs w;
   w.status = (int*)bp.take(256);
-  const size_t bt = (B + 15) / 16, groups = (size_t)N * bt;
+  const int tr = tile_rows_for(B, N, p.kw);
+  const size_t bt = (B + tr - 1) / tr, groups = (size_t)N * bt;
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * bwd_inbox_words(D, p.kw) * 8 : 0);
   w.zero_bytes = bp.off;
   w.Rt = bp.take((size_t)N * D * c.GR * D * es);
@@ -272,7 +284,8 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
   if (waves) *waves = p.waves;
   if (tiles_per_wave) *tiles_per_wave = p.utw;
   if (wgs_per_head) *wgs_per_head = p.kw;
-  if (active_wgs) *active_wgs = N * ((B + 15) / 16) * p.kw;
+  const int tr = tile_rows_for(B, N, p.kw);
+  if (active_wgs) *active_wgs = N * ((B + tr - 1) / tr) * p.kw;
   return 0;
 }
 
@@ -310,7 +323,8 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
   e = launch_fill_zero(workspace, w.zero_bytes, st);
   prof_end(st);
   if (e) return hip_fail(e, "workspace clear");
-  const int groups = N * ((B + 15) / 16);
+  const int tr = tile_rows_for(B, N, p.kw);
+  const int groups = N * ((B + tr - 1) / tr);
   int per_launch = groups;
   if (p.kw > 1) {  // workgroups that wait for each other must all be resident
     per_launch = device_cus() / p.kw;
@@ -319,7 +333,7 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
   FwdArgs a;
   a.Wx = Wx; a.R = R; a.b = b; a.s0 = s0; a.states = states; a.cache = cache;
   a.ll = w.ll; a.status = w.status;
-  a.B = B; a.T = T; a.N = N; a.groups_total = groups;
+  a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY", 0);
@@ -371,7 +385,8 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   prof_end(st);
   if (e) return hip_fail(e, "R transpose");
-  const int bt = (B + 15) / 16, groups = N * bt;
+  const int tr = tile_rows_for(B, N, p.kw);
+  const int bt = (B + tr - 1) / tr, groups = N * bt;
   int per_launch = groups;
   if (p.kw > 1) {
     per_launch = device_cus() / p.kw;
@@ -381,7 +396,7 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
   a.Rt = w.Rt; a.s0 = s0; a.states = states; a.cache = cache; a.dstates = dstates;
   a.dWx = dWx; a.dgx = w.dgx; a.ds0 = ds0; a.dbp = w.dbp;
   a.ll = w.ll; a.status = w.status;
-  a.B = B; a.T = T; a.N = N; a.groups_total = groups;
+  a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", 4);  // ~0.12 us: measured best on MI355X
   for (int g0 = 0; g0 < groups; g0 += per_launch) {

@@ -39,7 +39,7 @@ struct BwdArgs {
   float* dbp;      // [batch tiles][G_t][N][D] partial bias sums
   u64* ll; int* status;
   int B, T, N;
-  int grp0, groups, groups_total;
+  int grp0, groups, groups_total, tile_rows;
   int spin_limit, poll_delay;
 };
 
@@ -84,7 +84,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
   const int brow = O::row(r16), esub = O::sub(r16, q4);
-  const int bg = bt * 16 + brow;
+  const int TR = HALF ? 8 : 16;
+  const int bg = bt * TR + brow;
+  const unsigned Bpad = (unsigned)((a.B + 15) / 16) * 16;
   const bool bvalid = bg < B;
   const T* __restrict__ Rt = static_cast<const T*>(a.Rt);
   const unsigned ND = (unsigned)N * D;
@@ -92,7 +94,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
   const rsrc_t rS0 = make_rsrc(a.s0, (size_t)S * B * ND * ES);
   const rsrc_t rDs = make_rsrc(a.dstates, (size_t)S * B * Tn * ND * ES);
-  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * a.groups_total * 16 * D * NC * ES);
+  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * NC * ES);
   const rsrc_t rDw = make_rsrc(a.dWx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rDx = make_rsrc(a.dgx, (size_t)B * Tn * ND * ES);
 
@@ -105,7 +107,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
     st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
     s0_v[u] = bvalid ? ((unsigned)bg * ND + d0) * ES : kInvalidOff;
-    ca_v[u] = bvalid ? ((unsigned)(ub[u] >> 4) * NC * 256 + brow * 16 + esub) * ES : kInvalidOff;
+    ca_v[u] = bvalid ? (((unsigned)(ub[u] >> 4) * NC * Bpad + bg) * 16 + (esub & 15)) * ES : kInvalidOff;
   }
 
   // rtf[r][u][ks]: rows p of the tiles at this wave's position in workgroup (slice + r) % KW,
@@ -152,7 +154,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     for (int u = 0; u < UTW; ++u) {
 #pragma unroll
       for (int c = 0; c < NC; ++c)
-        p.cache[u][c] = buf_load<ND_>(rCa, ca_v[u], ((((unsigned)t * a.groups_total + grp) * (D / 16)) * NC + c) * 256 * ES);
+        p.cache[u][c] = buf_load<ND_>(rCa, ca_v[u], ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
         const unsigned so = ((unsigned)k * B * Tn + t) * ND * ES;

@@ -29,6 +29,7 @@ struct FwdArgs {
   u64* ll; int* status;
   int B, T, N;
   int grp0, groups, groups_total;  // this launch handles groups [grp0, grp0 + groups)
+  int tile_rows;                   // batch rows per group: 8 (half-tile ownership) or 16
   int training, spin_limit, poll_delay;
   long long* trace;  // phase cycle sums per workgroup; only written by -DFRNN_TRACE builds
 };
@@ -76,9 +77,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
   const int brow = O::row(r16), esub = O::sub(r16, q4);
-  const int bg = bt * 16 + brow;  // batch row this lane does the gate math for
+  const int TR = HALF ? 8 : 16;
+  const int bg = bt * TR + brow;  // batch row this lane does the gate math for
   const bool bvalid = bg < B;
-  const int rows_valid = min(16, B - bt * 16);
+  const int rows_valid = min(TR, B - bt * TR);
+  const unsigned Bpad = (unsigned)((B + 15) / 16) * 16;  // rows of the gate cache
   const T* __restrict__ R = static_cast<const T*>(a.R);
   const T* __restrict__ bias_g = static_cast<const T*>(a.b);
   const T* __restrict__ s0 = static_cast<const T*>(a.s0);
@@ -87,7 +90,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 
   const rsrc_t rWx = make_rsrc(a.Wx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
-  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * a.groups_total * 16 * D * NC * ES);
+  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * NC * ES);
 
   int ub[UTW];
   unsigned wx_v[UTW], st_v[UTW], ca_v[UTW];  // per-lane byte offsets; out of range for padded rows
@@ -97,7 +100,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     const unsigned d0 = n * D + ub[u] + esub;
     wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
     st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
-    ca_v[u] = (bvalid && a.training) ? ((unsigned)(ub[u] >> 4) * NC * 256 + brow * 16 + esub) * ES : kInvalidOff;
+    ca_v[u] = (bvalid && a.training) ? (((unsigned)(ub[u] >> 4) * NC * Bpad + bg) * 16 + (esub & 15)) * ES : kInvalidOff;
   }
 
   // ---- resident operands ----------------------------------------------------------------
@@ -136,10 +139,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   for (int idx = tid; idx < 16 * D / 4; idx += NT) {
     const int row = idx / (D / 4), k0 = (idx % (D / 4)) * 4;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
-    if (bt * 16 + row < B) unpack4(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * 16 + row) * ND + (size_t)n * D + k0), v);
+    const bool rv = row < TR && bt * TR + row < B;
+    if (rv) unpack4(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * TR + row) * ND + (size_t)n * D + k0), v);
     lds_write<4>(hbuf[0], row, k0, v);
     if (KW > 1 || HALF) {  // rows that are never rewritten must be finite in both buffers
-      if (bt * 16 + row >= B) lds_write<4>(hbuf[1], row, k0, v);
+      if (!rv) lds_write<4>(hbuf[1], row, k0, v);
     }
   }
 
@@ -239,11 +243,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
-      // private cache layout [t][group][unit tile][value][16 rows][16 units]
+      // private cache layout [t][head][unit tile][value][batch row][16 units]
 #pragma unroll
       for (int c = 0; c < NC; ++c)
         buf_store<ND_>(pack<E>(cv[c], (T*)0), rCa, ca_v[u],
-                       ((((unsigned)t * a.groups_total + grp) * (D / 16)) * NC + c) * 256 * ES);
+                       ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
     }
 #ifdef FRNN_TRACE
     FRNN_STAMP(c3);

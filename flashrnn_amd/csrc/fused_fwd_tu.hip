@@ -8,7 +8,7 @@ namespace frnn {
 template <>
 int fused_fwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const FwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
-  const bool half = a.B <= 8;  // one batch tile with at most 8 rows: two elements per lane
+  const bool half = a.tile_rows == 8;  // 8-row batch tiles: two elements per lane
 #define FRNN_CASE(Dv, VAR, W, U, K)                                                          \
   if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                 \
     if (half) hipLaunchKernelGGL((fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, true>), grid, dim3(W * 64), 0, st, a);  \
