@@ -116,14 +116,17 @@ static int device_cus() {
   return cached[dev];
 }
 
-// Batch rows per group.  8-row tiles halve the gate math per lane (the larger cost of a step) at
-// the price of twice the workgroups and copies of R, so they are used while every workgroup of the
-// call still gets a compute unit of its own.
+// Batch rows per group: 4, 8 or 16.  Fewer rows per tile mean less gate math per lane and fewer
+// words to poll per step (the larger costs of a step) at the price of more workgroups and copies
+// of R, so the smallest tile is used for which every workgroup of the call still gets a compute
+// unit of its own.
 static int tile_rows_for(int B, int N, int kw) {
   const int forced = env_int("FRNN_TILE_ROWS", 0);
-  if (forced == 8 || forced == 16) return B <= 8 ? 8 : forced;
-  if (B <= 8) return 8;
-  return (long)N * ((B + 7) / 8) * kw <= device_cus() ? 8 : 16;
+  if (forced == 4 || forced == 8 || forced == 16) return forced;
+  const int cus = device_cus();
+  for (int tr = 4; tr < 16; tr *= 2)
+    if ((long)N * ((B + tr - 1) / tr) * kw <= cus) return tr;
+  return 16;
 }
 
 struct Bump {

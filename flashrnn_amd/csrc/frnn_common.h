@@ -85,7 +85,9 @@ __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest e
 // E consecutive elements of the storage type as NDW dwords (bf16: two per dword, f32: one).
 // ---------------------------------------------------------------------------------------
 template <int N> struct Dw { unsigned v[N]; };
-template <typename T, int E> struct NDW { static constexpr int value = E * (int)sizeof(T) / 4; };
+// dwords that hold E elements of T; a single bf16 (E = 1) still takes one dword in registers and
+// is moved with 16-bit memory operations (the SUB flag below)
+template <typename T, int E> struct NDW { static constexpr int value = (E * (int)sizeof(T) + 3) / 4; static constexpr bool SUB = E * (int)sizeof(T) < 4; };
 
 typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
@@ -96,18 +98,24 @@ __device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {  // v_cvt_pk
   const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
   return __builtin_bit_cast(unsigned, h);
 }
-template <int E> __device__ __forceinline__ void unpack(const Dw<E / 2>& d, float* o, bf16_t*) {
+template <int E> __device__ __forceinline__ void unpack(const Dw<(E + 1) / 2>& d, float* o, bf16_t*) {
+  if constexpr (E == 1) { o[0] = __uint_as_float(d.v[0] << 16); }
+  else {
 #pragma unroll
-  for (int k = 0; k < E / 2; ++k) { o[2 * k] = __uint_as_float(d.v[k] << 16); o[2 * k + 1] = __uint_as_float(d.v[k] & 0xffff0000u); }
+    for (int k = 0; k < E / 2; ++k) { o[2 * k] = __uint_as_float(d.v[k] << 16); o[2 * k + 1] = __uint_as_float(d.v[k] & 0xffff0000u); }
+  }
 }
 template <int E> __device__ __forceinline__ void unpack(const Dw<E>& d, float* o, float*) {
 #pragma unroll
   for (int k = 0; k < E; ++k) o[k] = __uint_as_float(d.v[k]);
 }
-template <int E> __device__ __forceinline__ Dw<E / 2> pack(const float* i, bf16_t*) {
-  Dw<E / 2> d;
+template <int E> __device__ __forceinline__ Dw<(E + 1) / 2> pack(const float* i, bf16_t*) {
+  Dw<(E + 1) / 2> d;
+  if constexpr (E == 1) { d.v[0] = pack_bf16x2(i[0], 0.f); }
+  else {
 #pragma unroll
-  for (int k = 0; k < E / 2; ++k) d.v[k] = pack_bf16x2(i[2 * k], i[2 * k + 1]);
+    for (int k = 0; k < E / 2; ++k) d.v[k] = pack_bf16x2(i[2 * k], i[2 * k + 1]);
+  }
   return d;
 }
 template <int E> __device__ __forceinline__ Dw<E> pack(const float* i, float*) {
@@ -128,15 +136,17 @@ constexpr unsigned kInvalidOff = 0x80000000u;
 __device__ __forceinline__ rsrc_t make_rsrc(const void* p, size_t bytes) {
   return __builtin_amdgcn_make_buffer_rsrc(const_cast<void*>(p), 0, (int)(bytes > 0x7fffffffu ? 0x7fffffffu : bytes), 0x00020000);
 }
-template <int N> __device__ __forceinline__ Dw<N> buf_load(rsrc_t r, unsigned voff, unsigned soff) {
+template <int N, bool SUB = false> __device__ __forceinline__ Dw<N> buf_load(rsrc_t r, unsigned voff, unsigned soff) {
   Dw<N> d;
-  if constexpr (N == 1) { d.v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0); }
+  if constexpr (SUB) { static_assert(N == 1, "one 16-bit element"); d.v[0] = __builtin_amdgcn_raw_buffer_load_b16(r, voff, soff, 0); }
+  else if constexpr (N == 1) { d.v[0] = __builtin_amdgcn_raw_buffer_load_b32(r, voff, soff, 0); }
   else if constexpr (N == 2) { const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff, soff, 0); d.v[0] = t.x; d.v[1] = t.y; }
   else { static_assert(N == 4, "1, 2 or 4 dwords"); const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); d.v[0] = t.x; d.v[1] = t.y; d.v[2] = t.z; d.v[3] = t.w; }
   return d;
 }
-template <int N> __device__ __forceinline__ void buf_store(const Dw<N>& d, rsrc_t r, unsigned voff, unsigned soff) {
-  if constexpr (N == 1) { __builtin_amdgcn_raw_buffer_store_b32(d.v[0], r, voff, soff, 0); }
+template <int N, bool SUB = false> __device__ __forceinline__ void buf_store(const Dw<N>& d, rsrc_t r, unsigned voff, unsigned soff) {
+  if constexpr (SUB) { static_assert(N == 1, "one 16-bit element"); __builtin_amdgcn_raw_buffer_store_b16((unsigned short)d.v[0], r, voff, soff, 0); }
+  else if constexpr (N == 1) { __builtin_amdgcn_raw_buffer_store_b32(d.v[0], r, voff, soff, 0); }
   else if constexpr (N == 2) { __builtin_amdgcn_raw_buffer_store_b64(u32x2{d.v[0], d.v[1]}, r, voff, soff, 0); }
   else { static_assert(N == 4, "1, 2 or 4 dwords"); __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[0], d.v[1], d.v[2], d.v[3]}, r, voff, soff, 0); }
 }
@@ -174,6 +184,9 @@ __device__ __forceinline__ unsigned ll_payload(bf16_t*, u64 w) {
 }
 __device__ __forceinline__ unsigned ll_payload(float*, u64 w) { return (unsigned)w; }
 
+__device__ __forceinline__ void ll_store32(unsigned* p, unsigned v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ u64 ll_load(const u64* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

@@ -16,36 +16,45 @@
 // Ownership.  The 16x16 MFMA result gives lane l the 4 rows 4*(l/16)..+3 of column l%16, i.e.
 // (with A = weight rows, B = streamed vector) 4 consecutive units of batch row l%16.
 //   FULL: a lane keeps its 4 elements.
-//   HALF (batch <= 8): columns 8..15 are padding, so lanes 8..15 of every 16-lane row take
-//   elements 2,3 of the lane 8 below them (one DPP move each) and every lane does the gate
-//   math of 2 elements instead of 4.
+//   8-row tiles: columns 8..15 are padding, so lanes 8..15 of every 16-lane row take elements
+//   2,3 of the lane 8 below them (one DPP move each) and every lane does the gate math of 2
+//   elements instead of 4.
+//   4-row tiles: one more DPP move (row_shr:4) leaves one element per lane.
 #pragma once
 #include "frnn_common.h"
 
 namespace frnn {
 
-template <bool HALF> struct Own {
-  static constexpr int E = HALF ? 2 : 4;  // elements per lane per 16-unit tile
-  static __device__ __forceinline__ int row(int r16) { return HALF ? (r16 & 7) : r16; }              // batch row in the tile
-  static __device__ __forceinline__ int sub(int r16, int q4) { return q4 * 4 + (HALF ? 2 * (r16 >> 3) : 0); }  // first unit in the tile
+template <int TR> struct Own {  // TR = batch rows per tile: 16, 8 or 4
+  static_assert(TR == 16 || TR == 8 || TR == 4, "tile rows");
+  static constexpr int E = TR / 4;  // elements per lane per 16-unit tile
+  static __device__ __forceinline__ int row(int r16) { return r16 & (TR - 1); }                   // batch row in the tile
+  static __device__ __forceinline__ int sub(int r16, int q4) { return q4 * 4 + E * (r16 / TR); }  // first unit in the tile
 };
 
-// HALF: lanes 0..7 of a row keep `lo`, lanes 8..15 receive `hi` of the lane 8 below (row_shr:8)
+// lanes 0..7 of a 16-lane row keep `lo`, lanes 8..15 receive `hi` of the lane 8 below (row_shr:8)
 __device__ __forceinline__ float half_pick(float lo, float hi) {
   return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, lo), __builtin_bit_cast(int, hi),
                                                               0x118, 0xF, 0xC, false));
 }
-template <bool HALF> __device__ __forceinline__ void own_elems(const f32x4& acc, float* out) {
-  if constexpr (HALF) { out[0] = half_pick(acc[0], acc[2]); out[1] = half_pick(acc[1], acc[3]); }
-  else { out[0] = acc[0]; out[1] = acc[1]; out[2] = acc[2]; out[3] = acc[3]; }
+// lanes 0..3 and 8..11 keep `lo`, lanes 4..7 and 12..15 receive `hi` of the lane 4 below (row_shr:4)
+__device__ __forceinline__ float quarter_pick(float lo, float hi) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(__builtin_bit_cast(int, lo), __builtin_bit_cast(int, hi),
+                                                              0x114, 0xF, 0xA, false));
+}
+template <int TR> __device__ __forceinline__ void own_elems(const f32x4& acc, float* out) {
+  if constexpr (TR == 16) { out[0] = acc[0]; out[1] = acc[1]; out[2] = acc[2]; out[3] = acc[3]; }
+  else if constexpr (TR == 8) { out[0] = half_pick(acc[0], acc[2]); out[1] = half_pick(acc[1], acc[3]); }
+  else { out[0] = quarter_pick(half_pick(acc[0], acc[2]), half_pick(acc[1], acc[3])); }
 }
 
 // LDS writes of E consecutive elements (row, k0..k0+E-1) in fragment order; k0 % E == 0
 template <int E> __device__ __forceinline__ void lds_write(bf16_t* buf, int row, int k0, const float* v) {
-  const Dw<E / 2> p = pack<E>(v, (bf16_t*)0);
+  const Dw<(E + 1) / 2> p = pack<E>(v, (bf16_t*)0);
   unsigned* dst = reinterpret_cast<unsigned*>(buf + ST<bf16_t>::frag_elem(row, k0));
   if constexpr (E == 4) *reinterpret_cast<uint2*>(dst) = make_uint2(p.v[0], p.v[1]);
-  else dst[0] = p.v[0];
+  else if constexpr (E == 2) dst[0] = p.v[0];
+  else *reinterpret_cast<unsigned short*>(dst) = (unsigned short)p.v[0];
 }
 template <int E> __device__ __forceinline__ void lds_write(float* buf, int row, int k0, const float* v) {
 #pragma unroll
@@ -54,9 +63,13 @@ template <int E> __device__ __forceinline__ void lds_write(float* buf, int row, 
 
 // tagged global stores of E consecutive elements (row, k0..) for step t
 template <int E> __device__ __forceinline__ void ll_write(bf16_t*, u64* slot, int row, int k0, const float* v, int t) {
-  const int q = ST<bf16_t>::frag_elem(row, k0) >> 1;
+  if constexpr (E == 1) {  // one 32-bit tagged half of a word; the other half belongs to another lane
+    ll_store32(reinterpret_cast<unsigned*>(slot) + ST<bf16_t>::frag_elem(row, k0), (tag16(t) << 16) | (pack_bf16x2(v[0], 0.f) & 0xffffu));
+  } else {
+    const int q = ST<bf16_t>::frag_elem(row, k0) >> 1;
 #pragma unroll
-  for (int k = 0; k < E / 2; ++k) ll_store(slot + q + k, ll_pack((bf16_t*)0, v[2 * k], v[2 * k + 1], t));
+    for (int k = 0; k < E / 2; ++k) ll_store(slot + q + k, ll_pack((bf16_t*)0, v[2 * k], v[2 * k + 1], t));
+  }
 }
 template <int E> __device__ __forceinline__ void ll_write(float*, u64* slot, int row, int k0, const float* v, int t) {
 #pragma unroll

@@ -50,13 +50,13 @@ template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_
 template <> __device__ __forceinline__ bf16x8 load_frag_at<bf16_t>(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 template <> __device__ __forceinline__ float load_frag_at<float>(const float* p) { return *p; }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW, bool HALF>
+template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR>
 __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
   typedef typename X::Frag Frag;
-  typedef Own<HALF> O;
+  typedef Own<TR> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
   constexpr int NT = WAVES * 64, UT_WG = WAVES * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
@@ -69,6 +69,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   constexpr int RC = KW == 1 ? 1 : ((KW - 1) < 3 ? (KW - 1) : 3);  // remote sources polled together
   constexpr size_t INW = bwd_inbox_words(D, KW);
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
+  constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
   constexpr unsigned ES = sizeof(T);
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
@@ -84,7 +85,6 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
   const int brow = O::row(r16), esub = O::sub(r16, q4);
-  const int TR = HALF ? 8 : 16;
   const int bg = bt * TR + brow;
   const unsigned Bpad = (unsigned)((a.B + 15) / 16) * 16;
   const bool bvalid = bg < B;
@@ -127,7 +127,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     }
   }
 
-  // zero both LDS buffers once (rows 8..15 are never written in HALF mode) and the flag
+  // zero both LDS buffers once (rows beyond the tile are never written) and the flag
   for (int idx = tid; idx < (2 * 16 * KDL * (int)sizeof(T)) / 4 + 1; idx += NT) reinterpret_cast<unsigned*>(smem_raw)[idx] = 0u;
 
   float ds[UTW][E][S];
@@ -154,13 +154,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     for (int u = 0; u < UTW; ++u) {
 #pragma unroll
       for (int c = 0; c < NC; ++c)
-        p.cache[u][c] = buf_load<ND_>(rCa, ca_v[u], ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
+        p.cache[u][c] = buf_load<ND_, SB>(rCa, ca_v[u], ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
         const unsigned so = ((unsigned)k * B * Tn + t) * ND * ES;
-        p.sn[u][k] = buf_load<ND_>(rSt, st_v[u], so);
-        p.dso[u][k] = buf_load<ND_>(rDs, st_v[u], so);
-        p.sp[u][k] = buf_load<ND_>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * B * ND * ES : so - ND * ES);
+        p.sn[u][k] = buf_load<ND_, SB>(rSt, st_v[u], so);
+        p.dso[u][k] = buf_load<ND_, SB>(rDs, st_v[u], so);
+        p.sp[u][k] = buf_load<ND_, SB>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * B * ND * ES : so - ND * ES);
       }
     }
   };
@@ -202,8 +202,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
 #pragma unroll
       for (int g = 0; g < GW; ++g)
-        buf_store<ND_>(pack<E>(dgw[g], (T*)0), rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
-      if (F == FRNN_GRU) buf_store<ND_>(pack<E>(dgr[0], (T*)0), rDx, st_v[u], (unsigned)t * ND * ES);
+        buf_store<ND_, SB>(pack<E>(dgw[g], (T*)0), rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
+      if (F == FRNN_GRU) buf_store<ND_, SB>(pack<E>(dgr[0], (T*)0), rDx, st_v[u], (unsigned)t * ND * ES);
 #pragma unroll
       for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
     }
@@ -236,7 +236,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float own[E];
-      own_elems<HALF>(acc[0][u], own);
+      own_elems<TR>(acc[0][u], own);
 #pragma unroll
       for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
     }
@@ -250,7 +250,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
         for (int u = 0; u < UTW; ++u) {
           float part[E];
-          own_elems<HALF>(acc[r][u], part);
+          own_elems<TR>(acc[r][u], part);
           u64* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
 #pragma unroll
           for (int e = 0; e < E; ++e) ll_store(dst + e * 64, ll_pack((float*)0, part[e], t));
@@ -314,15 +314,16 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       float v[E];
 #pragma unroll
       for (int e = 0; e < E; ++e) v[e] = ds[u][e][k];
-      buf_store<ND_>(pack<E>(v, (T*)0), rD0, s0_v[u], (unsigned)k * B * ND * ES);
+      buf_store<ND_, SB>(pack<E>(v, (T*)0), rD0, s0_v[u], (unsigned)k * B * ND * ES);
     }
 #pragma unroll
     for (int g = 0; g < GT; ++g)
 #pragma unroll
       for (int e = 0; e < E; ++e) {
         float v = dead ? __uint_as_float(0x7fc00000u) : dbacc[u][e][g];
-        v += __shfl_xor(v, 1); v += __shfl_xor(v, 2); v += __shfl_xor(v, 4);
-        if (!HALF) v += __shfl_xor(v, 8);
+        v += __shfl_xor(v, 1); v += __shfl_xor(v, 2);
+        if (TR >= 8) v += __shfl_xor(v, 4);
+        if (TR == 16) v += __shfl_xor(v, 8);
         if (brow == 0) a.dbp[(((size_t)bt * GT + g) * N + n) * D + ub[u] + esub + e] = v;
       }
   }

@@ -48,14 +48,14 @@ template <> __device__ __forceinline__ float load_frag<float>(const float* row, 
   return row[ks * 4 + kq];
 }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW, bool HALF>
+template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR>
 __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
   typedef typename X::Vec4 Vec4;
   typedef typename X::Frag Frag;
-  typedef Own<HALF> O;
+  typedef Own<TR> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
   constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
@@ -64,6 +64,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int NCA = NC > 0 ? NC : 1;
   constexpr int GX = GT - GR > 0 ? GT - GR : 1;
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
+  constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
   constexpr unsigned ES = sizeof(T);
 
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
@@ -77,7 +78,6 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
   const int brow = O::row(r16), esub = O::sub(r16, q4);
-  const int TR = HALF ? 8 : 16;
   const int bg = bt * TR + brow;  // batch row this lane does the gate math for
   const bool bvalid = bg < B;
   const int rows_valid = min(TR, B - bt * TR);
@@ -142,7 +142,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     const bool rv = row < TR && bt * TR + row < B;
     if (rv) unpack4(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * TR + row) * ND + (size_t)n * D + k0), v);
     lds_write<4>(hbuf[0], row, k0, v);
-    if (KW > 1 || HALF) {  // rows that are never rewritten must be finite in both buffers
+    if (KW > 1 || TR < 16) {  // rows that are never rewritten must be finite in both buffers
       if (!rv) lds_write<4>(hbuf[1], row, k0, v);
     }
   }
@@ -157,7 +157,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
-      for (int g = 0; g < GW; ++g) dst[u][g] = buf_load<ND_>(rWx, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
+      for (int g = 0; g < GW; ++g) dst[u][g] = buf_load<ND_, SB>(rWx, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
   };
   load_wx(wxA, 0);
   __syncthreads();
@@ -219,7 +219,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     for (int u = 0; u < UTW; ++u) {
       float ryv[GR][E], wxv[GW][E];
 #pragma unroll
-      for (int g = 0; g < GR; ++g) own_elems<HALF>(acc[u][g], ryv[g]);
+      for (int g = 0; g < GR; ++g) own_elems<TR>(acc[u][g], ryv[g]);
 #pragma unroll
       for (int g = 0; g < GW; ++g) unpack<E>(wc[u][g], wxv[g], (T*)0);
       float cv[NCA][E];
@@ -242,11 +242,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       else ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
 #pragma unroll
       for (int k = 0; k < S; ++k)
-        buf_store<ND_>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
+        buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
       // private cache layout [t][head][unit tile][value][batch row][16 units]
 #pragma unroll
       for (int c = 0; c < NC; ++c)
-        buf_store<ND_>(pack<E>(cv[c], (T*)0), rCa, ca_v[u],
+        buf_store<ND_, SB>(pack<E>(cv[c], (T*)0), rCa, ca_v[u],
                        ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
     }
 #ifdef FRNN_TRACE
@@ -278,7 +278,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     for (int e = 0; e < E; ++e) nanv[e] = __uint_as_float(0x7fc00000u);
     for (int tt = 0; tt < Tn; ++tt)
 #pragma unroll
-      for (int u = 0; u < UTW; ++u) buf_store<ND_>(pack<E>(nanv, (T*)0), rSt, st_v[u], (unsigned)tt * ND * ES);
+      for (int u = 0; u < UTW; ++u) buf_store<ND_, SB>(pack<E>(nanv, (T*)0), rSt, st_v[u], (unsigned)tt * ND * ES);
   }
 }
 

@@ -9,11 +9,11 @@ template <>
 int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
   const size_t lds = (size_t)2 * 16 * Cell<FRNN_F>::GR * (p.D / p.kw) * sizeof(FRNN_TU_T) + 16;
-  const bool half = a.tile_rows == 8;
 #define FRNN_CASE(Dv, VAR, W, U, K)                                                                     \
   if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                            \
-    auto kern = half ? fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, true>                            \
-                     : fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, false>;                          \
+    auto kern = a.tile_rows == 4 ? fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4>                   \
+              : a.tile_rows == 8 ? fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 8>                   \
+                                 : fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 16>;                 \
     if (lds > 65536) {                                                                                   \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
       if (e != hipSuccess) return (int)e;                                                                \

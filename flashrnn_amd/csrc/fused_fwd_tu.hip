@@ -8,11 +8,11 @@ namespace frnn {
 template <>
 int fused_fwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const FwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
-  const bool half = a.tile_rows == 8;  // 8-row batch tiles: two elements per lane
 #define FRNN_CASE(Dv, VAR, W, U, K)                                                          \
   if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                 \
-    if (half) hipLaunchKernelGGL((fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, true>), grid, dim3(W * 64), 0, st, a);  \
-    else hipLaunchKernelGGL((fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, false>), grid, dim3(W * 64), 0, st, a);      \
+    if (a.tile_rows == 4) hipLaunchKernelGGL((fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4>), grid, dim3(W * 64), 0, st, a);       \
+    else if (a.tile_rows == 8) hipLaunchKernelGGL((fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 8>), grid, dim3(W * 64), 0, st, a);  \
+    else hipLaunchKernelGGL((fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 16>), grid, dim3(W * 64), 0, st, a);                       \
     return (int)hipGetLastError();                                                            \
   }
   FRNN_TU_PLANS(FRNN_CASE)

@@ -68,7 +68,8 @@ def test_plan_and_sizes(lib):
     out = [ctypes.c_int() for _ in range(4)]
     assert lib.frnn_fused_plan(L, 0, 8, 3, 256, 0, *[ctypes.byref(o) for o in out]) == 0
     waves, utw, kw, active = (o.value for o in out)
-    assert 16 * waves * utw * kw == 256 and active == 3 * kw
+    # workgroups = heads x batch tiles (of 4, 8 or 16 rows, by the compute units at hand) x kw
+    assert 16 * waves * utw * kw == 256 and active in (3 * kw, 6 * kw)
     # gate cache: T * N * padded batch * D * values * bytes
     assert lib.frnn_fused_cache_bytes(L, 0, 8, 1024, 3, 256) == 1024 * 3 * 16 * 256 * 4 * 2
     assert lib.frnn_alt_cache_bytes(L, 0, 8, 1024, 3, 256) == 1024 * 3 * 8 * 256 * 4 * 2

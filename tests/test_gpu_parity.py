@@ -11,10 +11,10 @@ FUSED_SMALL = [
     ("lstm", 4, 8, 1, 64, "float32"),
     ("lstm", 3, 5, 2, 32, "bfloat16"),
     ("lstm", 1, 1, 1, 32, "bfloat16"),       # single step, single row
-    ("lstm", 9, 3, 2, 64, "bfloat16"),       # ragged batch: one row over the half tile
+    ("lstm", 9, 3, 2, 64, "bfloat16"),       # ragged batch: one row over two 4-row tiles
     ("lstm", 20, 6, 2, 128, "bfloat16"),     # two batch tiles, second ragged
-    ("lstm", 8, 16, 3, 256, "bfloat16"),     # 4 workgroups per head, half-tile ownership
-    ("lstm", 16, 9, 1, 256, "bfloat16"),     # 4 workgroups per head, full tile
+    ("lstm", 8, 16, 3, 256, "bfloat16"),     # 4 workgroups per head
+    ("lstm", 16, 9, 1, 256, "bfloat16"),
     ("lstm", 33, 4, 1, 256, "bfloat16"),     # 3 batch tiles x 4 workgroups
     ("lstm", 16, 5, 1, 512, "bfloat16"),     # 8 workgroups per head
     ("lstm", 4, 6, 1, 256, "float32"),       # fp32, 4 workgroups per head
@@ -40,6 +40,26 @@ FUSED_SMALL = [
 def test_fused_matches_oracle(gpu, function, B, T, N, D, dtype, init):
     print(f"case fused {function} B{B} T{T} N{N} D{D} {dtype} init={init}", flush=True)
     check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=7, init=init)
+
+
+# The library picks 4-, 8- or 16-row batch tiles from the batch size and the device's compute
+# units; FRNN_TILE_ROWS forces one so that every ownership mode is covered on any device.
+TILINGS = [
+    ("lstm", 9, 6, 2, 256, "bfloat16"),      # ragged in every tiling, 4 workgroups per head
+    ("lstm", 21, 5, 1, 64, "float32"),
+    ("gru", 20, 7, 2, 128, "bfloat16"),
+    ("slstm", 6, 8, 2, 192, "bfloat16"),
+    ("elman", 18, 5, 1, 1024, "bfloat16"),
+    ("elman", 3, 6, 2, 32, "float32"),
+]
+
+
+@pytest.mark.parametrize("function,B,T,N,D,dtype", TILINGS)
+@pytest.mark.parametrize("tile_rows", [4, 8, 16])
+def test_fused_every_batch_tiling(gpu, monkeypatch, tile_rows, function, B, T, N, D, dtype):
+    print(f"case tiling rows={tile_rows} {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
+    monkeypatch.setenv("FRNN_TILE_ROWS", str(tile_rows))
+    check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=13, init="randn")
 
 
 ALT_SMALL = [

@@ -64,22 +64,27 @@ def test_fused_and_alternating_agree(gpu, function, B, T, N, D, seed, init, fb):
         assert not bool((err > 4e-2 * torch.clamp(ref.abs(), min=1.0)).any()), (k, float(err.max()))
 
 
-def test_batch_rows_are_independent_of_padding(gpu):
+@pytest.mark.parametrize("tile_rows", [4, 8, 16])
+def test_batch_rows_are_independent_of_padding(gpu, monkeypatch, tile_rows):
     """Rows of a run equal the same rows of a run with more rows: padded rows of the MFMA tile never
-    reach valid rows.  Bit for bit within one ownership mode (B <= 8: half tile; B > 8: full tiles);
-    between the two modes the compiler schedules the same fp32 math differently, so they agree to
-    rounding only."""
-    print("case padding", flush=True)
+    reach valid rows.  Bit for bit within one batch tiling (forced here); between tilings the
+    compiler schedules the same fp32 math differently, so those agree to rounding only."""
+    print(f"case padding rows={tile_rows}", flush=True)
     function, T, N, D = "lstm", 33, 2, 256
     inp = make_inputs(function, 21, T, N, D, 5, init="randn", round_to=torch.bfloat16)
-    outs = {}
-    for B in (5, 8, 16, 21):
+
+    def run(B):
         sub = {k: (v[:B] if k == "Wx" else v[:, :B] if k in ("states", "dstates") else v) for k, v in inp.items()}
-        outs[B] = _run(gpu, function, sub, "hip_fused")[0]
+        return _run(gpu, function, sub, "hip_fused")[0]
+
+    monkeypatch.setenv("FRNN_TILE_ROWS", str(tile_rows))
+    outs = {B: run(B) for B in (3, 5, 8, 16, 21)}
+    monkeypatch.setenv("FRNN_TILE_ROWS", str(16 if tile_rows == 4 else 4))
+    other = run(21)
     torch.cuda.synchronize()
-    assert torch.equal(outs[5], outs[8][:, :5])
-    assert torch.equal(outs[16], outs[21][:, :16])
-    assert float((outs[8].float() - outs[16][:, :8].float()).abs().max()) <= 2e-2
+    for B in (3, 5, 8, 16):
+        assert torch.equal(outs[B], outs[21][:, :B]), B
+    assert float((outs[21].float() - other.float()).abs().max()) <= 2e-2
 
 
 def test_padded_rows_do_not_reach_weight_gradients(gpu):
