@@ -4,42 +4,49 @@
 //
 // X(D, VARIANT, WAVES, UTW, KW):  D = 16 * UTW * WAVES * KW.
 //   R registers per lane = UTW * G_r * D / 8 (bf16) or UTW * G_r * D / 4 (f32); a workgroup of
-//   4 waves (one per SIMD) may use up to 512 VGPRs per lane, one of 8 waves 256.
+//   4 waves (one per SIMD) may use up to 512 VGPRs per lane, one of 8 waves 256, of 16 waves 128.
 // VARIANT 0 is the default; others are alternatives selectable with FRNN_FUSED_VARIANT for tuning.
-// Forward and backward may tile differently (the gate cache layout does not depend on the plan);
-// FRNN_BWD_PLANS_* default to the forward lists except where the backward kernel needs more
-// registers per tile.
+// Forward and backward tile independently (the gate cache layout does not depend on the plan).
 #pragma once
 
 namespace frnn {
 struct Plan { int D, variant, waves, utw, kw; };
 }
 
+// Measured on MI355X (T = 1024, bf16): when the head fits one workgroup, one tile per wave and
+// 8..16 waves (2..4 per SIMD, so one wave's gate math hides behind another's MFMAs) beats 4 waves
+// with several tiles each; when it does not fit, 4 waves with one tile each and more workgroups
+// beat fewer, fuller workgroups (the step is a dependency chain, not a throughput problem).
 // ---- 4 recurrent gate rows per unit (lstm, slstm) --------------------------------------------
 #define FRNN_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 2, 2, 1, 8) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 1, 3) \
+  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 2, 2, 1, 8) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+#define FRNN_BWD_PLANS_GR4_BF16(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 4, 1, 3) X(192, 1, 12, 1, 1) \
+  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 2, 2, 1, 8) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
 #define FRNN_PLANS_GR4_F32(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(128, 1, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+#define FRNN_BWD_PLANS_GR4_F32 FRNN_PLANS_GR4_F32
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
+  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+#define FRNN_BWD_PLANS_GR3_BF16(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 1, 3) \
+  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
 #define FRNN_PLANS_GR3_F32(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+#define FRNN_BWD_PLANS_GR3_F32 FRNN_PLANS_GR3_F32
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) X(256, 0, 4, 4, 1) \
-  X(512, 0, 4, 2, 4) X(512, 1, 4, 4, 2) X(1024, 0, 4, 1, 16)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
+  X(256, 0, 16, 1, 1) X(256, 1, 4, 4, 1) X(512, 0, 8, 1, 4) X(512, 1, 4, 2, 4) X(512, 2, 16, 1, 2) \
+  X(1024, 0, 8, 1, 8) X(1024, 1, 4, 1, 16)
+#define FRNN_BWD_PLANS_GR1_BF16(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
+  X(256, 0, 16, 1, 1) X(256, 1, 4, 4, 1) X(512, 0, 16, 1, 2) X(512, 1, 4, 2, 4) X(512, 2, 8, 1, 4) \
+  X(1024, 0, 8, 1, 8) X(1024, 1, 4, 1, 16)
 #define FRNN_PLANS_GR1_F32(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) X(256, 0, 4, 4, 1) \
   X(512, 0, 4, 2, 4) X(1024, 0, 4, 1, 16)
-
-#define FRNN_BWD_PLANS_GR4_BF16 FRNN_PLANS_GR4_BF16
-#define FRNN_BWD_PLANS_GR4_F32 FRNN_PLANS_GR4_F32
-#define FRNN_BWD_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(512, 0, 4, 1, 8)
-#define FRNN_BWD_PLANS_GR3_F32 FRNN_PLANS_GR3_F32
-#define FRNN_BWD_PLANS_GR1_BF16 FRNN_PLANS_GR1_BF16
 #define FRNN_BWD_PLANS_GR1_F32 FRNN_PLANS_GR1_F32
