@@ -183,28 +183,48 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     load_wx(wn, min(t + 1, Tn - 1));
 
     // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once
-    f32x4 acc[UTW][GR];
+    // NACC accumulators per (tile, gate), used round robin over the k-steps, so that at least ~4
+    // independent MFMA chains are in flight (a dependent MFMA waits ~3x longer than an independent one)
+    constexpr int NACC_ = UTW * GR >= 3 ? 1 : (UTW * GR == 2 ? 2 : 4);
+    constexpr int NACC = NACC_ < KS ? NACC_ : KS;
+    f32x4 accp[NACC][UTW][GR];
     const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane;
     constexpr int KC = chunk_of(KS);
     static_assert(KS % KC == 0, "k-steps must split into whole chunks");
     Frag hq[2][KC];
 #pragma unroll
     for (int k = 0; k < KC; ++k) hq[0][k] = hf[k * 64];
+    // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
+    __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
     for (int kc = 0; kc < KS / KC; ++kc) {
       if (kc + 1 < KS / KC) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) hq[(kc + 1) & 1][k] = hf[((kc + 1) * KC + k) * 64];
+        __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int k = 0; k < KC; ++k) {
-        const int ks = kc * KC + k;
+        const int ks = kc * KC + k, j = ks % NACC;
 #pragma unroll
         for (int u = 0; u < UTW; ++u)
 #pragma unroll
-          for (int g = 0; g < GR; ++g) acc[u][g] = X::mfma(rf[u][g][ks], hq[kc & 1][k], ks == 0 ? biasc[u][g] : acc[u][g]);
+          for (int g = 0; g < GR; ++g)
+            accp[j][u][g] = X::mfma(rf[u][g][ks], hq[kc & 1][k],
+                                    ks == 0 ? biasc[u][g] : (ks < NACC ? f32x4{0.f, 0.f, 0.f, 0.f} : accp[j][u][g]));
+        // group by group: consecutive MFMAs then never depend on each other
+        if (j == NACC - 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
+    f32x4 acc[UTW][GR];
+#pragma unroll
+    for (int u = 0; u < UTW; ++u)
+#pragma unroll
+      for (int g = 0; g < GR; ++g) {
+        acc[u][g] = accp[0][u][g];
+#pragma unroll
+        for (int j = 1; j < NACC; ++j) acc[u][g] += accp[j][u][g];
+      }
 
 #ifdef FRNN_TRACE
     { float sink = 0.f;
