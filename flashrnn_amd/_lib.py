@@ -15,7 +15,18 @@ DTYPE_IDS = {"bfloat16": 0, "float32": 1}
 # error codes of include/flashrnn_hip.h
 E_ARG, E_UNSUPPORTED, E_NULL, E_ALIGN, E_WORKSPACE, E_DEVICE = -1, -2, -3, -4, -5, -6
 
+
+
+class Options(ctypes.Structure):
+    """frnn_options of include/flashrnn_hip.h (0 / False = option off)."""
+
+    _fields_ = [("forward_clipval", ctypes.c_float), ("gradient_recurrent_clipval", ctypes.c_float),
+                ("gradient_recurrent_cut", c_int)]
+
+
 _P6 = [c_int] * 6
+_FWD = [c_int] * 7 + [c_void_p] * 7 + [c_size_t, c_void_p]
+_BWD = _P6 + [c_void_p] * 11 + [c_size_t, c_void_p]
 _SIGNATURES = {
     "frnn_last_error": (c_char_p, []),
     "frnn_version": (c_char_p, []),
@@ -36,6 +47,10 @@ _SIGNATURES = {
     "frnn_alt_workspace_bytes": (c_size_t, _P6 + [c_int]),
     "frnn_alt_forward": (c_int, [c_int] * 7 + [c_void_p] * 7 + [c_size_t, c_void_p]),
     "frnn_alt_backward": (c_int, _P6 + [c_void_p] * 11 + [c_size_t, c_void_p]),
+    "frnn_fused_forward_opt": (c_int, _FWD + [POINTER(Options)]),
+    "frnn_fused_backward_opt": (c_int, _BWD + [POINTER(Options)]),
+    "frnn_alt_forward_opt": (c_int, _FWD + [POINTER(Options)]),
+    "frnn_alt_backward_opt": (c_int, _BWD + [POINTER(Options)]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

@@ -6,7 +6,7 @@
 
 namespace frnn {
 
-struct AltProblem { int function, dtype, B, T, N, D, training; };
+struct AltProblem { int function, dtype, B, T, N, D, training; float h_clip, g_clip; int cut; };
 
 struct AltFwdBuffers {
   const void* Wx; const void* R; const void* b; const void* s0;

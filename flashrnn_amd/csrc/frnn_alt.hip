@@ -77,6 +77,7 @@ struct AltPwArgs {
                     // storage-type output, the recurrence itself is carried unrounded (only the h
                     // that feeds the GEMM is read back in the storage type), as in the fused path
   int B, T, N, D, t, training;
+  float h_clip;     // > 0: new h clamped to [-h_clip, h_clip]
 };
 
 template <int F, typename T>
@@ -107,6 +108,7 @@ __global__ void __launch_bounds__(256) alt_pw_fwd_kernel(const AltPwArgs a) {
   for (int k = 0; k < S; ++k)
     s[k] = t > 0 ? a.sfp[(size_t)k * BND + idx] : ld(s0 + ((size_t)k * B + b) * ND + (size_t)n * D + d);
   CM::fwd(ry, wx, bb, s, cc);
+  s[0] = clamp_if(s[0], a.h_clip);
 #pragma unroll
   for (int k = 0; k < S; ++k) {
     st_(states + (((size_t)k * B + b) * Tn + t) * ND + (size_t)n * D + d, s[k]);
@@ -126,6 +128,7 @@ struct AltPwBwdArgs {
   float* dsr;      // [S][B][N][D] running cotangent without the recurrent term
   const float* dh; // [B][N][D] recurrent term R^T dg of the step above
   int B, T, N, D, t;
+  float g_clip;    // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip]
 };
 
 template <int F, typename T>
@@ -153,7 +156,7 @@ __global__ void __launch_bounds__(256) alt_pw_bwd_kernel(const AltPwBwdArgs a) {
     sp[k] = t > 0 ? ld(states + so - ND) : ld(s0 + ((size_t)k * B + b) * ND + (size_t)n * D + d);
     ds[k] = a.dsr[(size_t)k * BND + idx];
   }
-  ds[0] += a.dh[idx];
+  ds[0] = clamp_if(ds[0] + a.dh[idx], a.g_clip);
   CM::bwd(cc, sp, sn, dso, ds, gr, gw, gb);
 #pragma unroll
   for (int k = 0; k < S; ++k) a.dsr[(size_t)k * BND + idx] = ds[k];
@@ -211,7 +214,7 @@ static int alt_forward_t(const AltProblem& p, const AltFwdBuffers& bf, hipStream
     g.out = bf.ry; g.B = p.B; g.N = p.N; g.D = p.D; g.M = GR * p.D; g.K = p.D;
     int e = launch_alt_gemm(ST<T>::ID, g, st);
     if (e) return e;
-    AltPwArgs a{bf.Wx, bf.b, bf.s0, bf.states, bf.cache, bf.ry, bf.sfp, p.B, p.T, p.N, p.D, t, p.training};
+    AltPwArgs a{bf.Wx, bf.b, bf.s0, bf.states, bf.cache, bf.ry, bf.sfp, p.B, p.T, p.N, p.D, t, p.training, p.h_clip};
     hipLaunchKernelGGL((alt_pw_fwd_kernel<F, T>), dim3(pw_blocks), dim3(256), 0, st, a);
     e = (int)hipGetLastError();
     if (e) return e;
@@ -227,10 +230,11 @@ static int alt_backward_t(const AltProblem& p, const AltBwdBuffers& bf, hipStrea
   int e = launch_fill_zero(bf.dsr, ((size_t)S * BND + BND) * sizeof(float), st);  // dsr and dh are adjacent
   if (e) return e;
   for (int t = p.T - 1; t >= 0; --t) {
-    AltPwBwdArgs a{bf.s0, bf.states, bf.cache, bf.dstates, bf.dWx, bf.dgx, bf.dg, bf.dsr, bf.dh, p.B, p.T, p.N, p.D, t};
+    AltPwBwdArgs a{bf.s0, bf.states, bf.cache, bf.dstates, bf.dWx, bf.dgx, bf.dg, bf.dsr, bf.dh, p.B, p.T, p.N, p.D, t, p.g_clip};
     hipLaunchKernelGGL((alt_pw_bwd_kernel<F, T>), dim3(pw_blocks), dim3(256), 0, st, a);
     e = (int)hipGetLastError();
     if (e) return e;
+    if (p.cut) continue;  // truncated backpropagation: dh stays zero
     AltGemmArgs g;
     g.A = bf.Rt; g.a_gstride = 0; g.a_hstride = (size_t)p.D * GR * p.D;
     g.V = bf.dg; g.v_bstride = (size_t)p.N * GR * p.D;

@@ -129,6 +129,21 @@ static int tile_rows_for(int B, int N, int kw) {
   return 16;
 }
 
+// Options as the kernels take them: a clip value of 0 switches the clamp off.
+struct Opts { float h_clip, g_clip; int cut; };
+static int parse_opts(const frnn_options* o, int function, bool forward, Opts* out) {
+  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0;
+  if (!o) return 0;
+  if (o->forward_clipval != o->forward_clipval || o->gradient_recurrent_clipval != o->gradient_recurrent_clipval ||
+      o->forward_clipval < 0.f || o->gradient_recurrent_clipval < 0.f)
+    return fail(FRNN_E_ARG, "clip values must be positive, or 0 for none (got %g, %g)", (double)o->forward_clipval,
+                (double)o->gradient_recurrent_clipval);
+  if (forward && o->forward_clipval > 0.f && function == FRNN_ELMAN)
+    return fail(FRNN_E_UNSUPPORTED, "forward_clipval is not available for elman: its backward pass rebuilds tanh' from the stored h");
+  out->h_clip = o->forward_clipval; out->g_clip = o->gradient_recurrent_clipval; out->cut = o->gradient_recurrent_cut != 0;
+  return 0;
+}
+
 struct Bump {
   unsigned char* base; size_t off;
   void* take(size_t bytes) { void* p = base ? base + off : nullptr; off += (bytes + 255) & ~(size_t)255; return p; }
@@ -308,8 +323,19 @@ size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, 
 int frnn_fused_forward(int function, int dtype, int training, int B, int T, int N, int D,
                        const void* Wx, const void* R, const void* b, const void* s0,
                        void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream) {
+  return frnn_fused_forward_opt(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, workspace,
+                                workspace_bytes, stream, nullptr);
+}
+
+int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
+                           const void* Wx, const void* R, const void* b, const void* s0,
+                           void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream,
+                           const frnn_options* opt) {
   g_err[0] = 0;
   int e = check_problem(function, dtype, B, T, N, D);
+  if (e) return e;
+  Opts o;
+  e = parse_opts(opt, function, true, &o);
   if (e) return e;
   Plan p;
   if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
@@ -340,6 +366,7 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY", 0);
+  a.h_clip = o.h_clip;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);
@@ -364,9 +391,21 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
                         const void* cache, const void* dstates,
                         void* dWx, void* ds0, float* dR, float* db,
                         void* workspace, size_t workspace_bytes, void* stream) {
+  return frnn_fused_backward_opt(function, dtype, B, T, N, D, R, b, s0, states, cache, dstates, dWx, ds0, dR, db,
+                                 workspace, workspace_bytes, stream, nullptr);
+}
+
+int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
+                            const void* R, const void* b, const void* s0, const void* states,
+                            const void* cache, const void* dstates,
+                            void* dWx, void* ds0, float* dR, float* db,
+                            void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
   g_err[0] = 0;
   (void)b;
   int e = check_problem(function, dtype, B, T, N, D);
+  if (e) return e;
+  Opts o;
+  e = parse_opts(opt, function, false, &o);
   if (e) return e;
   const CellDims c = cell_dims(function);
   Plan p;
@@ -402,6 +441,7 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", 4);  // ~0.12 us: measured best on MI355X
+  a.g_clip = o.g_clip; a.cut = o.cut;
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
     prof_begin("fused_bwd_kernel", st);
@@ -466,8 +506,19 @@ size_t frnn_alt_workspace_bytes(int function, int dtype, int B, int T, int N, in
 int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N, int D,
                      const void* Wx, const void* R, const void* b, const void* s0,
                      void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream) {
+  return frnn_alt_forward_opt(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, workspace,
+                              workspace_bytes, stream, nullptr);
+}
+
+int frnn_alt_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
+                         const void* Wx, const void* R, const void* b, const void* s0,
+                         void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream,
+                         const frnn_options* opt) {
   g_err[0] = 0;
   int e = frnn_alt_supported(function, dtype, B, N, D);
+  if (e) return e;
+  Opts o;
+  e = parse_opts(opt, function, true, &o);
   if (e) return e;
   if (T <= 0) return fail(FRNN_E_ARG, "non-positive T=%d", T);
   CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
@@ -475,7 +526,7 @@ int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N,
   if (need_cache) CHECK_PTR(cache)
   const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 0);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
-  AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0};
+  AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0, o.h_clip, 0.f, 0};
   AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.ry, w.sfp};
   prof_begin("alt_forward_steps", (hipStream_t)stream);
   e = alt_forward(p, bf, (hipStream_t)stream);
@@ -488,9 +539,21 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
                       const void* cache, const void* dstates,
                       void* dWx, void* ds0, float* dR, float* db,
                       void* workspace, size_t workspace_bytes, void* stream) {
+  return frnn_alt_backward_opt(function, dtype, B, T, N, D, R, b, s0, states, cache, dstates, dWx, ds0, dR, db,
+                               workspace, workspace_bytes, stream, nullptr);
+}
+
+int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
+                          const void* R, const void* b, const void* s0, const void* states,
+                          const void* cache, const void* dstates,
+                          void* dWx, void* ds0, float* dR, float* db,
+                          void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
   g_err[0] = 0;
   (void)b;
   int e = frnn_alt_supported(function, dtype, B, N, D);
+  if (e) return e;
+  Opts o;
+  e = parse_opts(opt, function, false, &o);
   if (e) return e;
   if (T <= 0) return fail(FRNN_E_ARG, "non-positive T=%d", T);
   const CellDims c = cell_dims(function);
@@ -502,7 +565,7 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
   hipStream_t st = (hipStream_t)stream;
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   if (e) return hip_fail(e, "R transpose");
-  AltProblem p{function, dtype, B, T, N, D, 1};
+  AltProblem p{function, dtype, B, T, N, D, 1, 0.f, o.g_clip, o.cut};
   AltBwdBuffers bf{w.Rt, s0, states, cache, dstates, dWx, w.dgx, ds0, w.dg, w.dsr, w.dh};
   prof_begin("alt_backward_steps", st);
   e = alt_backward_scan(p, bf, st);

@@ -125,6 +125,12 @@ template <int E> __device__ __forceinline__ Dw<E> pack(const float* i, float*) {
   return d;
 }
 
+// x clamped to [-v, v] if v > 0, else x untouched (a select, not a branch; NaN stays NaN when off)
+__device__ __forceinline__ float clamp_if(float x, float v) {
+  const float c = fminf(fmaxf(x, -v), v);
+  return v > 0.f ? c : x;
+}
+
 // ---------------------------------------------------------------------------------------
 // Raw buffer access: one descriptor per tensor in SGPRs, 32-bit byte offsets.  An offset at or
 // beyond the tensor's size makes a load return 0 and drops a store, so padded batch rows need

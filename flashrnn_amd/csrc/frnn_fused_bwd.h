@@ -20,6 +20,7 @@
 // Exchanging partial dh (D values per row) instead of dg (G_r*D values per row) moves 2-4x
 // fewer bytes through L2 per step.
 #pragma once
+#include <type_traits>
 #include "frnn_exchange.h"
 #include "frnn_fused_fwd.h"
 #include "frnn_pointwise.h"
@@ -41,6 +42,8 @@ struct BwdArgs {
   int B, T, N;
   int grp0, groups, groups_total, tile_rows;
   int spin_limit, poll_delay;
+  float g_clip;  // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip] (gradient_recurrent_clipval)
+  int cut;       // != 0: no gradient through R h (gradient_recurrent_cut)
 };
 
 // 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][element 4][lane 64]
@@ -168,8 +171,12 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   __syncthreads();
 
   bool dead = false, fail = false;
-  // one reverse step: consumes `pc` (operands of step t), prefetches those of step t-1 into `pn`
-  auto step = [&](const int t, Pre& pc, Pre& pn) __attribute__((always_inline)) {
+  // one reverse step: consumes `pc` (operands of step t), prefetches those of step t-1 into `pn`.
+  // CUT (a std::bool_constant): truncated backpropagation, the step ends with the pointwise carry;
+  // it is a compile-time variant of the step so that the full step carries no trace of it
+  // (a run-time early exit cost 8 % at D = 128)
+  auto step = [&](auto CUT, const int t, Pre& pc, Pre& pn) __attribute__((always_inline)) {
+    constexpr bool cut = decltype(CUT)::value;
     T* const gb = (t & 1) ? gbuf1 : gbuf0;
     load_pre(pn, max(t - 1, 0));
 #pragma unroll
@@ -189,6 +196,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         for (int c = 0; c < NC; ++c) cc[c] = cv[c][e];
 #pragma unroll
         for (int k = 0; k < S; ++k) { sp[k] = spv[k][e]; sn[k] = snv[k][e]; dso[k] = dsov[k][e]; }
+        ds[u][e][0] = clamp_if(ds[u][e][0], a.g_clip);
         CM::bwd(cc, sp, sn, dso, ds[u][e], gr, gw, gb_);
         // padded batch rows contribute nothing (selects, not branches)
 #pragma unroll
@@ -204,9 +212,12 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       for (int g = 0; g < GW; ++g)
         buf_store<ND_, SB>(pack<E>(dgw[g], (T*)0), rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
       if (F == FRNN_GRU) buf_store<ND_, SB>(pack<E>(dgr[0], (T*)0), rDx, st_v[u], (unsigned)t * ND * ES);
+      if constexpr (!cut) {
 #pragma unroll
-      for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
+        for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
+      }
     }
+    if constexpr (cut) return;
     // the barrier also spreads a failed wait of the previous step to the whole workgroup
     if (barrier_or(fail, dead_flag)) { dead = true; return; }
 
@@ -303,12 +314,20 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   };
 
   int t = Tn - 1;
-  for (; t >= 1 && !dead; t -= 2) {
-    step(t, pa, pb);
-    if (dead) break;
-    step(t - 1, pb, pa);
+  if (a.cut) {
+    for (; t >= 1; t -= 2) {
+      step(std::true_type{}, t, pa, pb);
+      step(std::true_type{}, t - 1, pb, pa);
+    }
+    if (t == 0) step(std::true_type{}, 0, pa, pb);
+  } else {
+    for (; t >= 1 && !dead; t -= 2) {
+      step(std::false_type{}, t, pa, pb);
+      if (dead) break;
+      step(std::false_type{}, t - 1, pb, pa);
+    }
+    if (!dead && t == 0) step(std::false_type{}, 0, pa, pb);
   }
-  if (!dead && t == 0) step(0, pa, pb);
   if (!dead && barrier_or(fail, dead_flag)) dead = true;
 
   if (dead) {

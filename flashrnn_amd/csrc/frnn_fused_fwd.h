@@ -31,6 +31,7 @@ struct FwdArgs {
   int grp0, groups, groups_total;  // this launch handles groups [grp0, grp0 + groups)
   int tile_rows;                   // batch rows per group: 8 (half-tile ownership) or 16
   int training, spin_limit, poll_delay;
+  float h_clip;      // > 0: new h clamped to [-h_clip, h_clip] (forward_clipval)
   long long* trace;  // phase cycle sums per workgroup; only written by -DFRNN_TRACE builds
 };
 
@@ -113,16 +114,26 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) rf[u][g][ks] = load_frag<T>(row, ks, q4);
     }
-  f32x4 biasc[UTW][GR];   // bias of the recurrent gate slots, in MFMA C layout
+  // bias of the recurrent gate slots: as the C operand of the first MFMA when a lane keeps all 4
+  // elements of a tile (costs nothing), else added to the lane's own elements in the gate math
+  // (4 registers per gate and tile would hold values the lane never uses)
+  constexpr bool BIAS_C = E == 4;
+  f32x4 biasc[BIAS_C ? UTW : 1][GR];
+  float bown[UTW][GR][BIAS_C ? 1 : E];
   float bx[UTW][E][GX];   // bias of the gate slots without recurrent input
   float s[UTW][E][S];
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
 #pragma unroll
     for (int g = 0; g < GR; ++g) {
-      float v[4];
-      unpack4(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
-      biasc[u][g] = f32x4{v[0], v[1], v[2], v[3]};
+      if constexpr (BIAS_C) {
+        float v[4];
+        unpack4(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
+        biasc[u][g] = f32x4{v[0], v[1], v[2], v[3]};
+      } else {
+#pragma unroll
+        for (int e = 0; e < E; ++e) bown[u][g][e] = (float)bias_g[(size_t)(g * N + n) * D + ub[u] + esub + e];
+      }
     }
 #pragma unroll
     for (int e = 0; e < E; ++e) {
@@ -211,7 +222,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
           for (int g = 0; g < GR; ++g)
             accp[j][u][g] = X::mfma(rf[u][g][ks], hq[kc & 1][k],
-                                    ks == 0 ? biasc[u][g] : (ks < NACC ? f32x4{0.f, 0.f, 0.f, 0.f} : accp[j][u][g]));
+                                    ks < NACC ? ((BIAS_C && ks == 0) ? biasc[u][g] : f32x4{0.f, 0.f, 0.f, 0.f}) : accp[j][u][g]);
         // group by group: consecutive MFMAs then never depend on each other
         if (j == NACC - 1) __builtin_amdgcn_sched_barrier(0);
       }
@@ -239,7 +250,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     for (int u = 0; u < UTW; ++u) {
       float ryv[GR][E], wxv[GW][E];
 #pragma unroll
-      for (int g = 0; g < GR; ++g) own_elems<TR>(acc[u][g], ryv[g]);
+      for (int g = 0; g < GR; ++g) {
+        own_elems<TR>(acc[u][g], ryv[g]);
+        if constexpr (!BIAS_C) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) ryv[g][e] += bown[u][g][e];
+        }
+      }
 #pragma unroll
       for (int g = 0; g < GW; ++g) unpack<E>(wc[u][g], wxv[g], (T*)0);
       float cv[NCA][E];
@@ -252,6 +269,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
         for (int g = 0; g < GW; ++g) wx[g] = wxv[g][e];
         CM::fwd(ry, wx, bx[u][e], s[u][e], cc);
+        s[u][e][0] = clamp_if(s[u][e][0], a.h_clip);
 #pragma unroll
         for (int c = 0; c < NC; ++c) cv[c][e] = cc[c];
 #pragma unroll

@@ -44,8 +44,12 @@ class FlashRNNConfig:
     num_heads: int = -1
     hidden_dim: int = -1
     batch_size: int = 8
+    # truncated backpropagation: no gradient through R h (flashrnn.py:132, backward_cut)
     gradient_recurrent_cut: bool = False
+    # clamp of the cotangent carried into h_t from step t+1 (flashrnn.py:134)
     gradient_recurrent_clipval: Optional[float] = None
+    # clamp of every new h, invisible to the backward pass (flashrnn.py:136); unlike the reference,
+    # which wires gradient_recurrent_clipval into both clamps (:361-382), it acts on its own
     forward_clipval: Optional[float] = None
     num_states: int = 0
     num_gates_r: int = 0
@@ -63,9 +67,10 @@ class FlashRNNConfig:
                 "'vanilla' loop is the test oracle and is not part of the package")
         if self.dtype not in DTYPE_DICT:
             raise ValueError(f"dtype {self.dtype} not supported (bfloat16, float32)")
-        if self.gradient_recurrent_cut or self.gradient_recurrent_clipval is not None \
-                or self.forward_clipval is not None:
-            raise NotImplementedError("gradient cut / clip options are not implemented")
+        for name in ("gradient_recurrent_clipval", "forward_clipval"):
+            v = getattr(self, name)
+            if v is not None and not v > 0:
+                raise ValueError(f"{name} must be positive or None, got {v}")
         (self.num_gates_r, self.num_gates_w, self.num_gates_i, self.num_gates_t,
          self.num_states) = rnn_function_registry[self.function]["gates_states"]
         self.simple_agg = rnn_function_registry[self.function]["simple_agg"]
@@ -82,6 +87,13 @@ class FlashRNNConfig:
 def _entry(backend: str, name: str):
     prefix = "frnn_fused_" if backend == "hip_fused" else "frnn_alt_"
     return getattr(_lib.load_library(), prefix + name)
+
+
+def _options(cfg: "FlashRNNConfig"):
+    import ctypes
+
+    return ctypes.byref(_lib.Options(float(cfg.forward_clipval or 0.0), float(cfg.gradient_recurrent_clipval or 0.0),
+                                     int(bool(cfg.gradient_recurrent_cut))))
 
 
 def _raise(code: int, what: str):
@@ -139,10 +151,10 @@ class _FlashRNNFunction(torch.autograd.Function):
             ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 0)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx.device)
             stream = torch.cuda.current_stream().cuda_stream
-            rc = _entry(cfg.backend, "forward")(
+            rc = _entry(cfg.backend, "forward_opt")(
                 f_id, d_id, int(training), B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(),
                 s0_k.data_ptr(), states.data_ptr(), cache.data_ptr() if training else None,
-                ws.data_ptr(), ws.numel(), stream)
+                ws.data_ptr(), ws.numel(), stream, _options(cfg))
             if rc != 0:
                 _raise(rc, f"{cfg.backend} forward")
         if cfg.backend == "hip_fused":
@@ -173,10 +185,10 @@ class _FlashRNNFunction(torch.autograd.Function):
             ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 1)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
             stream = torch.cuda.current_stream().cuda_stream
-            rc = _entry(cfg.backend, "backward")(
+            rc = _entry(cfg.backend, "backward_opt")(
                 f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
                 cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
-                ws.data_ptr(), ws.numel(), stream)
+                ws.data_ptr(), ws.numel(), stream, _options(cfg))
             if rc != 0:
                 _raise(rc, f"{cfg.backend} backward")
         if cfg.backend == "hip_fused":

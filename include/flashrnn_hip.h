@@ -131,6 +131,48 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
                       void* dWx, void* ds0, float* dR, float* db,
                       void* workspace, size_t workspace_bytes, void* stream);
 
+/* ---- options of FlashRNNConfig that change what the kernels compute (flashrnn.py:132-136) ------
+ * The reference compiles them in (-DFLASHRNN_FORWARD_CLIPVAL..., -DFLASHRNN_GRADIENT_RECURRENT_CLIPVAL...,
+ * flashrnn.py:361-382) and has a separate backward_cut method (fused/flashrnn.cc:248-336,
+ * alternating/flashrnn.cc:220-302); here they are run-time arguments of *_opt twins of the four
+ * entry points above (opt == NULL or all fields zero: identical to the plain entry point).
+ *   forward_clipval > 0:  every new h is clamped to [-v, v] before it is stored and fed back
+ *     (lstm_fused_pointwise.cuh:75-80); the backward pass does not see the clamp.  Not available
+ *     for FRNN_ELMAN (its backward rebuilds tanh' from the stored h): FRNN_E_UNSUPPORTED.
+ *   gradient_recurrent_clipval > 0:  in every reverse step the cotangent carried into h_t from
+ *     step t+1 is clamped to [-v, v] before the upstream cotangent is added
+ *     (lstm_fused_pointwise.cuh:115-121); ds0 itself is not clamped.
+ *   gradient_recurrent_cut != 0:  no gradient through R h (FLASHRNNCellFusedBackwardCut,
+ *     fused/flashrnn_fused_backward_cut.cu:89-178); dR, db, dWx are still computed.
+ * Unlike the reference (which feeds gradient_recurrent_clipval into both clip defines) each
+ * option acts on its own. */
+typedef struct frnn_options {
+  float forward_clipval;
+  float gradient_recurrent_clipval;
+  int gradient_recurrent_cut;
+} frnn_options;
+
+int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
+                           const void* Wx, const void* R, const void* b, const void* s0,
+                           void* states, void* cache, void* workspace, size_t workspace_bytes,
+                           void* stream, const frnn_options* opt);
+int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
+                            const void* R, const void* b, const void* s0, const void* states,
+                            const void* cache, const void* dstates,
+                            void* dWx, void* ds0, float* dR, float* db,
+                            void* workspace, size_t workspace_bytes, void* stream,
+                            const frnn_options* opt);
+int frnn_alt_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
+                         const void* Wx, const void* R, const void* b, const void* s0,
+                         void* states, void* cache, void* workspace, size_t workspace_bytes,
+                         void* stream, const frnn_options* opt);
+int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
+                          const void* R, const void* b, const void* s0, const void* states,
+                          const void* cache, const void* dstates,
+                          void* dWx, void* ds0, float* dR, float* db,
+                          void* workspace, size_t workspace_bytes, void* stream,
+                          const frnn_options* opt);
+
 #ifdef __cplusplus
 }
 #endif

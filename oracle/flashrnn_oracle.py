@@ -21,11 +21,25 @@ What follows the reference, and where:
   slstm_pointwise.cu:135-214, elman_pointwise.cu:80-120 (and what each forward caches,
   same files, forward kernels).
 
+* options ``forward_clipval`` / ``gradient_recurrent_clipval`` / ``gradient_recurrent_cut``
+  -- what the native pointwise functions do under FLASHRNN_FORWARD_CLIPVAL_VALID and
+  FLASHRNN_GRADIENT_RECURRENT_CLIPVAL_VALID (flashrnn/flashrnn/fused/lstm_fused_pointwise.cuh:75-80,
+  115-121 and the same lines of the gru/elman/slstm files) and what ``backward_cut`` leaves out
+  (flashrnn/flashrnn/fused/flashrnn_fused_backward_cut.cu:89-178: no ``dg R^T`` term).  Each option
+  has its own value here; the reference feeds ``gradient_recurrent_clipval`` into both defines
+  (flashrnn/flashrnn/flashrnn.py:361-382).
+
 Pinning (tests/test_oracle_*.py, none of them re-types these formulas):
   LSTM / GRU / Elman forward and all gradients against torch.nn.LSTM / GRU / RNN;
   sLSTM forward against an un-stabilised float64 brute-force recurrence, the T=1 closed
   form and its invariants; every manual adjoint against float64 autograd of the forward;
-  recurrence glue by the chunked-sequence invariant and non-symmetric R with N > 1.
+  recurrence glue by the chunked-sequence invariant and non-symmetric R with N > 1;
+  the three options by hand-derived closed forms on a scalar Elman cell, by the agreement of
+  the autograd formulation (identity-forward / clamp-backward node, detach) with the explicit
+  reverse scan, and by their no-op limits (huge clip value, R = 0).
+  PARITY UNPINNED: the sLSTM backward under ``forward_clipval`` -- the native adjoint reads the
+  stored (clamped) h (slstm_fused_pointwise.cuh:117-186); only ``flashrnn_oracle_fwbw_manual``
+  restates that and nothing independent checks it.
   The reference holds no golden vectors for this path (its only known-answer test is
   flashrnn/tests/test_lstm.py:70-115, LSTM vs torch.nn.LSTM, which is reproduced).
 """
@@ -102,6 +116,20 @@ def _pw_slstm(Wx_t, Ry, b, s, per_element_first_step=False):
 _PW = {"lstm": _pw_lstm, "gru": _pw_gru, "elman": _pw_elman, "slstm": _pw_slstm}
 
 
+class _ClampGrad(torch.autograd.Function):
+    """Identity whose cotangent is clamped to [-c, c]: the clip the native backward pointwise
+    functions apply to the gradient carried into h_t from step t+1 (lstm_fused_pointwise.cuh:115-121)."""
+
+    @staticmethod
+    def forward(ctx, x, c):
+        ctx.c = c
+        return x.view_as(x)
+
+    @staticmethod
+    def backward(ctx, g):
+        return g.clamp(-ctx.c, ctx.c), None
+
+
 def flashrnn_oracle(
     Wx: torch.Tensor,
     R: torch.Tensor,
@@ -109,8 +137,17 @@ def flashrnn_oracle(
     states: Optional[torch.Tensor] = None,
     function: str = "lstm",
     slstm_per_element_first_step: bool = False,
+    forward_clipval: Optional[float] = None,
+    gradient_recurrent_clipval: Optional[float] = None,
+    gradient_recurrent_cut: bool = False,
 ):
     """Differentiable CPU forward in the arithmetic of ``Wx.dtype``.
+
+    ``forward_clipval``: the new h of every step is clamped to [-v, v]; the backward pass does not
+    see the clamp (straight-through), as the native backward pointwise functions do not.
+    ``gradient_recurrent_clipval``: the cotangent that step t+1 sends to h_t (through R and through
+    the pointwise carry) is clamped before the upstream cotangent of h_t is added; the cotangent
+    of the initial state is not clamped.  ``gradient_recurrent_cut``: no gradient through R h.
 
     Returns ``(all_states [S,B,T,N,D], last_states [S,B,1,N,D])``.
     """
@@ -126,12 +163,19 @@ def flashrnn_oracle(
     pw = _PW[function]
     outs = []
     for t in range(T):
-        Ry = torch.matmul(s[0].transpose(0, 1), Rm)  # [N,B,G_r*D]
+        s_in = s
+        if gradient_recurrent_clipval is not None and t > 0:
+            s_in = (_ClampGrad.apply(s[0], float(gradient_recurrent_clipval)),) + tuple(s[1:])
+        h_rec = s_in[0].detach() if gradient_recurrent_cut else s_in[0]
+        Ry = torch.matmul(h_rec.transpose(0, 1), Rm)  # [N,B,G_r*D]
         Ry = Ry.reshape(N, B, Gr, D).permute(1, 2, 0, 3)  # [B,G_r,N,D]
         if function == "slstm":
-            s = pw(Wx[:, t], Ry, b, s, slstm_per_element_first_step)
+            s = pw(Wx[:, t], Ry, b, s_in, slstm_per_element_first_step)
         else:
-            s = pw(Wx[:, t], Ry, b, s)
+            s = pw(Wx[:, t], Ry, b, s_in)
+        if forward_clipval is not None:
+            h = s[0]
+            s = (h + (h.clamp(-forward_clipval, forward_clipval) - h).detach(),) + tuple(s[1:])
         outs.append(torch.stack(s, 0))  # [S,B,N,D]
     all_states = torch.stack(outs, 2)  # [S,B,T,N,D]
     return all_states, all_states[:, :, -1:]
@@ -141,7 +185,10 @@ def flashrnn_oracle_backward(Wx, R, b, states, function, dstates, **kw):
     """Autograd gradients of ``sum(all_states * dstates)`` w.r.t. (Wx, R, b, states)."""
     leaves = [x.detach().clone().requires_grad_(True) for x in (Wx, R, b, states)]
     out, _ = flashrnn_oracle(leaves[0], leaves[1], leaves[2], leaves[3], function, **kw)
-    grads = torch.autograd.grad(out, leaves, grad_outputs=dstates)
+    grads = torch.autograd.grad(out, leaves, grad_outputs=dstates, allow_unused=True)
+    # a leaf without a path to the output (the initial state of an Elman cell under
+    # gradient_recurrent_cut) has a zero gradient
+    grads = tuple(torch.zeros_like(x) if g is None else g for g, x in zip(grads, leaves))
     return out.detach(), grads
 
 
@@ -221,7 +268,8 @@ def _bw_pointwise(function, cache, s_prev, s_new, ds_out, ds_run):
     raise KeyError(function)
 
 
-def flashrnn_oracle_fwbw_manual(Wx, R, b, states, function, dstates):
+def flashrnn_oracle_fwbw_manual(Wx, R, b, states, function, dstates, forward_clipval=None,
+                                gradient_recurrent_clipval=None, gradient_recurrent_cut=False):
     """Forward with gate cache, then the explicit reverse scan; no autograd.
 
     Returns ``(all_states [S,B,T,N,D], (dWx, dR, db, dstates0 [S,B,1,N,D]))``.
@@ -234,6 +282,8 @@ def flashrnn_oracle_fwbw_manual(Wx, R, b, states, function, dstates):
         for t in range(T):
             Ry = torch.einsum("bnp,gndp->bgnd", s[0], R)
             s, cache = _fw_cache(function, Wx[:, t], Ry, b, s)
+            if forward_clipval is not None:  # after the cache is taken: the cache holds unclipped gates
+                s = (s[0].clamp(-forward_clipval, forward_clipval),) + tuple(s[1:])
             traj.append(s)
             caches.append(cache)
         out = torch.stack([torch.stack(x, 0) for x in traj[1:]], 2)
@@ -243,9 +293,12 @@ def flashrnn_oracle_fwbw_manual(Wx, R, b, states, function, dstates):
         db = torch.zeros_like(b)
         for t in range(T - 1, -1, -1):
             ds_out = [dstates[k, :, t] for k in range(S)]
+            if gradient_recurrent_clipval is not None:
+                ds[0] = ds[0].clamp(-gradient_recurrent_clipval, gradient_recurrent_clipval)
             dg_r, dg_w, dg_b, ds = _bw_pointwise(function, caches[t], traj[t], traj[t + 1], ds_out, ds)
             dg_r = torch.stack(dg_r, 1)  # [B,G_r,N,D]
-            ds[0] = ds[0] + torch.einsum("bgnd,gndp->bnp", dg_r, R)
+            if not gradient_recurrent_cut:
+                ds[0] = ds[0] + torch.einsum("bgnd,gndp->bnp", dg_r, R)
             dR += torch.einsum("bgnd,bnp->gndp", dg_r, traj[t][0])
             dWx[:, t] = torch.stack(dg_w, 1)
             db += torch.stack(dg_b, 1).sum(0)

@@ -21,23 +21,33 @@ of the oracle fed the same bf16-rounded inputs):
 import torch
 
 from oracle import FUNCTIONS, flashrnn_oracle, flashrnn_oracle_backward, make_inputs
+from oracle.flashrnn_oracle import flashrnn_oracle_fwbw_manual
 
 
-def oracle_run(function, inp, dtype, backward=True):
+def oracle_run(function, inp, dtype, backward=True, options=None):
     odt = torch.float32 if dtype == "bfloat16" else torch.float64
+    options = dict(options or {})
     kw = {"slstm_per_element_first_step": True} if function == "slstm" else {}
     args = [inp[k].to(odt) for k in ("Wx", "R", "b", "states")]
+    if backward and function == "slstm" and options.get("forward_clipval") is not None:
+        # the native sLSTM adjoint reads the stored (clamped) h: only the explicit scan states that
+        out, (dWx, dR, db, ds0) = flashrnn_oracle_fwbw_manual(*args, function, inp["dstates"].to(odt), **options)
+        return out, (dWx, dR, db, ds0)
+    kw.update(options)
     if backward:
         return flashrnn_oracle_backward(*args, function, inp["dstates"].to(odt), **kw)
     with torch.no_grad():
         return flashrnn_oracle(*args, function, **kw)[0], None
 
 
-def hip_run(function, inp, dtype, backend, device, backward=True):
-    from flashrnn_amd import flashrnn, last_status
+def hip_run(function, inp, dtype, backend, device, backward=True, options=None):
+    from flashrnn_amd import FlashRNNConfig, flashrnn, last_status
 
     leaves = [inp[k].to(device).requires_grad_(backward) for k in ("Wx", "R", "b", "states")]
-    out, last = flashrnn(*leaves, function=function, backend=backend, dtype=dtype)
+    B, _, _, N, D = inp["Wx"].shape
+    config = FlashRNNConfig(backend=backend, function=function, dtype=dtype, head_dim=D, num_heads=N, batch_size=B,
+                            **(options or {}))
+    out, last = flashrnn(*leaves, config=config)
     grads = None
     if backward:
         grads = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(device).to(out.dtype))
@@ -72,13 +82,13 @@ def assert_close(name, got, ref, dtype, kind):
 
 
 def check_case(device, function, B, T, N, D, dtype, backend, seed=1, init="randn", backward=True,
-               forget_bias_linspace=False):
+               forget_bias_linspace=False, options=None):
     grad_on = "h" if function == "slstm" else "all"
     inp = make_inputs(function, B, T, N, D, seed, init=init,
                       round_to=torch.bfloat16 if dtype == "bfloat16" else None, grad_on=grad_on,
                       forget_bias_linspace=forget_bias_linspace)
-    ref_out, ref_g = oracle_run(function, inp, dtype, backward)
-    out, grads = hip_run(function, inp, dtype, backend, device, backward)
+    ref_out, ref_g = oracle_run(function, inp, dtype, backward, options)
+    out, grads = hip_run(function, inp, dtype, backend, device, backward, options)
     S = FUNCTIONS[function][4]
     for k in range(S):
         assert_close(f"state {k}", out[k], ref_out[k], dtype, "h" if k == 0 else "state")

@@ -131,8 +131,9 @@ def test_python_api_argument_errors():
         FlashRNNConfig(function="rnn")
     with pytest.raises(ValueError):
         FlashRNNConfig(dtype="float16")
-    with pytest.raises(NotImplementedError):
-        FlashRNNConfig(gradient_recurrent_cut=True)
+    with pytest.raises(ValueError):
+        FlashRNNConfig(gradient_recurrent_clipval=-1.0)
+    assert FlashRNNConfig(gradient_recurrent_cut=True, forward_clipval=2.0).gradient_recurrent_cut
     cfg = FlashRNNConfig(function="gru", head_dim=64, num_heads=3)
     assert (cfg.num_gates_r, cfg.num_gates_w, cfg.num_gates_t, cfg.num_states, cfg.hidden_dim) == (3, 3, 4, 1, 192)
     Wx = torch.zeros(2, 3, 4, 1, 32)
@@ -154,3 +155,24 @@ def test_missing_library_is_an_error(monkeypatch, tmp_path):
     monkeypatch.setattr(_lib, "_LIB", None)
     with pytest.raises(RuntimeError, match="missing"):
         _lib.load_library()
+
+
+def test_options_are_validated_before_launch(lib):
+    """frnn_options: negative or NaN clip values are argument errors; forward_clipval has no elman kernel."""
+    import math
+
+    def fwd(entry, function=0, **opt):
+        o = _lib.Options(opt.get("f", 0.0), opt.get("g", 0.0), opt.get("cut", 0))
+        return getattr(lib, entry)(function, 0, 1, 8, 4, 1, 64, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, FAKE, 0, None,
+                                   ctypes.byref(o))
+
+    for entry in ("frnn_fused_forward_opt", "frnn_alt_forward_opt"):
+        assert fwd(entry, f=-1.0) == _lib.E_ARG
+        assert fwd(entry, g=math.nan) == _lib.E_ARG
+        assert fwd(entry, function=_lib.FUNCTION_IDS["elman"], f=0.5) == _lib.E_UNSUPPORTED
+        assert b"elman" in lib.frnn_last_error()
+        assert fwd(entry, f=0.5) == _lib.E_WORKSPACE  # options accepted: the next check is the workspace size
+    for entry in ("frnn_fused_backward_opt", "frnn_alt_backward_opt"):
+        o = _lib.Options(0.0, -2.0, 0)
+        assert getattr(lib, entry)(0, 0, 8, 4, 1, 64, *([FAKE] * 11), 0, None, ctypes.byref(o)) == _lib.E_ARG
+        assert getattr(lib, entry)(0, 0, 8, 4, 1, 64, *([FAKE] * 11), 0, None, None) == _lib.E_WORKSPACE

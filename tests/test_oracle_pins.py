@@ -244,3 +244,121 @@ def test_heads_are_independent_and_R_orientation():
     want = torch.zeros(B, N, D, dtype=DT)
     want[0, 1, 0] = math.tanh(h1)
     assert torch.allclose(out[0, :, 1], want)
+
+
+# ---- clip / cut options -----------------------------------------------------------------------
+def _scalar_elman(w, r, b, h0):
+    """A 1-unit Elman cell over T = len(w) steps, written out: h_t = tanh(w_t + r h_{t-1} + b)."""
+    import math
+
+    h = [h0]
+    for wt in w:
+        h.append(math.tanh(wt + r * h[-1] + b))
+    return h
+
+
+def test_gradient_clip_and_cut_closed_form_scalar_elman():
+    """Loss = h_3 on a scalar Elman cell, T = 3.  By hand: dpre_3 = 1 - h_3^2; the cotangent sent
+    back to h_2 is r*dpre_3, to h_1 r*dpre_2, ...; the clip clamps exactly those carried values,
+    the cut replaces them by 0; the cotangent of h_0 is never clamped."""
+    w, r, b, h0 = [0.3, -0.2, 0.5], 2.5, 0.1, 0.4
+    h = _scalar_elman(w, r, b, h0)
+    d = [1 - x * x for x in h]  # tanh' at h_t
+    Wx = torch.tensor(w, dtype=torch.float64).reshape(1, 3, 1, 1, 1)
+    R = torch.tensor([[[[r]]]], dtype=torch.float64)
+    bb = torch.tensor([[[b]]], dtype=torch.float64)
+    s0 = torch.tensor(h0, dtype=torch.float64).reshape(1, 1, 1, 1, 1)
+    ds = torch.zeros(1, 1, 3, 1, 1, dtype=torch.float64)
+    ds[0, 0, 2] = 1.0
+    clamp = lambda x, c: max(-c, min(c, x))
+    for c in (0.05, 0.7, 100.0):
+        dpre3 = d[3]
+        dpre2 = clamp(r * dpre3, c) * d[2]
+        dpre1 = clamp(r * dpre2, c) * d[1]
+        want_dWx = [dpre1, dpre2, dpre3]
+        want_ds0 = r * dpre1  # not clamped
+        want_dR = dpre1 * h[0] + dpre2 * h[1] + dpre3 * h[2]
+        for run in (lambda: flashrnn_oracle_backward(Wx, R, bb, s0, "elman", ds, gradient_recurrent_clipval=c)[1],
+                    lambda: flashrnn_oracle_fwbw_manual(Wx, R, bb, s0, "elman", ds, gradient_recurrent_clipval=c)[1]):
+            dWx, dR, db, ds0 = run()
+            assert torch.allclose(dWx.flatten(), torch.tensor(want_dWx, dtype=torch.float64), atol=1e-14)
+            assert abs(float(ds0) - want_ds0) < 1e-14 and abs(float(dR) - want_dR) < 1e-14
+            assert abs(float(db) - sum(want_dWx)) < 1e-14
+    # cut: nothing flows back through r
+    for run in (lambda: flashrnn_oracle_backward(Wx, R, bb, s0, "elman", ds, gradient_recurrent_cut=True)[1],
+                lambda: flashrnn_oracle_fwbw_manual(Wx, R, bb, s0, "elman", ds, gradient_recurrent_cut=True)[1]):
+        dWx, dR, db, ds0 = run()
+        assert torch.allclose(dWx.flatten(), torch.tensor([0.0, 0.0, d[3]], dtype=torch.float64), atol=1e-14)
+        assert float(ds0) == 0.0 and abs(float(dR) - d[3] * h[2]) < 1e-14
+
+
+def test_forward_clip_closed_form_scalar_elman():
+    """h is clamped before it is stored and fed back; the gradient is the unclamped one evaluated
+    on the clamped trajectory (straight-through)."""
+    import math
+
+    w, r, b, h0, c = [1.5, -0.2], 0.8, 0.0, 0.0, 0.6
+    g1 = math.tanh(w[0] + r * h0 + b)
+    h1 = max(-c, min(c, g1))
+    assert h1 == c  # the clamp is active at step 1
+    g2 = math.tanh(w[1] + r * h1 + b)
+    Wx = torch.tensor(w, dtype=torch.float64).reshape(1, 2, 1, 1, 1)
+    R = torch.tensor([[[[r]]]], dtype=torch.float64)
+    bb = torch.zeros(1, 1, 1, dtype=torch.float64)
+    s0 = torch.zeros(1, 1, 1, 1, 1, dtype=torch.float64)
+    ds = torch.zeros(1, 1, 2, 1, 1, dtype=torch.float64)
+    ds[0, 0, 1] = 1.0
+    out, (dWx, dR, db, ds0) = flashrnn_oracle_backward(Wx, R, bb, s0, "elman", ds, forward_clipval=c)
+    assert abs(float(out[0, 0, 0]) - c) < 1e-15 and abs(float(out[0, 0, 1]) - g2) < 1e-15
+    dpre2 = 1 - g2 * g2
+    dpre1 = r * dpre2 * (1 - g1 * g1)  # tanh' of the unclamped gate value, as the native kernels cache it
+    assert torch.allclose(dWx.flatten(), torch.tensor([dpre1, dpre2], dtype=torch.float64), atol=1e-14)
+    out2, (dWx2, _, _, _) = flashrnn_oracle_fwbw_manual(Wx, R, bb, s0, "elman", ds, forward_clipval=c)
+    assert torch.equal(out, out2) and torch.allclose(dWx, dWx2, atol=1e-14)
+
+
+@pytest.mark.parametrize("function", ["lstm", "gru", "elman", "slstm"])
+def test_options_autograd_and_explicit_scan_agree(function):
+    """Two independent statements of every option: a clamp-the-cotangent node / detach /
+    straight-through clamp under autograd against the explicit reverse scan."""
+    inp = make_inputs(function, 3, 7, 2, 8, 21, init="randn", grad_on="h" if function == "slstm" else "all")
+    a = [inp[k].double() for k in ("Wx", "R", "b", "states")]
+    a[1] = a[1] * 3  # a recurrent gradient large enough for the clamp to bite
+    ds = inp["dstates"].double()
+    base = {"slstm_per_element_first_step": True} if function == "slstm" else {}
+    plain = flashrnn_oracle_backward(*a, function, ds, **base)[1]
+    cases = [dict(gradient_recurrent_clipval=0.05), dict(gradient_recurrent_cut=True),
+             dict(gradient_recurrent_clipval=0.05, gradient_recurrent_cut=True)]
+    if function != "slstm":  # the native sLSTM adjoint reads the clamped h: only the explicit scan states that
+        cases += [dict(forward_clipval=0.3), dict(forward_clipval=0.3, gradient_recurrent_clipval=0.05)]
+    for kw in cases:
+        o1, g1 = flashrnn_oracle_backward(*a, function, ds, **base, **kw)
+        o2, g2 = flashrnn_oracle_fwbw_manual(*a, function, ds, **kw)
+        assert torch.allclose(o1, o2, atol=1e-12)
+        for k, (x, y) in enumerate(zip(g1, g2)):
+            if function == "slstm" and k == 3:
+                x, y = x[:3], y[:3]  # the stabiliser's cotangent is 0 by design in the explicit scan
+            assert torch.allclose(x, y, atol=1e-10), (kw, k, float((x - y).abs().max()))
+        assert float((g1[0] - plain[0]).abs().max()) > 1e-3, kw  # the option did change something
+
+
+@pytest.mark.parametrize("function", ["lstm", "gru", "elman", "slstm"])
+def test_options_noop_limits(function):
+    """A clip value above every carried value changes nothing; with R = 0 the cut changes nothing."""
+    inp = make_inputs(function, 2, 5, 2, 8, 22, init="randn", grad_on="h" if function == "slstm" else "all")
+    a = [inp[k].double() for k in ("Wx", "R", "b", "states")]
+    ds = inp["dstates"].double()
+    base = {"slstm_per_element_first_step": True} if function == "slstm" else {}
+    o0, g0 = flashrnn_oracle_backward(*a, function, ds, **base)
+    o1, g1 = flashrnn_oracle_backward(*a, function, ds, **base, gradient_recurrent_clipval=1e9, forward_clipval=1e9)
+    assert torch.equal(o0, o1) and all(torch.allclose(x, y, atol=1e-13) for x, y in zip(g0, g1))
+    a0 = [a[0], torch.zeros_like(a[1]), a[2], a[3]]
+    _, g2 = flashrnn_oracle_backward(*a0, function, ds, **base)
+    _, g3 = flashrnn_oracle_backward(*a0, function, ds, **base, gradient_recurrent_cut=True)
+    for k, (x, y) in enumerate(zip(g2, g3)):
+        if k == 1:
+            continue  # dR itself is not zero when R is
+        assert torch.allclose(x, y, atol=1e-13), k
+    # forward clamp: every stored h lies inside the interval and the untouched steps are unchanged
+    o4, _ = flashrnn_oracle_backward(*a, function, ds, **base, forward_clipval=0.25)
+    assert float(o4[0].abs().max()) <= 0.25 + 1e-15
