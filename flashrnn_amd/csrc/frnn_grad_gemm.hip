@@ -42,8 +42,13 @@ int launch_transpose_r(int dtype, const void* R, void* Rt, int N, int D, int GR,
 template <typename T, int TM> struct GemmStage;
 
 template <int TM> struct GemmStage<bf16_t, TM> {
-  static constexpr int LD = 40;  // 32 rows + pad, 80-byte row stride keeps 16-byte alignment
-  bf16_t a[TM][LD], b[TM][LD];   // transposed: [unit][row]
+  // transposed: [unit][row pair], one dword = rows (2k, 2k+1) of a unit.  17 dwords per unit (16 + 1 pad):
+  // an odd stride puts the 64 lanes of a transposing store on 32 different banks and keeps the fragment
+  // reads (4 consecutive dwords per lane) conflict-free; an 8-element row stride would be a multiple of
+  // the bank count for every choice of padding that keeps 16-byte reads aligned (measured: bank
+  // conflicts in 83 % of the LDS-active cycles, the kernel was LDS-bound)
+  static constexpr int LD = 17;
+  unsigned a[TM][LD], b[TM][LD];
 };
 template <int TM> struct GemmStage<float, TM> {
   static constexpr int LD = TM + 4;
@@ -77,53 +82,82 @@ __global__ void __launch_bounds__(256) grad_gemm_kernel(const GradGemmArgs a) {
   const T* __restrict__ H = static_cast<const T*>(a.states_h) + (size_t)n * D + pt * TM;
   const T* __restrict__ H0 = static_cast<const T*>(a.s0_h) + (size_t)n * D + pt * TM;
 
-  const int rr = tid / (TM / EV), cc = (tid % (TM / EV)) * EV;
-
   f32x4 acc[WT][WT];
 #pragma unroll
   for (int i = 0; i < WT; ++i)
 #pragma unroll
     for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  T ga[EV], hb[EV];
-  auto fetch = [&](long r0) __attribute__((always_inline)) {
-    const long r = r0 + rr;
-    if (r < r_end) {
-      const long b = r / Tn, t = r - b * Tn;
-      const T* gp = G + (size_t)r * gld + cc;
-      const T* hp = (t > 0) ? H + (size_t)(r - 1) * ND + cc : H0 + (size_t)b * ND + cc;
+  if constexpr (sizeof(T) == 2) {
+    // thread -> (row pair rp, 4 units from uc): two 8-byte loads per operand, four dword stores
+    const int rp = tid / (TM / 4), uc = (tid % (TM / 4)) * 4;
+    const bool active = rp < 16;
+    uint2 ga[2], hb[2];
+    auto fetch = [&](long r0) __attribute__((always_inline)) {
 #pragma unroll
-      for (int e = 0; e < EV; ++e) { ga[e] = gp[e]; hb[e] = hp[e]; }
-    } else {
-#pragma unroll
-      for (int e = 0; e < EV; ++e) { ga[e] = (T)0.0f; hb[e] = (T)0.0f; }
-    }
-  };
-
-  fetch(r_begin);
-  for (long r0 = r_begin; r0 < r_end; r0 += 32) {
-    __syncthreads();  // previous stage fully consumed
-    if constexpr (sizeof(T) == 2) {
-#pragma unroll
-      for (int e = 0; e < EV; ++e) { sm.a[cc + e][rr] = ga[e]; sm.b[cc + e][rr] = hb[e]; }
-    } else {
-#pragma unroll
-      for (int e = 0; e < EV; ++e) { sm.a[rr][cc + e] = ga[e]; sm.b[rr][cc + e] = hb[e]; }
-    }
-    __syncthreads();
-    if (r0 + 32 < r_end) fetch(r0 + 32);
-    if constexpr (sizeof(T) == 2) {
+      for (int h = 0; h < 2; ++h) {
+        const long r = r0 + 2 * rp + h;
+        ga[h] = make_uint2(0u, 0u); hb[h] = make_uint2(0u, 0u);
+        if (active && r < r_end) {
+          const long b = r / Tn, t = r - b * Tn;
+          ga[h] = *reinterpret_cast<const uint2*>(G + (size_t)r * gld + uc);
+          hb[h] = *reinterpret_cast<const uint2*>((t > 0) ? H + (size_t)(r - 1) * ND + uc : H0 + (size_t)b * ND + uc);
+        }
+      }
+    };
+    fetch(r_begin);
+    for (long r0 = r_begin; r0 < r_end; r0 += 32) {
+      __syncthreads();  // previous stage fully consumed
+      if (active) {
+        // element e of row 2rp in the low half, of row 2rp+1 in the high half
+        sm.a[uc + 0][rp] = (ga[0].x & 0xffffu) | (ga[1].x << 16);
+        sm.a[uc + 1][rp] = (ga[0].x >> 16) | (ga[1].x & 0xffff0000u);
+        sm.a[uc + 2][rp] = (ga[0].y & 0xffffu) | (ga[1].y << 16);
+        sm.a[uc + 3][rp] = (ga[0].y >> 16) | (ga[1].y & 0xffff0000u);
+        sm.b[uc + 0][rp] = (hb[0].x & 0xffffu) | (hb[1].x << 16);
+        sm.b[uc + 1][rp] = (hb[0].x >> 16) | (hb[1].x & 0xffff0000u);
+        sm.b[uc + 2][rp] = (hb[0].y & 0xffffu) | (hb[1].y << 16);
+        sm.b[uc + 3][rp] = (hb[0].y >> 16) | (hb[1].y & 0xffff0000u);
+      }
+      __syncthreads();
+      if (r0 + 32 < r_end) fetch(r0 + 32);
       bf16x8 af[WT], bfr[WT];
 #pragma unroll
       for (int i = 0; i < WT; ++i) {
-        af[i] = *reinterpret_cast<const bf16x8*>(&sm.a[wm * (TM / 2) + i * 16 + r16][q4 * 8]);
-        bfr[i] = *reinterpret_cast<const bf16x8*>(&sm.b[wn * (TM / 2) + i * 16 + r16][q4 * 8]);
+        const unsigned* pa = &sm.a[wm * (TM / 2) + i * 16 + r16][q4 * 4];
+        const unsigned* pb = &sm.b[wn * (TM / 2) + i * 16 + r16][q4 * 4];
+        const u32x4 va = {pa[0], pa[1], pa[2], pa[3]}, vb = {pb[0], pb[1], pb[2], pb[3]};
+        af[i] = __builtin_bit_cast(bf16x8, va);
+        bfr[i] = __builtin_bit_cast(bf16x8, vb);
       }
 #pragma unroll
       for (int i = 0; i < WT; ++i)
 #pragma unroll
         for (int j = 0; j < WT; ++j) acc[i][j] = X::mfma(af[i], bfr[j], acc[i][j]);
-    } else {
+    }
+  } else {
+    const int rr = tid / (TM / EV), cc = (tid % (TM / EV)) * EV;
+    T ga[EV], hb[EV];
+    auto fetch = [&](long r0) __attribute__((always_inline)) {
+      const long r = r0 + rr;
+      if (r < r_end) {
+        const long b = r / Tn, t = r - b * Tn;
+        const T* gp = G + (size_t)r * gld + cc;
+        const T* hp = (t > 0) ? H + (size_t)(r - 1) * ND + cc : H0 + (size_t)b * ND + cc;
+#pragma unroll
+        for (int e = 0; e < EV; ++e) { ga[e] = gp[e]; hb[e] = hp[e]; }
+      } else {
+#pragma unroll
+        for (int e = 0; e < EV; ++e) { ga[e] = (T)0.0f; hb[e] = (T)0.0f; }
+      }
+    };
+    fetch(r_begin);
+    for (long r0 = r_begin; r0 < r_end; r0 += 32) {
+      __syncthreads();  // previous stage fully consumed
+#pragma unroll
+      for (int e = 0; e < EV; ++e) { sm.a[rr][cc + e] = ga[e]; sm.b[rr][cc + e] = hb[e]; }
+      __syncthreads();
+      if (r0 + 32 < r_end) fetch(r0 + 32);
 #pragma unroll
       for (int k4 = 0; k4 < 8; ++k4) {
         float af[WT], bfr[WT];
