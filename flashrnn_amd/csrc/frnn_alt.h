@@ -11,16 +11,14 @@ struct AltProblem { int function, dtype, B, T, N, D, training; float h_clip, g_c
 struct AltFwdBuffers {
   const void* Wx; const void* R; const void* b; const void* s0;
   void* states; void* cache;
-  float* ry;   // [B][N][G_r*D]
   float* sfp;  // [S][B][N][D]
 };
 
 struct AltBwdBuffers {
   const void* Rt; const void* s0; const void* states; const void* cache; const void* dstates;
   void* dWx; void* dgx; void* ds0;
-  void* dg;    // [B][N][G_r*D] storage type
-  float* dsr;  // [S][B][N][D], immediately followed by dh
-  float* dh;   // [B][N][D]
+  void* dg;    // 2 x [B][N][G_r*D] storage type (steps of even / odd index)
+  float* dsr;  // [S][B][N][D]
 };
 
 int alt_forward(const AltProblem& p, const AltFwdBuffers& bf, hipStream_t st);

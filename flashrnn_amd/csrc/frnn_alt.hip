@@ -1,112 +1,120 @@
-// Alternating backend ("hip"): per time step one MFMA GEMM kernel over all heads, then one
-// pointwise kernel; the recurrent matrix is re-read from L2/HBM every step, so any head
-// dimension works.  Replaces flashrnn/flashrnn/alternating/flashrnn_forward.cu:150-267,
+// Alternating backend ("hip"): one kernel launch per time step (the recurrent product of a tile
+// on MFMA, then its gate math); the recurrent matrix is re-read from L2/HBM every step, so any
+// head dimension works.  Replaces flashrnn/flashrnn/alternating/flashrnn_forward.cu:150-267,
 // flashrnn_backward.cu:267-431 and the four *_pointwise.cu files.
 //
-// Differences from the reference: the recurrent pre-activations stay fp32 between the two
-// kernels (the reference rounds them to the storage type, flashrnn_forward.cu:176-181); tensors
-// are read and written in the public layouts; everything runs on the caller's stream.
+// Differences from the reference: product and gate math of a step share one launch and the
+// pre-activations stay in fp32 registers/LDS between them (the reference launches a cuBLAS GEMM and
+// a pointwise kernel and rounds the pre-activations to the storage type in between,
+// flashrnn_forward.cu:176-181); tensors are read and written in the public layouts; everything
+// runs on the caller's stream.
 #include "frnn_alt.h"
 #include "frnn_pointwise.h"
 
 namespace frnn {
 
-// ---------------------------------------------------------------------------------------------
-// out[b][n][m] = sum_k A(n, m)[k] * V[b][n][k]      (M rows per head, K contraction, 16-row
-// batch tiles).  One workgroup = one 16-row M tile x one batch tile; its 4 waves split K and
-// reduce through LDS.  Operands go from global memory straight into MFMA fragments: both are
-// contiguous in k.
-//   row m of head n:  A + (m / D) * a_gstride + n * a_hstride + (m % D) * K
-//   V element:        V + b * v_bstride + n * K + k
-// ---------------------------------------------------------------------------------------------
-struct AltGemmArgs {
-  const void* A; size_t a_gstride, a_hstride;
-  const void* V; size_t v_bstride;
-  float* out;
-  int B, N, D, M, K;
-};
-
-template <typename T>
-__global__ void __launch_bounds__(256) alt_gemm_kernel(const AltGemmArgs a) {
-  typedef ST<T> X;
-  typedef typename X::Frag Frag;
-  __shared__ f32x4 red[3][64];
-  const int m0 = blockIdx.x * 16, n = blockIdx.y, bt = blockIdx.z;
-  const int lane = threadIdx.x & 63, w = threadIdx.x >> 6;
-  const int r16 = lane & 15, q4 = lane >> 4;
-  const int m = m0 + r16;
-  const T* arow = static_cast<const T*>(a.A) + (size_t)(m / a.D) * a.a_gstride + (size_t)n * a.a_hstride + (size_t)(m % a.D) * a.K;
-  const int b = bt * 16 + r16;
-  const bool bvalid = b < a.B;
-  const T* vrow = static_cast<const T*>(a.V) + (size_t)(bvalid ? b : 0) * a.v_bstride + (size_t)n * a.K;
-  const int KS = a.K / X::KM;
-  f32x4 acc = {0.f, 0.f, 0.f, 0.f};
-  for (int ks = w; ks < KS; ks += 4) {
-    const Frag af = load_frag<T>(arow, ks, q4);
-    Frag vf = load_frag<T>(vrow, ks, q4);
-    if (!bvalid) vf = Frag{};
-    acc = X::mfma(af, vf, acc);
-  }
-  if (w > 0) red[w - 1][lane] = acc;
-  __syncthreads();
-  if (w == 0) {
-    acc += red[0][lane]; acc += red[1][lane]; acc += red[2][lane];
-    if (bvalid) *reinterpret_cast<f32x4*>(a.out + ((size_t)b * a.N + n) * a.M + m0 + q4 * 4) = acc;
-  }
-}
-
-static int launch_alt_gemm(int dtype, const AltGemmArgs& a, hipStream_t st) {
-  const dim3 grid(a.M / 16, a.N, (a.B + 15) / 16);
-  if (dtype == FRNN_BF16) hipLaunchKernelGGL(alt_gemm_kernel<bf16_t>, grid, dim3(256), 0, st, a);
-  else hipLaunchKernelGGL(alt_gemm_kernel<float>, grid, dim3(256), 0, st, a);
-  return (int)hipGetLastError();
-}
-
-// ---------------------------------------------------------------------------------------------
-// pointwise kernels: one thread per (b, n, d)
-// ---------------------------------------------------------------------------------------------
 __device__ __forceinline__ float ld(const bf16_t* p) { return (float)*p; }
 __device__ __forceinline__ float ld(const float* p) { return *p; }
 __device__ __forceinline__ void st_(bf16_t* p, float v) { *reinterpret_cast<unsigned short*>(p) = f2bf(v); }
 __device__ __forceinline__ void st_(float* p, float v) { *p = v; }
 
-struct AltPwArgs {
-  const void* Wx; const void* b; const void* s0; void* states; void* cache;
-  const float* ry;  // [B][N][G_r*D]
+// ---------------------------------------------------------------------------------------------
+// One launch per time step.  A workgroup owns a 16-unit tile of one head (all its gate rows) and
+// a 16-row batch tile: its 4 waves split the contraction of the recurrent product, operands go
+// from global memory straight into MFMA fragments (both are contiguous in k), the partial sums
+// meet in LDS, and the tile's 256 elements get their gate math one per thread.  The product and
+// the gate math of a step were two launches at first; at 2-3 us per dependent launch, fusing
+// them halved the time of a sequence.
+//   MFMA result layout: lane l holds units 4*(l/16)+i (i = 0..3) of batch row l%16.
+// ---------------------------------------------------------------------------------------------
+__device__ __forceinline__ int red_index(int u, int bl) { return ((u >> 2) * 16 + bl) * 4 + (u & 3); }
+
+struct AltStepFwdArgs {
+  const void* Wx; const void* R; const void* b; const void* s0; void* states; void* cache;
   float* sfp;       // [S][B][N][D] fp32 copy of the running state: the states tensor is the
                     // storage-type output, the recurrence itself is carried unrounded (only the h
-                    // that feeds the GEMM is read back in the storage type), as in the fused path
+                    // that feeds the product is read back in the storage type), as in the fused path
   int B, T, N, D, t, training;
   float h_clip;     // > 0: new h clamped to [-h_clip, h_clip]
 };
 
 template <int F, typename T>
-__global__ void __launch_bounds__(256) alt_pw_fwd_kernel(const AltPwArgs a) {
+__global__ void __launch_bounds__(256) alt_step_fwd_kernel(const AltStepFwdArgs a) {
   typedef Cell<F> C;
-  typedef CellMath<F, ST<T>::FAST> CM;
+  typedef ST<T> X;
+  typedef typename X::Frag Frag;
+  typedef CellMath<F, X::FAST> CM;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  __shared__ __attribute__((aligned(16))) float red[4][GR][256];
+  const int d0 = blockIdx.x * 16, n = blockIdx.y, bt = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int r16 = lane & 15, q4 = lane >> 4;
   const int D = a.D, N = a.N, B = a.B, Tn = a.T, t = a.t;
-  if (idx >= (size_t)B * N * D) return;
-  const int d = idx % D, n = (idx / D) % N, b = idx / ((size_t)D * N);
-  const size_t ND = (size_t)N * D;
+  const size_t ND = (size_t)N * D, BND = (size_t)B * ND;
   const T* Wx = static_cast<const T*>(a.Wx);
+  const T* R = static_cast<const T*>(a.R);
   const T* bias = static_cast<const T*>(a.b);
   const T* s0 = static_cast<const T*>(a.s0);
   T* states = static_cast<T*>(a.states);
+
+  // thread -> unit d0 + tid % 16 of batch row bt*16 + tid / 16 for the gate math; its operands are
+  // requested before the product so that their latency hides behind it
+  const int u = tid & 15, bl = tid >> 4;
+  const int b = bt * 16 + bl, d = d0 + u;
+  const bool evalid = b < B;
+  const int be = evalid ? b : 0;
+  const size_t idx = ((size_t)be * N + n) * D + d;
   float ry[GR], wx[GW], bb[GT - GR + 1], s[S], cc[NC > 0 ? NC : 1];
 #pragma unroll
-  for (int g = 0; g < GR; ++g) ry[g] = a.ry[((size_t)b * N + n) * GR * D + (size_t)g * D + d];
+  for (int g = 0; g < GR; ++g) ry[g] = ld(bias + (size_t)(g * N + n) * D + d);
 #pragma unroll
-  for (int g = 0; g < GW; ++g) wx[g] = ld(Wx + (((size_t)b * Tn + t) * GW + g) * ND + (size_t)n * D + d);
-#pragma unroll
-  for (int g = 0; g < GR; ++g) ry[g] += ld(bias + (size_t)(g * N + n) * D + d);
+  for (int g = 0; g < GW; ++g) wx[g] = ld(Wx + (((size_t)be * Tn + t) * GW + g) * ND + (size_t)n * D + d);
 #pragma unroll
   for (int g = GR; g < GT; ++g) bb[g - GR] = ld(bias + (size_t)(g * N + n) * D + d);
-  const size_t BND = (size_t)B * ND;
 #pragma unroll
   for (int k = 0; k < S; ++k)
-    s[k] = t > 0 ? a.sfp[(size_t)k * BND + idx] : ld(s0 + ((size_t)k * B + b) * ND + (size_t)n * D + d);
+    s[k] = t > 0 ? a.sfp[(size_t)k * BND + idx] : ld(s0 + ((size_t)k * B + be) * ND + (size_t)n * D + d);
+
+  // ---- R h_{t-1} of the tile: acc[g] = rows (g, n, d0..d0+15) x batch rows bt*16..+15 ----
+  {
+    const int bm = bt * 16 + r16;
+    const bool bvalid = bm < B;
+    const T* vrow = (t > 0 ? states + (size_t)(bvalid ? bm : 0) * Tn * ND + (size_t)(t - 1) * ND
+                           : s0 + (size_t)(bvalid ? bm : 0) * ND) + (size_t)n * D;
+    const int KS = D / X::KM;
+    f32x4 acc[GR];
+#pragma unroll
+    for (int g = 0; g < GR; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // 4 k-steps of this wave per round: all their fragments are requested before the first MFMA,
+    // so a round costs one trip to L2 instead of four
+    for (int ks0 = w; ks0 < KS; ks0 += 16) {
+      Frag vf[4], af[4][GR];
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int ks = ks0 + 4 * j;
+        vf[j] = Frag{};
+#pragma unroll
+        for (int g = 0; g < GR; ++g) af[j][g] = Frag{};
+        if (ks < KS) {  // uniform over the wave
+          vf[j] = load_frag<T>(vrow, ks, q4);
+#pragma unroll
+          for (int g = 0; g < GR; ++g) af[j][g] = load_frag<T>(R + ((size_t)(g * N + n) * D + d0 + r16) * D, ks, q4);
+          if (!bvalid) vf[j] = Frag{};
+        }
+      }
+#pragma unroll
+      for (int j = 0; j < 4; ++j)
+#pragma unroll
+        for (int g = 0; g < GR; ++g) acc[g] = X::mfma(af[j][g], vf[j], acc[g]);
+    }
+#pragma unroll
+    for (int g = 0; g < GR; ++g) *reinterpret_cast<f32x4*>(&red[w][g][lane * 4]) = acc[g];
+  }
+  __syncthreads();
+  if (!evalid) return;
+  const int src = red_index(u, bl);
+#pragma unroll
+  for (int g = 0; g < GR; ++g) ry[g] += red[0][g][src] + red[1][g][src] + red[2][g][src] + red[3][g][src];
   CM::fwd(ry, wx, bb, s, cc);
   s[0] = clamp_if(s[0], a.h_clip);
 #pragma unroll
@@ -121,61 +129,111 @@ __global__ void __launch_bounds__(256) alt_pw_fwd_kernel(const AltPwArgs a) {
   }
 }
 
-struct AltPwBwdArgs {
-  const void* s0; const void* states; const void* cache; const void* dstates;
-  void* dWx; void* dgx;
-  void* dg;        // [B][N][G_r*D] storage type: operand of the next GEMM
-  float* dsr;      // [S][B][N][D] running cotangent without the recurrent term
-  const float* dh; // [B][N][D] recurrent term R^T dg of the step above
+// Reverse step t: the recurrent term R^T dg_{t+1} of the tile's 16 units (dg of the step above
+// comes from the previous launch, in the storage type, as the product's operand), then the
+// adjoint of step t for the same units, which leaves dg_t for the next launch.  t == -1: only the
+// recurrent term of step 0, added to the running cotangent to give ds0.
+struct AltStepBwdArgs {
+  const void* Rt; const void* s0; const void* states; const void* cache; const void* dstates;
+  void* dWx; void* dgx; void* ds0;
+  const void* dg_in;  // [B][N][G_r*D] of step t+1
+  void* dg_out;       // same for step t (the other of two buffers)
+  float* dsr;         // [S][B][N][D] running cotangent without the recurrent term
   int B, T, N, D, t;
-  float g_clip;    // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip]
+  int has_dg;         // 0: no recurrent term (first reverse step, or gradient_recurrent_cut)
+  float g_clip;       // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip]
 };
 
 template <int F, typename T>
-__global__ void __launch_bounds__(256) alt_pw_bwd_kernel(const AltPwBwdArgs a) {
+__global__ void __launch_bounds__(256) alt_step_bwd_kernel(const AltStepBwdArgs a) {
   typedef Cell<F> C;
-  typedef CellMath<F, ST<T>::FAST> CM;
+  typedef ST<T> X;
+  typedef typename X::Frag Frag;
+  typedef CellMath<F, X::FAST> CM;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
-  const size_t idx = (size_t)blockIdx.x * 256 + threadIdx.x;
+  __shared__ __attribute__((aligned(16))) float red[4][256];
+  const int d0 = blockIdx.x * 16, n = blockIdx.y, bt = blockIdx.z;
+  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
+  const int r16 = lane & 15, q4 = lane >> 4;
   const int D = a.D, N = a.N, B = a.B, Tn = a.T, t = a.t;
-  if (idx >= (size_t)B * N * D) return;
-  const int d = idx % D, n = (idx / D) % N, b = idx / ((size_t)D * N);
   const size_t ND = (size_t)N * D, BND = (size_t)B * ND;
+
+  // operands of the adjoint first (thread -> unit d0 + tid % 16 of batch row bt*16 + tid / 16), so
+  // that their latency hides behind the product
+  const int u = tid & 15, bl = tid >> 4;
+  const int b = bt * 16 + bl, d = d0 + u;
+  const bool evalid = b < B;
+  const int be = evalid ? b : 0;
+  const size_t idx = ((size_t)be * N + n) * D + d;
   const T* s0 = static_cast<const T*>(a.s0);
   const T* states = static_cast<const T*>(a.states);
   const T* dstates = static_cast<const T*>(a.dstates);
   float cc[NC > 0 ? NC : 1], sp[S], sn[S], dso[S], ds[S], gr[GR], gw[GW], gb[GT];
-  const T* cache = static_cast<const T*>(a.cache) + (((size_t)t * B + b) * N + n) * NC * D + d;
 #pragma unroll
-  for (int c = 0; c < NC; ++c) cc[c] = ld(cache + (size_t)c * D);
+  for (int k = 0; k < S; ++k) ds[k] = a.dsr[(size_t)k * BND + idx];
+  if (t >= 0) {  // uniform
+    const T* cache = static_cast<const T*>(a.cache) + (((size_t)t * B + be) * N + n) * NC * D + d;
 #pragma unroll
-  for (int k = 0; k < S; ++k) {
-    const size_t so = (((size_t)k * B + b) * Tn + t) * ND + (size_t)n * D + d;
-    sn[k] = ld(states + so);
-    dso[k] = ld(dstates + so);
-    sp[k] = t > 0 ? ld(states + so - ND) : ld(s0 + ((size_t)k * B + b) * ND + (size_t)n * D + d);
-    ds[k] = a.dsr[(size_t)k * BND + idx];
+    for (int c = 0; c < NC; ++c) cc[c] = ld(cache + (size_t)c * D);
+#pragma unroll
+    for (int k = 0; k < S; ++k) {
+      const size_t so = (((size_t)k * B + be) * Tn + t) * ND + (size_t)n * D + d;
+      sn[k] = ld(states + so);
+      dso[k] = ld(dstates + so);
+      sp[k] = t > 0 ? ld(states + so - ND) : ld(s0 + ((size_t)k * B + be) * ND + (size_t)n * D + d);
+    }
   }
-  ds[0] = clamp_if(ds[0] + a.dh[idx], a.g_clip);
+
+  if (a.has_dg) {  // uniform
+    const int bm = bt * 16 + r16;
+    const bool bvalid = bm < B;
+    const int K = GR * D, KS = K / X::KM;
+    const T* arow = static_cast<const T*>(a.Rt) + ((size_t)n * D + d0 + r16) * K;
+    const T* vrow = static_cast<const T*>(a.dg_in) + ((size_t)(bvalid ? bm : 0) * N + n) * K;
+    f32x4 acc = {0.f, 0.f, 0.f, 0.f};
+    f32x4 acc2 = {0.f, 0.f, 0.f, 0.f};  // two chains: a dependent MFMA waits ~3x longer than an independent one
+    for (int ks0 = w; ks0 < KS; ks0 += 32) {  // 8 k-steps of this wave per round, requested together
+      Frag vf[8], af[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {  // out-of-range k-steps load the last one and are zeroed: branch-free (measured faster here)
+        const int ks = ks0 + 4 * j, kc = ks < KS ? ks : KS - 1;
+        vf[j] = load_frag<T>(vrow, kc, q4);
+        af[j] = load_frag<T>(arow, kc, q4);
+        if (!bvalid || ks >= KS) vf[j] = Frag{};
+      }
+#pragma unroll
+      for (int j = 0; j < 8; j += 2) {
+        acc = X::mfma(af[j], vf[j], acc);
+        acc2 = X::mfma(af[j + 1], vf[j + 1], acc2);
+      }
+    }
+    acc += acc2;
+    *reinterpret_cast<f32x4*>(&red[w][lane * 4]) = acc;
+    __syncthreads();
+  }
+  if (!evalid) return;
+  float dh = 0.f;
+  if (a.has_dg) {
+    const int src = red_index(u, bl);
+    dh = red[0][src] + red[1][src] + red[2][src] + red[3][src];
+  }
+  if (t < 0) {
+    T* ds0 = static_cast<T*>(a.ds0);
+#pragma unroll
+    for (int k = 0; k < S; ++k) st_(ds0 + (size_t)k * BND + idx, ds[k] + (k == 0 ? dh : 0.f));
+    return;
+  }
+  ds[0] = clamp_if(ds[0] + dh, a.g_clip);
   CM::bwd(cc, sp, sn, dso, ds, gr, gw, gb);
 #pragma unroll
   for (int k = 0; k < S; ++k) a.dsr[(size_t)k * BND + idx] = ds[k];
-  T* dg = static_cast<T*>(a.dg) + ((size_t)b * N + n) * GR * D + d;
+  T* dg = static_cast<T*>(a.dg_out) + ((size_t)b * N + n) * GR * D + d;
 #pragma unroll
   for (int g = 0; g < GR; ++g) st_(dg + (size_t)g * D, gr[g]);
   T* dWx = static_cast<T*>(a.dWx);
 #pragma unroll
   for (int g = 0; g < GW; ++g) st_(dWx + (((size_t)b * Tn + t) * GW + g) * ND + (size_t)n * D + d, gw[g]);
   if (F == FRNN_GRU) st_(static_cast<T*>(a.dgx) + ((size_t)b * Tn + t) * ND + (size_t)n * D + d, gr[0]);
-}
-
-template <typename T>
-__global__ void __launch_bounds__(256) alt_finish_kernel(const float* dsr, const float* dh, T* ds0, int S, size_t BND) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
-  if (i >= (size_t)S * BND) return;
-  float v = dsr[i];
-  if (i < BND) v += dh[i];
-  st_(ds0 + i, v);
 }
 
 // partial bias sums: thread per bias element, rows split over blockIdx.y
@@ -203,20 +261,11 @@ __global__ void __launch_bounds__(256) alt_bias_kernel(const AltBiasArgs a) {
 // ---------------------------------------------------------------------------------------------
 template <int F, typename T>
 static int alt_forward_t(const AltProblem& p, const AltFwdBuffers& bf, hipStream_t st) {
-  constexpr int GR = Cell<F>::GR;
-  const size_t ND = (size_t)p.N * p.D;
-  const unsigned pw_blocks = (unsigned)(((size_t)p.B * ND + 255) / 256);
+  const dim3 grid(p.D / 16, p.N, (p.B + 15) / 16);
   for (int t = 0; t < p.T; ++t) {
-    AltGemmArgs g;
-    g.A = bf.R; g.a_gstride = (size_t)p.N * p.D * p.D; g.a_hstride = (size_t)p.D * p.D;
-    if (t == 0) { g.V = bf.s0; g.v_bstride = ND; }
-    else { g.V = static_cast<const T*>(bf.states) + (size_t)(t - 1) * ND; g.v_bstride = (size_t)p.T * ND; }
-    g.out = bf.ry; g.B = p.B; g.N = p.N; g.D = p.D; g.M = GR * p.D; g.K = p.D;
-    int e = launch_alt_gemm(ST<T>::ID, g, st);
-    if (e) return e;
-    AltPwArgs a{bf.Wx, bf.b, bf.s0, bf.states, bf.cache, bf.ry, bf.sfp, p.B, p.T, p.N, p.D, t, p.training, p.h_clip};
-    hipLaunchKernelGGL((alt_pw_fwd_kernel<F, T>), dim3(pw_blocks), dim3(256), 0, st, a);
-    e = (int)hipGetLastError();
+    AltStepFwdArgs a{bf.Wx, bf.R, bf.b, bf.s0, bf.states, bf.cache, bf.sfp, p.B, p.T, p.N, p.D, t, p.training, p.h_clip};
+    hipLaunchKernelGGL((alt_step_fwd_kernel<F, T>), grid, dim3(256), 0, st, a);
+    const int e = (int)hipGetLastError();
     if (e) return e;
   }
   return 0;
@@ -225,26 +274,20 @@ static int alt_forward_t(const AltProblem& p, const AltFwdBuffers& bf, hipStream
 template <int F, typename T>
 static int alt_backward_t(const AltProblem& p, const AltBwdBuffers& bf, hipStream_t st) {
   constexpr int GR = Cell<F>::GR, S = Cell<F>::S;
-  const size_t ND = (size_t)p.N * p.D, BND = (size_t)p.B * ND;
-  const unsigned pw_blocks = (unsigned)((BND + 255) / 256);
-  int e = launch_fill_zero(bf.dsr, ((size_t)S * BND + BND) * sizeof(float), st);  // dsr and dh are adjacent
+  const size_t BND = (size_t)p.B * p.N * p.D;
+  int e = launch_fill_zero(bf.dsr, (size_t)S * BND * sizeof(float), st);
   if (e) return e;
-  for (int t = p.T - 1; t >= 0; --t) {
-    AltPwBwdArgs a{bf.s0, bf.states, bf.cache, bf.dstates, bf.dWx, bf.dgx, bf.dg, bf.dsr, bf.dh, p.B, p.T, p.N, p.D, t, p.g_clip};
-    hipLaunchKernelGGL((alt_pw_bwd_kernel<F, T>), dim3(pw_blocks), dim3(256), 0, st, a);
+  const dim3 grid(p.D / 16, p.N, (p.B + 15) / 16);
+  T* dg[2] = {static_cast<T*>(bf.dg), static_cast<T*>(bf.dg) + BND * GR};
+  for (int t = p.T - 1; t >= -1; --t) {
+    AltStepBwdArgs a{bf.Rt, bf.s0, bf.states, bf.cache, bf.dstates, bf.dWx, bf.dgx, bf.ds0,
+                     dg[(t + 1) & 1], dg[t & 1], bf.dsr, p.B, p.T, p.N, p.D, t,
+                     (t < p.T - 1 && !p.cut) ? 1 : 0, p.g_clip};
+    hipLaunchKernelGGL((alt_step_bwd_kernel<F, T>), grid, dim3(256), 0, st, a);
     e = (int)hipGetLastError();
     if (e) return e;
-    if (p.cut) continue;  // truncated backpropagation: dh stays zero
-    AltGemmArgs g;
-    g.A = bf.Rt; g.a_gstride = 0; g.a_hstride = (size_t)p.D * GR * p.D;
-    g.V = bf.dg; g.v_bstride = (size_t)p.N * GR * p.D;
-    g.out = bf.dh; g.B = p.B; g.N = p.N; g.D = p.D; g.M = p.D; g.K = GR * p.D;
-    e = launch_alt_gemm(ST<T>::ID, g, st);
-    if (e) return e;
   }
-  hipLaunchKernelGGL(alt_finish_kernel<T>, dim3((unsigned)(((size_t)S * BND + 255) / 256)), dim3(256), 0, st,
-                     (const float*)bf.dsr, (const float*)bf.dh, static_cast<T*>(bf.ds0), S, BND);
-  return (int)hipGetLastError();
+  return 0;
 }
 
 #define FRNN_ALT_DISPATCH(NAME, ...)                                                     \

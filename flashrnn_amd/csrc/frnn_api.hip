@@ -471,7 +471,7 @@ size_t frnn_alt_cache_bytes(int function, int dtype, int B, int T, int N, int D)
 }
 
 namespace {
-struct AltWs { float* ry; float* sfp; void* Rt; void* dgx; void* dg; float* dsr; float* dh; float* dbp; int bsplits; float* part; int splits; size_t total; };
+struct AltWs { float* sfp; void* Rt; void* dgx; void* dg; float* dsr; float* dbp; int bsplits; float* part; int splits; size_t total; };
 AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, int backward) {
   const CellDims c = cell_dims(function);
   const size_t es = dtype_size(dtype), ND = (size_t)N * D, BND = (size_t)B * ND;
@@ -479,14 +479,12 @@ AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, i
   AltWs w;
   memset(&w, 0, sizeof(w));
   if (!backward) {
-    w.ry = (float*)bp.take(BND * c.GR * 4);
     w.sfp = (float*)bp.take(BND * c.S * 4);
   } else {
     w.Rt = bp.take(ND * c.GR * D * es);
     w.dgx = bp.take(function == FRNN_GRU ? (size_t)T * BND * es : 0);
-    w.dg = bp.take(BND * c.GR * es);
-    w.dsr = (float*)bp.take(((size_t)c.S * BND + BND) * 4);
-    w.dh = w.dsr + (size_t)c.S * BND;
+    w.dg = bp.take(2 * BND * c.GR * es);
+    w.dsr = (float*)bp.take((size_t)c.S * BND * 4);
     const long rows = (long)B * T;
     w.bsplits = rows < 64 ? (int)rows : 64;
     w.dbp = (float*)bp.take((size_t)w.bsplits * c.GT * ND * 4);
@@ -527,7 +525,7 @@ int frnn_alt_forward_opt(int function, int dtype, int training, int B, int T, in
   const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 0);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0, o.h_clip, 0.f, 0};
-  AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.ry, w.sfp};
+  AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.sfp};
   prof_begin("alt_forward_steps", (hipStream_t)stream);
   e = alt_forward(p, bf, (hipStream_t)stream);
   prof_end((hipStream_t)stream);
@@ -566,7 +564,7 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   if (e) return hip_fail(e, "R transpose");
   AltProblem p{function, dtype, B, T, N, D, 1, 0.f, o.g_clip, o.cut};
-  AltBwdBuffers bf{w.Rt, s0, states, cache, dstates, dWx, w.dgx, ds0, w.dg, w.dsr, w.dh};
+  AltBwdBuffers bf{w.Rt, s0, states, cache, dstates, dWx, w.dgx, ds0, w.dg, w.dsr};
   prof_begin("alt_backward_steps", st);
   e = alt_backward_scan(p, bf, st);
   prof_end(st);

@@ -116,15 +116,17 @@ int frnn_alt_supported(int function, int dtype, int B, int N, int D);
 size_t frnn_alt_cache_bytes(int function, int dtype, int B, int T, int N, int D);
 size_t frnn_alt_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward);
 
-/* Per time step: one MFMA GEMM kernel (R h_{t-1} for all heads) then one pointwise kernel.
+/* One kernel launch per time step: R h_{t-1} of a 16-unit x 16-row tile on MFMA, then its gate
+ * math (the reference launches a cuBLAS GEMM and a pointwise kernel per step).
  * Replaces ForwardPass::Run / IterateInternal, alternating/flashrnn_forward.cu:150-267. */
 int frnn_alt_forward(int function, int dtype, int training, int B, int T, int N, int D,
                      const void* Wx, const void* R, const void* b, const void* s0,
                      void* states, void* cache, void* workspace, size_t workspace_bytes,
                      void* stream);
 
-/* Per reverse step: pointwise adjoint kernel then MFMA GEMM (R^T dg); then dR GEMM and bias
- * reduction.  Replaces BackwardPass::Run, alternating/flashrnn_backward.cu:267-431. */
+/* One kernel launch per reverse step: R^T dg_{t+1} of a tile on MFMA, then the adjoint of step t;
+ * after the scan the dR GEMM and the bias reduction.
+ * Replaces BackwardPass::Run, alternating/flashrnn_backward.cu:267-431. */
 int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
                       const void* R, const void* b, const void* s0, const void* states,
                       const void* cache, const void* dstates,
