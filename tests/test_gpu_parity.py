@@ -62,6 +62,15 @@ def test_fused_every_batch_tiling(gpu, monkeypatch, tile_rows, function, B, T, N
     check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=13, init="randn")
 
 
+def test_fused_more_groups_than_one_launch_holds(gpu):
+    """Workgroups that wait for each other must be co-resident, so a call with more (head, batch tile)
+    groups than compute units / workgroups-per-head is split into several launches over the groups:
+    5 heads x 13 batch tiles x 4 workgroups = 260 > 256 compute units."""
+    print("case chunked launches", flush=True)
+    check_case(gpu, "lstm", 208, 3, 5, 256, "bfloat16", "hip_fused", seed=19, init="randn")
+    check_case(gpu, "elman", 130, 3, 2, 1024, "bfloat16", "hip_fused", seed=19, init="randn")  # 2 x 9 x 8 at 16 rows
+
+
 ALT_SMALL = [
     ("lstm", 4, 8, 1, 64, "float32"),
     ("lstm", 3, 5, 2, 32, "bfloat16"),
