@@ -10,7 +10,7 @@ _HERE = os.path.dirname(os.path.abspath(__file__))
 _LIB = None
 
 FUNCTION_IDS = {"lstm": 0, "slstm": 1, "gru": 2, "elman": 3}
-DTYPE_IDS = {"bfloat16": 0, "float32": 1}
+DTYPE_IDS = {"bfloat16": 0, "float32": 1, "float16": 2}
 
 # error codes of include/flashrnn_hip.h
 E_ARG, E_UNSUPPORTED, E_NULL, E_ALIGN, E_WORKSPACE, E_DEVICE = -1, -2, -3, -4, -5, -6

@@ -14,8 +14,10 @@
 namespace frnn {
 
 __device__ __forceinline__ float ld(const bf16_t* p) { return (float)*p; }
+__device__ __forceinline__ float ld(const half_t* p) { return (float)*p; }
 __device__ __forceinline__ float ld(const float* p) { return *p; }
 __device__ __forceinline__ void st_(bf16_t* p, float v) { *reinterpret_cast<unsigned short*>(p) = f2bf(v); }
+__device__ __forceinline__ void st_(half_t* p, float v) { *p = (half_t)v; }
 __device__ __forceinline__ void st_(float* p, float v) { *p = v; }
 
 // ---------------------------------------------------------------------------------------------
@@ -291,15 +293,19 @@ static int alt_backward_t(const AltProblem& p, const AltBwdBuffers& bf, hipStrea
 }
 
 #define FRNN_ALT_DISPATCH(NAME, ...)                                                     \
-  switch (p.function * 2 + p.dtype) {                                                    \
-    case FRNN_LSTM * 2 + FRNN_BF16:  return NAME<FRNN_LSTM, bf16_t>(__VA_ARGS__);        \
-    case FRNN_LSTM * 2 + FRNN_F32:   return NAME<FRNN_LSTM, float>(__VA_ARGS__);         \
-    case FRNN_SLSTM * 2 + FRNN_BF16: return NAME<FRNN_SLSTM, bf16_t>(__VA_ARGS__);       \
-    case FRNN_SLSTM * 2 + FRNN_F32:  return NAME<FRNN_SLSTM, float>(__VA_ARGS__);        \
-    case FRNN_GRU * 2 + FRNN_BF16:   return NAME<FRNN_GRU, bf16_t>(__VA_ARGS__);         \
-    case FRNN_GRU * 2 + FRNN_F32:    return NAME<FRNN_GRU, float>(__VA_ARGS__);          \
-    case FRNN_ELMAN * 2 + FRNN_BF16: return NAME<FRNN_ELMAN, bf16_t>(__VA_ARGS__);       \
-    case FRNN_ELMAN * 2 + FRNN_F32:  return NAME<FRNN_ELMAN, float>(__VA_ARGS__);        \
+  switch (p.function * 3 + p.dtype) {                                                    \
+    case FRNN_LSTM * 3 + FRNN_BF16:  return NAME<FRNN_LSTM, bf16_t>(__VA_ARGS__);        \
+    case FRNN_LSTM * 3 + FRNN_F32:   return NAME<FRNN_LSTM, float>(__VA_ARGS__);         \
+    case FRNN_LSTM * 3 + FRNN_F16:   return NAME<FRNN_LSTM, half_t>(__VA_ARGS__);        \
+    case FRNN_SLSTM * 3 + FRNN_BF16: return NAME<FRNN_SLSTM, bf16_t>(__VA_ARGS__);       \
+    case FRNN_SLSTM * 3 + FRNN_F32:  return NAME<FRNN_SLSTM, float>(__VA_ARGS__);        \
+    case FRNN_SLSTM * 3 + FRNN_F16:  return NAME<FRNN_SLSTM, half_t>(__VA_ARGS__);       \
+    case FRNN_GRU * 3 + FRNN_BF16:   return NAME<FRNN_GRU, bf16_t>(__VA_ARGS__);         \
+    case FRNN_GRU * 3 + FRNN_F32:    return NAME<FRNN_GRU, float>(__VA_ARGS__);          \
+    case FRNN_GRU * 3 + FRNN_F16:    return NAME<FRNN_GRU, half_t>(__VA_ARGS__);         \
+    case FRNN_ELMAN * 3 + FRNN_BF16: return NAME<FRNN_ELMAN, bf16_t>(__VA_ARGS__);       \
+    case FRNN_ELMAN * 3 + FRNN_F32:  return NAME<FRNN_ELMAN, float>(__VA_ARGS__);        \
+    case FRNN_ELMAN * 3 + FRNN_F16:  return NAME<FRNN_ELMAN, half_t>(__VA_ARGS__);       \
   }                                                                                      \
   return FRNN_E_ARG;
 
@@ -313,6 +319,7 @@ int launch_bias_partial(int dtype, const void* const* src, const long* ld, int G
   a.part = part; a.GT = GT; a.N = N; a.D = D; a.rows = rows; a.rows_per_split = (rows + splits - 1) / splits;
   const dim3 grid((unsigned)(((size_t)GT * N * D + 255) / 256), splits);
   if (dtype == FRNN_BF16) hipLaunchKernelGGL(alt_bias_kernel<bf16_t>, grid, dim3(256), 0, st, a);
+  else if (dtype == FRNN_F16) hipLaunchKernelGGL(alt_bias_kernel<half_t>, grid, dim3(256), 0, st, a);
   else hipLaunchKernelGGL(alt_bias_kernel<float>, grid, dim3(256), 0, st, a);
   return (int)hipGetLastError();
 }

@@ -79,13 +79,13 @@ bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out) {
   size_t n = 0;
 #define PICK(T) { tab = T; n = sizeof(T) / sizeof(Plan); }
   if (!backward) {
-    if (GR == 4) { if (dtype == FRNN_BF16) PICK(kFwd4B) else PICK(kFwd4F) }
-    else if (GR == 3) { if (dtype == FRNN_BF16) PICK(kFwd3B) else PICK(kFwd3F) }
-    else { if (dtype == FRNN_BF16) PICK(kFwd1B) else PICK(kFwd1F) }
+    if (GR == 4) { if (dtype != FRNN_F32) PICK(kFwd4B) else PICK(kFwd4F) }
+    else if (GR == 3) { if (dtype != FRNN_F32) PICK(kFwd3B) else PICK(kFwd3F) }
+    else { if (dtype != FRNN_F32) PICK(kFwd1B) else PICK(kFwd1F) }
   } else {
-    if (GR == 4) { if (dtype == FRNN_BF16) PICK(kBwd4B) else PICK(kBwd4F) }
-    else if (GR == 3) { if (dtype == FRNN_BF16) PICK(kBwd3B) else PICK(kBwd3F) }
-    else { if (dtype == FRNN_BF16) PICK(kBwd1B) else PICK(kBwd1F) }
+    if (GR == 4) { if (dtype != FRNN_F32) PICK(kBwd4B) else PICK(kBwd4F) }
+    else if (GR == 3) { if (dtype != FRNN_F32) PICK(kBwd3B) else PICK(kBwd3F) }
+    else { if (dtype != FRNN_F32) PICK(kBwd1B) else PICK(kBwd1F) }
   }
 #undef PICK
   const Plan* dflt = nullptr;
@@ -151,7 +151,7 @@ struct Bump {
 
 static int check_problem(int function, int dtype, int B, int T, int N, int D) {
   if (function < 0 || function > 3) return fail(FRNN_E_ARG, "unknown function id %d", function);
-  if (dtype != FRNN_BF16 && dtype != FRNN_F32) return fail(FRNN_E_ARG, "unknown dtype id %d", dtype);
+  if (dtype != FRNN_BF16 && dtype != FRNN_F32 && dtype != FRNN_F16) return fail(FRNN_E_ARG, "unknown dtype id %d", dtype);
   if (B <= 0 || T <= 0 || N <= 0 || D <= 0) return fail(FRNN_E_ARG, "non-positive size B=%d T=%d N=%d D=%d", B, T, N, D);
   if ((long)B * T >= (1L << 31)) return fail(FRNN_E_ARG, "B*T too large");
   return 0;
@@ -181,7 +181,7 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   w.status = (int*)bp.take(256);
   const int tr = tile_rows_for(B, N, p.kw);
   const size_t groups = (size_t)N * ((B + tr - 1) / tr);
-  const size_t llw = (size_t)16 * D / (dtype == FRNN_BF16 ? 2 : 1);
+  const size_t llw = (size_t)16 * D / (dtype == FRNN_F32 ? 1 : 2);
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
   w.zero_bytes = bp.off;  // status + exchange slots must start at zero for every call
 #ifdef FRNN_TRACE
@@ -211,10 +211,12 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
 }
 
 template <int F> static int fused_fwd_dispatch(int dtype, const Plan& p, const FwdArgs& a, hipStream_t st) {
-  return dtype == FRNN_BF16 ? fused_fwd_launch<F, FRNN_BF16>(p, a, st) : fused_fwd_launch<F, FRNN_F32>(p, a, st);
+  return dtype == FRNN_BF16 ? fused_fwd_launch<F, FRNN_BF16>(p, a, st)
+       : dtype == FRNN_F16 ? fused_fwd_launch<F, FRNN_F16>(p, a, st) : fused_fwd_launch<F, FRNN_F32>(p, a, st);
 }
 template <int F> static int fused_bwd_dispatch(int dtype, const Plan& p, const BwdArgs& a, hipStream_t st) {
-  return dtype == FRNN_BF16 ? fused_bwd_launch<F, FRNN_BF16>(p, a, st) : fused_bwd_launch<F, FRNN_F32>(p, a, st);
+  return dtype == FRNN_BF16 ? fused_bwd_launch<F, FRNN_BF16>(p, a, st)
+       : dtype == FRNN_F16 ? fused_bwd_launch<F, FRNN_F16>(p, a, st) : fused_bwd_launch<F, FRNN_F32>(p, a, st);
 }
 
 // common tail of both backward paths: dR GEMM, final reductions

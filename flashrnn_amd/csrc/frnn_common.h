@@ -11,6 +11,9 @@ namespace frnn {
 typedef __bf16 bf16_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef __bf16 bf16x4 __attribute__((ext_vector_type(4)));
+typedef _Float16 half_t;
+typedef _Float16 f16x8 __attribute__((ext_vector_type(8)));
+typedef _Float16 f16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 typedef unsigned long long u64;
 
@@ -35,7 +38,7 @@ inline CellDims cell_dims(int f) {
   }
   return {0, 0, 0, 0, 0};
 }
-inline int dtype_size(int dt) { return dt == FRNN_BF16 ? 2 : 4; }
+inline int dtype_size(int dt) { return dt == FRNN_F32 ? 4 : 2; }
 
 // ---------------------------------------------------------------------------------------
 // Storage-type traits.
@@ -43,21 +46,31 @@ inline int dtype_size(int dt) { return dt == FRNN_BF16 ? 2 : 4; }
 //  Frag : per-lane A/B operand of one MFMA
 //  EPW  : elements carried by one 64-bit tagged exchange word
 // Fragment order of a [16 rows x K] operand (row = batch for the streamed operand):
-//  bf16: element (row, k) -> ((k/32)*64 + ((k%32)/8)*16 + row)*8 + k%8
+//  bf16, f16: element (row, k) -> ((k/32)*64 + ((k%32)/8)*16 + row)*8 + k%8
 //  f32 : element (row, k) -> (k/4)*64 + (k%4)*16 + row
 // so that lane l of k-step ks reads one contiguous Frag at (ks*64 + l).
 // ---------------------------------------------------------------------------------------
 template <typename T> struct ST;
-template <> struct ST<bf16_t> {
-  static constexpr int KM = 32, EPW = 2, ID = FRNN_BF16;
+struct ST16 {  // what the two 16-bit storage types share
+  static constexpr int KM = 32, EPW = 2;
   static constexpr bool FAST = true;
-  typedef bf16x8 Frag;
   typedef uint2 Vec4;  // 4 packed elements
   static __device__ __forceinline__ int frag_elem(int row, int k) {
     return (((k >> 5) * 64 + ((k & 31) >> 3) * 16 + row) << 3) + (k & 7);
   }
+};
+template <> struct ST<bf16_t> : ST16 {
+  static constexpr int ID = FRNN_BF16;
+  typedef bf16x8 Frag;
   static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
     return __builtin_amdgcn_mfma_f32_16x16x32_bf16(a, b, c, 0, 0, 0);
+  }
+};
+template <> struct ST<half_t> : ST16 {
+  static constexpr int ID = FRNN_F16;
+  typedef f16x8 Frag;
+  static __device__ __forceinline__ f32x4 mfma(Frag a, Frag b, f32x4 c) {
+    return __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c, 0, 0, 0);
   }
 };
 template <> struct ST<float> {
@@ -94,29 +107,49 @@ typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 
-__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) {  // v_cvt_pk_bf16_f32, round to nearest even
-  const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
-  return __builtin_bit_cast(unsigned, h);
-}
-template <int E> __device__ __forceinline__ void unpack(const Dw<(E + 1) / 2>& d, float* o, bf16_t*) {
-  if constexpr (E == 1) { o[0] = __uint_as_float(d.v[0] << 16); }
+// 16-bit storage types: the two elements of a dword <-> float, round to nearest even
+template <typename T> struct H16;
+template <> struct H16<bf16_t> {
+  static __device__ __forceinline__ float lo(unsigned d) { return __uint_as_float(d << 16); }
+  static __device__ __forceinline__ float hi(unsigned d) { return __uint_as_float(d & 0xffff0000u); }
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {  // v_cvt_pk_bf16_f32
+    const bf16x2 h = __builtin_convertvector(f32x2{a, b}, bf16x2);
+    return __builtin_bit_cast(unsigned, h);
+  }
+};
+template <> struct H16<half_t> {
+  static __device__ __forceinline__ float lo(unsigned d) { return (float)__builtin_bit_cast(half_t, (unsigned short)d); }
+  static __device__ __forceinline__ float hi(unsigned d) { return (float)__builtin_bit_cast(half_t, (unsigned short)(d >> 16)); }
+  static __device__ __forceinline__ unsigned pack2(float a, float b) {  // two v_cvt_f16_f32 (the packed convert rounds toward zero)
+    const f16x2 h = {(half_t)a, (half_t)b};
+    return __builtin_bit_cast(unsigned, h);
+  }
+};
+__device__ __forceinline__ unsigned pack_bf16x2(float a, float b) { return H16<bf16_t>::pack2(a, b); }
+
+template <int E, typename T> __device__ __forceinline__ void unpack16(const Dw<(E + 1) / 2>& d, float* o) {
+  if constexpr (E == 1) { o[0] = H16<T>::lo(d.v[0]); }
   else {
 #pragma unroll
-    for (int k = 0; k < E / 2; ++k) { o[2 * k] = __uint_as_float(d.v[k] << 16); o[2 * k + 1] = __uint_as_float(d.v[k] & 0xffff0000u); }
+    for (int k = 0; k < E / 2; ++k) { o[2 * k] = H16<T>::lo(d.v[k]); o[2 * k + 1] = H16<T>::hi(d.v[k]); }
   }
 }
+template <int E, typename T> __device__ __forceinline__ Dw<(E + 1) / 2> pack16(const float* i) {
+  Dw<(E + 1) / 2> d;
+  if constexpr (E == 1) { d.v[0] = H16<T>::pack2(i[0], 0.f); }
+  else {
+#pragma unroll
+    for (int k = 0; k < E / 2; ++k) d.v[k] = H16<T>::pack2(i[2 * k], i[2 * k + 1]);
+  }
+  return d;
+}
+template <int E> __device__ __forceinline__ void unpack(const Dw<(E + 1) / 2>& d, float* o, bf16_t*) { unpack16<E, bf16_t>(d, o); }
+template <int E> __device__ __forceinline__ void unpack(const Dw<(E + 1) / 2>& d, float* o, half_t*) { unpack16<E, half_t>(d, o); }
+template <int E> __device__ __forceinline__ Dw<(E + 1) / 2> pack(const float* i, bf16_t*) { return pack16<E, bf16_t>(i); }
+template <int E> __device__ __forceinline__ Dw<(E + 1) / 2> pack(const float* i, half_t*) { return pack16<E, half_t>(i); }
 template <int E> __device__ __forceinline__ void unpack(const Dw<E>& d, float* o, float*) {
 #pragma unroll
   for (int k = 0; k < E; ++k) o[k] = __uint_as_float(d.v[k]);
-}
-template <int E> __device__ __forceinline__ Dw<(E + 1) / 2> pack(const float* i, bf16_t*) {
-  Dw<(E + 1) / 2> d;
-  if constexpr (E == 1) { d.v[0] = pack_bf16x2(i[0], 0.f); }
-  else {
-#pragma unroll
-    for (int k = 0; k < E / 2; ++k) d.v[k] = pack_bf16x2(i[2 * k], i[2 * k + 1]);
-  }
-  return d;
 }
 template <int E> __device__ __forceinline__ Dw<E> pack(const float* i, float*) {
   Dw<E> d;
@@ -158,36 +191,41 @@ template <int N, bool SUB = false> __device__ __forceinline__ void buf_store(con
 }
 
 // 4 consecutive elements <-> 4 floats (vector form, used outside the time loops)
-__device__ __forceinline__ void unpack4(uint2 v, float* o) {
-  o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
-  o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+template <typename T> __device__ __forceinline__ void unpack4(uint2 v, float* o) {
+  o[0] = H16<T>::lo(v.x); o[1] = H16<T>::hi(v.x); o[2] = H16<T>::lo(v.y); o[3] = H16<T>::hi(v.y);
 }
-__device__ __forceinline__ void unpack4(float4 v, float* o) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
+template <typename T> __device__ __forceinline__ void unpack4(float4 v, float* o) { o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w; }
 
 // ---------------------------------------------------------------------------------------
 // Tagged exchange words ("data + step tag in one store"): a reader that sees the tag of the
 // step it waits for has the data of that step; no separate flag, no fence.  32-bit stores
 // are single-copy atomic, so each tagged element is validated on its own.
-//  bf16: 64-bit word = two (tag16 << 16 | bf16) halves;  f32: (tag32 << 32 | f32 bits).
+//  bf16, f16: 64-bit word = two (tag16 << 16 | element) halves;  f32: (tag32 << 32 | f32 bits).
 // Tag of step t is never 0, so zero-filled memory never validates.
 // ---------------------------------------------------------------------------------------
 __device__ __forceinline__ unsigned tag16(int t) { return (unsigned)(t % 65535) + 1u; }
-__device__ __forceinline__ u64 ll_pack(bf16_t*, float a, float b, int t) {
-  const unsigned tg = tag16(t) << 16, ab = pack_bf16x2(a, b);
+template <typename T> __device__ __forceinline__ u64 ll_pack16(float a, float b, int t) {
+  const unsigned tg = tag16(t) << 16, ab = H16<T>::pack2(a, b);
   return (u64)(tg | (ab & 0xffffu)) | ((u64)(tg | (ab >> 16)) << 32);
 }
+__device__ __forceinline__ u64 ll_pack(bf16_t*, float a, float b, int t) { return ll_pack16<bf16_t>(a, b, t); }
+__device__ __forceinline__ u64 ll_pack(half_t*, float a, float b, int t) { return ll_pack16<half_t>(a, b, t); }
 __device__ __forceinline__ u64 ll_pack(float*, float a, int t) {
   return (u64)__float_as_uint(a) | ((u64)(unsigned)(t + 1) << 32);
 }
-__device__ __forceinline__ bool ll_ok(bf16_t*, u64 w, int t) {
+__device__ __forceinline__ bool ll_ok16(u64 w, int t) {
   unsigned tg = tag16(t);
   return ((unsigned)(w >> 16) & 0xffffu) == tg && (unsigned)(w >> 48) == tg;
 }
+__device__ __forceinline__ bool ll_ok(bf16_t*, u64 w, int t) { return ll_ok16(w, t); }
+__device__ __forceinline__ bool ll_ok(half_t*, u64 w, int t) { return ll_ok16(w, t); }
 __device__ __forceinline__ bool ll_ok(float*, u64 w, int t) { return (unsigned)(w >> 32) == (unsigned)(t + 1); }
 // payload as the 32 bits that go to LDS (bf16: two elements; f32: one)
-__device__ __forceinline__ unsigned ll_payload(bf16_t*, u64 w) {
+__device__ __forceinline__ unsigned ll_payload16(u64 w) {
   return ((unsigned)w & 0xffffu) | (((unsigned)(w >> 32) & 0xffffu) << 16);
 }
+__device__ __forceinline__ unsigned ll_payload(bf16_t*, u64 w) { return ll_payload16(w); }
+__device__ __forceinline__ unsigned ll_payload(half_t*, u64 w) { return ll_payload16(w); }
 __device__ __forceinline__ unsigned ll_payload(float*, u64 w) { return (unsigned)w; }
 
 __device__ __forceinline__ void ll_store32(unsigned* p, unsigned v) {

@@ -49,28 +49,32 @@ template <int TR> __device__ __forceinline__ void own_elems(const f32x4& acc, fl
 }
 
 // LDS writes of E consecutive elements (row, k0..k0+E-1) in fragment order; k0 % E == 0
-template <int E> __device__ __forceinline__ void lds_write(bf16_t* buf, int row, int k0, const float* v) {
-  const Dw<(E + 1) / 2> p = pack<E>(v, (bf16_t*)0);
-  unsigned* dst = reinterpret_cast<unsigned*>(buf + ST<bf16_t>::frag_elem(row, k0));
+template <int E, typename T> __device__ __forceinline__ void lds_write16(T* buf, int row, int k0, const float* v) {
+  const Dw<(E + 1) / 2> p = pack16<E, T>(v);
+  unsigned* dst = reinterpret_cast<unsigned*>(buf + ST16::frag_elem(row, k0));
   if constexpr (E == 4) *reinterpret_cast<uint2*>(dst) = make_uint2(p.v[0], p.v[1]);
   else if constexpr (E == 2) dst[0] = p.v[0];
   else *reinterpret_cast<unsigned short*>(dst) = (unsigned short)p.v[0];
 }
+template <int E> __device__ __forceinline__ void lds_write(bf16_t* buf, int row, int k0, const float* v) { lds_write16<E>(buf, row, k0, v); }
+template <int E> __device__ __forceinline__ void lds_write(half_t* buf, int row, int k0, const float* v) { lds_write16<E>(buf, row, k0, v); }
 template <int E> __device__ __forceinline__ void lds_write(float* buf, int row, int k0, const float* v) {
 #pragma unroll
   for (int i = 0; i < E; ++i) buf[ST<float>::frag_elem(row, k0 + i)] = v[i];
 }
 
 // tagged global stores of E consecutive elements (row, k0..) for step t
-template <int E> __device__ __forceinline__ void ll_write(bf16_t*, u64* slot, int row, int k0, const float* v, int t) {
+template <int E, typename T> __device__ __forceinline__ void ll_write16(u64* slot, int row, int k0, const float* v, int t) {
   if constexpr (E == 1) {  // one 32-bit tagged half of a word; the other half belongs to another lane
-    ll_store32(reinterpret_cast<unsigned*>(slot) + ST<bf16_t>::frag_elem(row, k0), (tag16(t) << 16) | (pack_bf16x2(v[0], 0.f) & 0xffffu));
+    ll_store32(reinterpret_cast<unsigned*>(slot) + ST16::frag_elem(row, k0), (tag16(t) << 16) | (H16<T>::pack2(v[0], 0.f) & 0xffffu));
   } else {
-    const int q = ST<bf16_t>::frag_elem(row, k0) >> 1;
+    const int q = ST16::frag_elem(row, k0) >> 1;
 #pragma unroll
-    for (int k = 0; k < E / 2; ++k) ll_store(slot + q + k, ll_pack((bf16_t*)0, v[2 * k], v[2 * k + 1], t));
+    for (int k = 0; k < E / 2; ++k) ll_store(slot + q + k, ll_pack16<T>(v[2 * k], v[2 * k + 1], t));
   }
 }
+template <int E> __device__ __forceinline__ void ll_write(bf16_t*, u64* slot, int row, int k0, const float* v, int t) { ll_write16<E, bf16_t>(slot, row, k0, v, t); }
+template <int E> __device__ __forceinline__ void ll_write(half_t*, u64* slot, int row, int k0, const float* v, int t) { ll_write16<E, half_t>(slot, row, k0, v, t); }
 template <int E> __device__ __forceinline__ void ll_write(float*, u64* slot, int row, int k0, const float* v, int t) {
 #pragma unroll
   for (int i = 0; i < E; ++i) ll_store(slot + ST<float>::frag_elem(row, k0 + i), ll_pack((float*)0, v[i], t));

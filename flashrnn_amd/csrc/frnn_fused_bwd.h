@@ -51,6 +51,7 @@ constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) *
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_at(const T* p);
 template <> __device__ __forceinline__ bf16x8 load_frag_at<bf16_t>(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
+template <> __device__ __forceinline__ f16x8 load_frag_at<half_t>(const half_t* p) { return *reinterpret_cast<const f16x8*>(p); }
 template <> __device__ __forceinline__ float load_frag_at<float>(const float* p) { return *p; }
 
 template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR>

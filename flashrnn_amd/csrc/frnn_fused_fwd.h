@@ -45,6 +45,9 @@ template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag(
 template <> __device__ __forceinline__ bf16x8 load_frag<bf16_t>(const bf16_t* row, int ks, int kq) {
   return *reinterpret_cast<const bf16x8*>(row + ks * 32 + kq * 8);
 }
+template <> __device__ __forceinline__ f16x8 load_frag<half_t>(const half_t* row, int ks, int kq) {
+  return *reinterpret_cast<const f16x8*>(row + ks * 32 + kq * 8);
+}
 template <> __device__ __forceinline__ float load_frag<float>(const float* row, int ks, int kq) {
   return row[ks * 4 + kq];
 }
@@ -128,7 +131,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     for (int g = 0; g < GR; ++g) {
       if constexpr (BIAS_C) {
         float v[4];
-        unpack4(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
+        unpack4<T>(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
         biasc[u][g] = f32x4{v[0], v[1], v[2], v[3]};
       } else {
 #pragma unroll
@@ -151,7 +154,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     const int row = idx / (D / 4), k0 = (idx % (D / 4)) * 4;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     const bool rv = row < TR && bt * TR + row < B;
-    if (rv) unpack4(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * TR + row) * ND + (size_t)n * D + k0), v);
+    if (rv) unpack4<T>(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * TR + row) * ND + (size_t)n * D + k0), v);
     lds_write<4>(hbuf[0], row, k0, v);
     if (KW > 1 || TR < 16) {  // rows that are never rewritten must be finite in both buffers
       if (!rv) lds_write<4>(hbuf[1], row, k0, v);

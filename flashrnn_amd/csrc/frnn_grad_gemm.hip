@@ -28,7 +28,7 @@ __global__ void __launch_bounds__(256) transpose_r_kernel(const T* __restrict__ 
 
 int launch_transpose_r(int dtype, const void* R, void* Rt, int N, int D, int GR, hipStream_t st) {
   const dim3 grid(D / 32, D / 32, GR * N);
-  if (dtype == FRNN_BF16)
+  if (dtype != FRNN_F32)
     hipLaunchKernelGGL(transpose_r_kernel<unsigned short>, grid, dim3(256), 0, st, (const unsigned short*)R, (unsigned short*)Rt, N, D, GR);
   else
     hipLaunchKernelGGL(transpose_r_kernel<float>, grid, dim3(256), 0, st, (const float*)R, (float*)Rt, N, D, GR);
@@ -41,7 +41,7 @@ int launch_transpose_r(int dtype, const void* R, void* Rt, int N, int D, int GR,
 // ---------------------------------------------------------------------------------------------
 template <typename T, int TM> struct GemmStage;
 
-template <int TM> struct GemmStage<bf16_t, TM> {
+template <int TM> struct GemmStage16 {
   // transposed: [unit][row pair], one dword = rows (2k, 2k+1) of a unit.  17 dwords per unit (16 + 1 pad):
   // an odd stride puts the 64 lanes of a transposing store on 32 different banks and keeps the fragment
   // reads (4 consecutive dwords per lane) conflict-free; an 8-element row stride would be a multiple of
@@ -50,6 +50,8 @@ template <int TM> struct GemmStage<bf16_t, TM> {
   static constexpr int LD = 17;
   unsigned a[TM][LD], b[TM][LD];
 };
+template <int TM> struct GemmStage<bf16_t, TM> : GemmStage16<TM> {};
+template <int TM> struct GemmStage<half_t, TM> : GemmStage16<TM> {};
 template <int TM> struct GemmStage<float, TM> {
   static constexpr int LD = TM + 4;
   float a[32][LD], b[32][LD];    // as stored: [row][unit]
@@ -121,14 +123,14 @@ __global__ void __launch_bounds__(256) grad_gemm_kernel(const GradGemmArgs a) {
       }
       __syncthreads();
       if (r0 + 32 < r_end) fetch(r0 + 32);
-      bf16x8 af[WT], bfr[WT];
+      typename X::Frag af[WT], bfr[WT];
 #pragma unroll
       for (int i = 0; i < WT; ++i) {
         const unsigned* pa = &sm.a[wm * (TM / 2) + i * 16 + r16][q4 * 4];
         const unsigned* pb = &sm.b[wn * (TM / 2) + i * 16 + r16][q4 * 4];
         const u32x4 va = {pa[0], pa[1], pa[2], pa[3]}, vb = {pb[0], pb[1], pb[2], pb[3]};
-        af[i] = __builtin_bit_cast(bf16x8, va);
-        bfr[i] = __builtin_bit_cast(bf16x8, vb);
+        af[i] = __builtin_bit_cast(typename X::Frag, va);
+        bfr[i] = __builtin_bit_cast(typename X::Frag, vb);
       }
 #pragma unroll
       for (int i = 0; i < WT; ++i)
@@ -205,6 +207,9 @@ int launch_grad_gemm(int dtype, GradGemmArgs a, int splits, hipStream_t st) {
   if (dtype == FRNN_BF16) {
     if (TM == 64) hipLaunchKernelGGL((grad_gemm_kernel<bf16_t, 64>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((grad_gemm_kernel<bf16_t, 32>), grid, dim3(256), 0, st, a);
+  } else if (dtype == FRNN_F16) {
+    if (TM == 64) hipLaunchKernelGGL((grad_gemm_kernel<half_t, 64>), grid, dim3(256), 0, st, a);
+    else hipLaunchKernelGGL((grad_gemm_kernel<half_t, 32>), grid, dim3(256), 0, st, a);
   } else {
     if (TM == 64) hipLaunchKernelGGL((grad_gemm_kernel<float, 64>), grid, dim3(256), 0, st, a);
     else hipLaunchKernelGGL((grad_gemm_kernel<float, 32>), grid, dim3(256), 0, st, a);

@@ -22,11 +22,13 @@ bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out);
 #if defined(FRNN_F) && defined(FRNN_DT)
 #if FRNN_DT == 0
 #define FRNN_TU_T frnn::bf16_t
+#elif FRNN_DT == 2
+#define FRNN_TU_T frnn::half_t
 #else
 #define FRNN_TU_T float
 #endif
 #if FRNN_F == 0 || FRNN_F == 1
-#if FRNN_DT == 0
+#if FRNN_DT != 1
 #define FRNN_TU_PLANS FRNN_PLANS_GR4_BF16
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16
 #else
@@ -34,7 +36,7 @@ bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out);
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_F32
 #endif
 #elif FRNN_F == 2
-#if FRNN_DT == 0
+#if FRNN_DT != 1
 #define FRNN_TU_PLANS FRNN_PLANS_GR3_BF16
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR3_BF16
 #else
@@ -42,7 +44,7 @@ bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out);
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR3_F32
 #endif
 #else
-#if FRNN_DT == 0
+#if FRNN_DT != 1
 #define FRNN_TU_PLANS FRNN_PLANS_GR1_BF16
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR1_BF16
 #else

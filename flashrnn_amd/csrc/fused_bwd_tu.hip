@@ -1,5 +1,5 @@
 // One translation unit per (function, storage type): instantiates the fused backward kernel for
-// every tiling in the plan table.  Build with -DFRNN_F=<0..3> -DFRNN_DT=<0|1>.
+// every tiling in the plan table.  Build with -DFRNN_F=<0..3> -DFRNN_DT=<0|1|2>.
 #include "frnn_fused_bwd.h"
 #include "frnn_launch.h"
 

@@ -28,7 +28,7 @@ rnn_function_registry = {
     "elman": {"gates_states": (1, 1, 1, 1, 1), "constants": {}, "simple_agg": True},
 }
 
-DTYPE_DICT = {"bfloat16": torch.bfloat16, "float32": torch.float32}
+DTYPE_DICT = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}
 BACKENDS = ("hip_fused", "hip")
 
 
@@ -66,7 +66,7 @@ class FlashRNNConfig:
                 f"Unknown backend {self.backend}: this package provides {BACKENDS}; the pure-PyTorch "
                 "'vanilla' loop is the test oracle and is not part of the package")
         if self.dtype not in DTYPE_DICT:
-            raise ValueError(f"dtype {self.dtype} not supported (bfloat16, float32)")
+            raise ValueError(f"dtype {self.dtype} not supported (bfloat16, float16, float32)")
         for name in ("gradient_recurrent_clipval", "forward_clipval"):
             v = getattr(self, name)
             if v is not None and not v > 0:

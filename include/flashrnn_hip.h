@@ -22,7 +22,9 @@
  *  - dR and db are returned in fp32 whatever the storage type (reference: storage type).
  *
  * All pointers are device pointers, 16-byte aligned, tensors contiguous.  Element type is
- * bf16 (FRNN_BF16) or fp32 (FRNN_F32) for Wx, R, b, s0, states, dstates, dWx, ds0.
+ * bf16 (FRNN_BF16), fp16 (FRNN_F16) or fp32 (FRNN_F32) for Wx, R, b, s0, states, dstates, dWx,
+ * ds0.  Whatever the storage type, MFMA accumulation and all gate math are fp32 (the reference
+ * accumulates fp16 in fp16 and computes the gates in the storage type).
  *
  * Return value: 0 ok; negative = argument error found on the host before any launch
  * (FRNN_E_*; text in frnn_last_error()); positive = hipError_t of a failed launch.
@@ -38,7 +40,7 @@ extern "C" {
 
 /* function ids: gate/state counts as in flashrnn.py:49-71 */
 enum { FRNN_LSTM = 0, FRNN_SLSTM = 1, FRNN_GRU = 2, FRNN_ELMAN = 3 };
-enum { FRNN_BF16 = 0, FRNN_F32 = 1 };
+enum { FRNN_BF16 = 0, FRNN_F32 = 1, FRNN_F16 = 2 };  /* DTYPE_DICT, flashrnn.py:73-78 */
 
 enum {
   FRNN_OK = 0,

@@ -17,6 +17,8 @@ of the oracle fed the same bf16-rounded inputs):
                             rounding error of 2^-9, so the error of the sum grows like sqrt(B*T)
                             (measured 0.17 on |dR| <= 56 at B*T = 8192); the kernel accumulates and
                             returns them in fp32.
+  fp16   as bf16 with every bound divided by 4 (3 more mantissa bits; the reference states no
+         fp16 tolerance).
 """
 import torch
 
@@ -25,7 +27,7 @@ from oracle.flashrnn_oracle import flashrnn_oracle_fwbw_manual
 
 
 def oracle_run(function, inp, dtype, backward=True, options=None):
-    odt = torch.float32 if dtype == "bfloat16" else torch.float64
+    odt = torch.float64 if dtype == "float32" else torch.float32
     options = dict(options or {})
     kw = {"slstm_per_element_first_step": True} if function == "slstm" else {}
     args = [inp[k].to(odt) for k in ("Wx", "R", "b", "states")]
@@ -65,27 +67,30 @@ def assert_close(name, got, ref, dtype, kind):
     got, ref = got.double(), ref.double()
     err = (got - ref).abs()
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
+    # float16 carries 3 more mantissa bits than bfloat16: its tolerances are the bf16 ones / 4
+    q = 0.25 if dtype == "float16" else 1.0
     if dtype == "float32":
         tol = 1e-5 * max(1.0, float(ref.abs().max()))
         assert float(err.max()) <= tol, f"{name}: max err {float(err.max()):.3e} > {tol:.3e}"
     elif kind == "h":
-        assert float(err.max()) <= 2e-2, f"{name}: max abs err {float(err.max()):.4f} > 2e-2"
+        assert float(err.max()) <= 2e-2 * q, f"{name}: max abs err {float(err.max()):.3e} > {2e-2 * q:.1e}"
     elif kind == "state":
-        bad = err > 2e-2 * torch.clamp(ref.abs(), min=1.0)
-        assert not bool(bad.any()), f"{name}: {int(bad.sum())} elements beyond 2e-2*max(1,|ref|); max err {float(err.max()):.4f}"
+        bad = err > 2e-2 * q * torch.clamp(ref.abs(), min=1.0)
+        assert not bool(bad.any()), f"{name}: max err {float(err.max()):.3e} (|ref| there {float(ref.abs()[err.argmax()]) if err.dim()==1 else float(ref.abs().flatten()[err.argmax()]):.2f})"
     elif kind == "token":
-        bad = err > torch.clamp(2e-2 * torch.clamp(ref.abs(), min=1.0), min=5e-3 * float(ref.abs().max()))
-        assert not bool(bad.any()), f"{name}: {int(bad.sum())} elements beyond tolerance; max err {float(err.max()):.4f}"
-    else:  # "sum": accumulated over B*T
-        tol = max(2e-2, 1e-2 * float(ref.abs().max()))
-        assert float(err.max()) <= tol, f"{name}: max err {float(err.max()):.4f} > {tol:.4f}"
+        tol = torch.clamp(2e-2 * q * torch.clamp(ref.abs(), min=1.0), min=5e-3 * q * float(ref.abs().max()))
+        bad = err > tol
+        assert not bool(bad.any()), f"{name}: max err {float(err.max()):.3e}, max ref {float(ref.abs().max()):.2f}"
+    else:  # sums over B*T tokens
+        tol = max(2e-2 * q, 1e-2 * q * float(ref.abs().max()))
+        assert float(err.max()) <= tol, f"{name}: max err {float(err.max()):.3e} > {tol:.3e}"
 
 
 def check_case(device, function, B, T, N, D, dtype, backend, seed=1, init="randn", backward=True,
                forget_bias_linspace=False, options=None):
     grad_on = "h" if function == "slstm" else "all"
     inp = make_inputs(function, B, T, N, D, seed, init=init,
-                      round_to=torch.bfloat16 if dtype == "bfloat16" else None, grad_on=grad_on,
+                      round_to={"bfloat16": torch.bfloat16, "float16": torch.float16}.get(dtype), grad_on=grad_on,
                       forget_bias_linspace=forget_bias_linspace)
     ref_out, ref_g = oracle_run(function, inp, dtype, backward, options)
     out, grads = hip_run(function, inp, dtype, backend, device, backward, options)

@@ -130,7 +130,8 @@ def test_python_api_argument_errors():
     with pytest.raises(ValueError):
         FlashRNNConfig(function="rnn")
     with pytest.raises(ValueError):
-        FlashRNNConfig(dtype="float16")
+        FlashRNNConfig(dtype="float64")
+    assert FlashRNNConfig(dtype="float16").dtype == "float16"
     with pytest.raises(ValueError):
         FlashRNNConfig(gradient_recurrent_clipval=-1.0)
     assert FlashRNNConfig(gradient_recurrent_cut=True, forward_clipval=2.0).gradient_recurrent_cut

@@ -71,6 +71,27 @@ def test_fused_more_groups_than_one_launch_holds(gpu):
     check_case(gpu, "elman", 130, 3, 2, 1024, "bfloat16", "hip_fused", seed=19, init="randn")  # 2 x 9 x 8 at 16 rows
 
 
+HALF = [
+    # function, B, T, N, D, backend
+    ("lstm", 8, 16, 3, 256, "hip_fused"),      # 4 workgroups per head
+    ("lstm", 20, 6, 2, 128, "hip_fused"),
+    ("gru", 7, 9, 2, 192, "hip_fused"),
+    ("slstm", 5, 8, 2, 64, "hip_fused"),
+    ("elman", 18, 6, 1, 1024, "hip_fused"),
+    ("lstm", 6, 5, 2, 96, "hip"),
+    ("gru", 17, 4, 1, 64, "hip"),
+    ("slstm", 4, 6, 1, 192, "hip"),
+    ("elman", 9, 7, 2, 320, "hip"),
+]
+
+
+@pytest.mark.parametrize("function,B,T,N,D,backend", HALF)
+def test_float16_matches_oracle(gpu, function, B, T, N, D, backend):
+    """fp16 storage, fp32 accumulation and gate math (the reference's third dtype, flashrnn.py:73-78)."""
+    print(f"case fp16 {backend} {function} B{B} T{T} N{N} D{D}", flush=True)
+    check_case(gpu, function, B, T, N, D, "float16", backend, seed=23, init="randn")
+
+
 ALT_SMALL = [
     ("lstm", 4, 8, 1, 64, "float32"),
     ("lstm", 3, 5, 2, 32, "bfloat16"),
