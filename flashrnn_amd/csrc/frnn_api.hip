@@ -201,6 +201,9 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   const size_t bt = (B + tr - 1) / tr, groups = (size_t)N * bt;
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * bwd_inbox_words(D, p.kw) * 8 : 0);
   w.zero_bytes = bp.off;
+#ifdef FRNN_TRACE
+  bp.take(1 << 20);
+#endif
   w.Rt = bp.take((size_t)N * D * c.GR * D * es);
   w.dgx = bp.take(function == FRNN_GRU ? (size_t)B * T * N * D * es : 0);
   w.dbp = (float*)bp.take(bt * c.GT * N * D * 4);
@@ -444,6 +447,10 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", 4);  // ~0.12 us: measured best on MI355X
   a.g_clip = o.g_clip; a.cut = o.cut;
+  a.trace = nullptr;
+#ifdef FRNN_TRACE
+  a.trace = (long long*)((char*)workspace + w.zero_bytes);
+#endif
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
     prof_begin("fused_bwd_kernel", st);

@@ -160,14 +160,26 @@ __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, 
   return fail;
 }
 
+// Workgroup barrier that orders LDS accesses only.  __syncthreads() also waits for every global
+// load and store the wave has in flight (s_waitcnt vmcnt(0)): inside the time loops that exposed
+// the full HBM latency of the operand prefetch once per step (measured: ~1000 of 2200 cycles per
+// reverse step at D = 64).  The steps exchange data between waves through LDS only (and between
+// workgroups through the tagged words, which carry their own validity), so LDS order is all the
+// barrier has to provide and the prefetches keep flying across it.
+__device__ __forceinline__ void lds_barrier() { asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory"); }
+
 // Workgroup barrier that also tells every wave whether any lane passed `fail`; `flag` is one LDS
 // word that starts at 0 and is only ever set.  Costs one LDS read more than a plain barrier.
 // The result is read back through readfirstlane so that the compiler knows it is wave-uniform
 // and keeps the time-step counter (and every address derived from it) in scalar registers.
-__device__ __forceinline__ bool barrier_or(bool fail, volatile int* flag) {
-  if (fail) *flag = 1;
-  __syncthreads();
-  return __builtin_amdgcn_readfirstlane(*flag) != 0;
+__device__ __forceinline__ bool barrier_or(bool fail, int* flag) {
+  // an explicit LDS pointer: through a generic (or volatile) pointer the compiler emits a flat load,
+  // which counts as a global access and drains every global load in flight before it returns
+  typedef __attribute__((address_space(3))) int lds_int;
+  lds_int* const f = (lds_int*)flag;
+  if (fail) *f = 1;
+  lds_barrier();  // also a compiler barrier: the read below is a fresh one
+  return __builtin_amdgcn_readfirstlane(*f) != 0;
 }
 
 }  // namespace frnn

@@ -31,6 +31,14 @@
 
 namespace frnn {
 
+#ifndef FRNN_STAMP
+#ifdef FRNN_TRACE
+#define FRNN_STAMP(var) __builtin_amdgcn_sched_barrier(0); const long long var = clock64(); __builtin_amdgcn_sched_barrier(0)
+#else
+#define FRNN_STAMP(var)
+#endif
+#endif
+
 struct BwdArgs {
   const void* Rt;  // [N][D (previous unit p)][G_r*D (k = g*D + d)]
   const void* s0; const void* states; const void* cache; const void* dstates;
@@ -44,6 +52,7 @@ struct BwdArgs {
   int spin_limit, poll_delay;
   float g_clip;  // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip] (gradient_recurrent_clipval)
   int cut;       // != 0: no gradient through R h (gradient_recurrent_cut)
+  long long* trace;  // phase cycle sums per wave; only written by -DFRNN_TRACE builds
 };
 
 // 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][element 4][lane 64]
@@ -79,7 +88,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);
   T* const gbuf1 = gbuf0 + 16 * KDL;
-  int* const dead_flag = reinterpret_cast<int*>(gbuf1 + 16 * KDL);
+  // a static LDS word, not a slice of the dynamic array: through a pointer computed from the
+  // dynamic array the compiler reads the flag with a flat load, which has to wait for every global
+  // load in flight (measured: the operand prefetch's full HBM latency, once per step)
+  __shared__ int dead_flag_word;
+  int* const dead_flag = &dead_flag_word;
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -132,7 +145,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   }
 
   // zero both LDS buffers once (rows beyond the tile are never written) and the flag
-  for (int idx = tid; idx < (2 * 16 * KDL * (int)sizeof(T)) / 4 + 1; idx += NT) reinterpret_cast<unsigned*>(smem_raw)[idx] = 0u;
+  for (int idx = tid; idx < (2 * 16 * KDL * (int)sizeof(T)) / 4; idx += NT) reinterpret_cast<unsigned*>(smem_raw)[idx] = 0u;
+  if (tid == 0) dead_flag_word = 0;
 
   float ds[UTW][E][S];
   float dbacc[UTW][E][GT];
@@ -171,6 +185,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   load_pre(pa, Tn - 1);
   __syncthreads();
 
+#ifdef FRNN_TRACE
+  long long tr[4] = {0, 0, 0, 0};
+  const long long tr_begin = clock64();
+#endif
   bool dead = false, fail = false;
   // one reverse step: consumes `pc` (operands of step t), prefetches those of step t-1 into `pn`.
   // CUT (a std::bool_constant): truncated backpropagation, the step ends with the pointwise carry;
@@ -179,6 +197,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   auto step = [&](auto CUT, const int t, Pre& pc, Pre& pn) __attribute__((always_inline)) {
     constexpr bool cut = decltype(CUT)::value;
     T* const gb = (t & 1) ? gbuf1 : gbuf0;
+    FRNN_STAMP(c0);
     load_pre(pn, max(t - 1, 0));
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
@@ -219,8 +238,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
     }
     if constexpr (cut) return;
+    FRNN_STAMP(c1);
     // the barrier also spreads a failed wait of the previous step to the whole workgroup
     if (barrier_or(fail, dead_flag)) { dead = true; return; }
+    FRNN_STAMP(c2);
 
     // one accumulator per tile: splitting a lone chain over several accumulators (as the forward
     // kernel does) measured 5-8 % slower here
@@ -269,6 +290,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
     }
 
+#ifdef FRNN_TRACE
+    { float sink = 0.f;
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) sink += ds[u][0][0];
+      asm volatile("" ::"v"(sink)); }
+#endif
+    FRNN_STAMP(c3);
     if constexpr (KW > 1) {
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
       u64* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
@@ -312,6 +340,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
           }
       }
     }
+#ifdef FRNN_TRACE
+    FRNN_STAMP(c4);
+    tr[0] += c1 - c0; tr[1] += c2 - c1; tr[2] += c3 - c2; tr[3] += c4 - c3;
+#endif
   };
 
   int t = Tn - 1;
@@ -330,6 +362,12 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     if (!dead && t == 0) step(std::false_type{}, 0, pa, pb);
   }
   if (!dead && barrier_or(fail, dead_flag)) dead = true;
+#ifdef FRNN_TRACE
+  if (lane == 0 && a.trace) {
+    long long* o = a.trace + ((size_t)blockIdx.x * WAVES + w) * 8;
+    o[0] = tr[0]; o[1] = tr[1]; o[2] = tr[2]; o[3] = tr[3]; o[4] = clock64() - tr_begin;
+  }
+#endif
 
   if (dead) {
     if (tid == 0) __hip_atomic_store(a.status, (int)STATUS_WAIT_EXPIRED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);

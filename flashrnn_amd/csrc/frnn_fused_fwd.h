@@ -190,7 +190,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         const bool fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
         if (barrier_or(fail, &dead_flag)) { dead = true; return; }
       } else {
-        __syncthreads();
+        lds_barrier();
       }
     }
     FRNN_STAMP(c1);
