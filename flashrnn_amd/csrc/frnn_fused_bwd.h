@@ -79,7 +79,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   static_assert(KDL % X::KM == 0 && DL % 8 == 0, "own gate rows must fill whole k-steps");
   constexpr int KE = X::KM / 4;         // consecutive k held by one lane of a fragment
   constexpr int NCA = NC > 0 ? NC : 1;
-  constexpr int RC = KW == 1 ? 1 : ((KW - 1) < 3 ? (KW - 1) : 3);  // remote sources polled together
+  // remote sources polled together: every round of polling costs at least one trip to L2 and back,
+  // so as few rounds as 16 words per lane and probe allow, of equal size (no dummy loads)
+  constexpr int RC_MAX = 16 / (UTW * (TR / 4)) > 0 ? 16 / (UTW * (TR / 4)) : 1;
+  constexpr int ROUNDS = KW == 1 ? 1 : (KW - 1 + RC_MAX - 1) / RC_MAX;
+  constexpr int RC = KW == 1 ? 1 : (KW - 1 + ROUNDS - 1) / ROUNDS;
   constexpr size_t INW = bwd_inbox_words(D, KW);
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
   constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
@@ -244,7 +248,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     FRNN_STAMP(c2);
 
     // one accumulator per tile: splitting a lone chain over several accumulators (as the forward
-    // kernel does) measured 5-8 % slower here
+    // kernel does) measured 3-8 % slower here, before and after the barrier was made LDS-only
     constexpr int NACC = 1;
     f32x4 accp[NACC][KW][UTW];
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;

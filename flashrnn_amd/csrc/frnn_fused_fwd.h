@@ -64,7 +64,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
   constexpr int LLW = 16 * D / X::EPW;  // 64-bit words per exchange slot
-  constexpr int NP = (LLW + NT - 1) / NT;
+  constexpr int NP = (LLW * TR / 16 + NT - 1) / NT;  // words a thread polls per step: only the TR rows of the tile
   constexpr int NCA = NC > 0 ? NC : 1;
   constexpr int GX = GT - GR > 0 ? GT - GR : 1;
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
