@@ -370,7 +370,7 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
-  a.poll_delay = env_int("FRNN_POLL_DELAY", 0);
+  a.poll_delay = env_int("FRNN_POLL_DELAY", 4);  // s_sleep units before the first probe of a step (measured best: 4)
   a.h_clip = o.h_clip;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

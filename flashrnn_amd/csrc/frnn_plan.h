@@ -40,7 +40,7 @@ struct Plan { int D, variant, waves, utw, kw; };
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
-  X(256, 0, 16, 1, 1) X(256, 1, 4, 4, 1) X(512, 0, 8, 1, 4) X(512, 1, 4, 2, 4) X(512, 2, 16, 1, 2) \
+  X(256, 0, 16, 1, 1) X(256, 1, 4, 4, 1) X(512, 0, 4, 2, 4) X(512, 1, 8, 1, 4) X(512, 2, 16, 1, 2) \
   X(1024, 0, 8, 1, 8) X(1024, 1, 4, 1, 16)
 #define FRNN_BWD_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
