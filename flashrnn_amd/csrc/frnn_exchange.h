@@ -102,41 +102,58 @@ __device__ __forceinline__ void ll_plan(int tid, int rows_valid, int kdim, int* 
 
 // Poll NW tagged words (addresses base + off[i]; every lane polls NW words, lanes or entries
 // with nothing to wait for pass need[i] = false and may point anywhere valid) until all carry the
-// tag of step t.  PD probes of the whole set are kept in flight, so a word that becomes visible is
-// seen within 1/PD of a memory round trip; loads are unconditional and the exit test is a wave
-// vote, so the waits between probes are exact counts, not drains.  Returns true if the bounded
-// wait ran out (or another workgroup already reported that).
+// tag of step t.  Loads are unconditional and the exit test is a wave vote.  Returns true if the
+// bounded wait ran out (or another workgroup already reported that).
 template <typename TAG, int NW, int PD>
 __device__ __forceinline__ bool poll_words(const u64* base, const int* off, const bool* need, int t, u64* out,
                                            int* status, int spin_limit, int first_delay) {
+  static_assert(PD == 1, "one probe of the set in flight: more only add congestion (measured again with exact waits)");
   // the producers finish their step at about the same time as this wave: a probe sent at once
   // reaches memory before their stores and costs a whole extra round trip
   for (int i = 0; i < first_delay; ++i) __builtin_amdgcn_s_sleep(1);
-  u64 v[PD][NW];
-#pragma unroll
-  for (int p = 0; p < PD; ++p)
-#pragma unroll
-    for (int i = 0; i < NW; ++i) v[p][i] = ll_load(base + off[i]);
   for (int spins = 0;; ++spins) {
 #pragma unroll
-    for (int p = 0; p < PD; ++p) {
-      bool ok = true;
+    for (int i = 0; i < NW; ++i) out[i] = ll_load(base + off[i]);
+    // straight-line test of the whole set (bitwise, no short circuit: a short-circuit && turns into
+    // a chain of divergent branches with a wait inside each)
+    bool ok = true;
 #pragma unroll
-      for (int i = 0; i < NW; ++i) ok = ok && (!need[i] || ll_ok((TAG*)0, v[p][i], t));
-      if (__all(ok)) {
-#pragma unroll
-        for (int i = 0; i < NW; ++i) out[i] = v[p][i];
-        return false;
-      }
-#pragma unroll
-      for (int i = 0; i < NW; ++i) v[p][i] = ll_load(base + off[i]);
-    }
+    for (int i = 0; i < NW; ++i) ok = ok & (!need[i] | ll_ok((TAG*)0, out[i], t));
+    if (__all(ok)) return false;
     if (spins > spin_limit) return true;
     if ((spins & 63) == 63 &&
         __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
   }
 }
-constexpr int probe_depth(int) { return 1; }  // more probes in flight only add congestion (measured)
+
+// The same wait with a short-circuit test: the words are examined in the order their loads return
+// and the first missing one sends the next probe at once, while the tail of the last one is still
+// in flight.  Measured 3 % faster than the straight-line form for the 3-word sets of the backward
+// exchange (and 4 % slower for the 2-word sets of the forward one).
+template <typename TAG, int NW>
+__device__ __forceinline__ bool poll_words_staggered(const u64* base, const int* off, const bool* need, int t, u64* out,
+                                                     int* status, int spin_limit, int first_delay) {
+  for (int i = 0; i < first_delay; ++i) __builtin_amdgcn_s_sleep(1);
+  u64 v[NW];
+#pragma unroll
+  for (int i = 0; i < NW; ++i) v[i] = ll_load(base + off[i]);
+  for (int spins = 0;; ++spins) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) ok = ok && (!need[i] || ll_ok((TAG*)0, v[i], t));
+    if (__all(ok)) {
+#pragma unroll
+      for (int i = 0; i < NW; ++i) out[i] = v[i];
+      return false;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) v[i] = ll_load(base + off[i]);
+    if (spins > spin_limit) return true;
+    if ((spins & 63) == 63 &&
+        __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
+  }
+}
+constexpr int probe_depth(int) { return 1; }
 
 // Forward gather: poll the planned words of slot, then copy their payloads to LDS.
 template <typename T, int NP>

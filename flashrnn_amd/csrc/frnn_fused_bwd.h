@@ -25,9 +25,6 @@
 #include "frnn_fused_fwd.h"
 #include "frnn_pointwise.h"
 
-#ifndef FRNN_BWD_PD
-#define FRNN_BWD_PD 1
-#endif
 
 namespace frnn {
 
@@ -333,7 +330,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
               need[(rr * UTW + u) * E + e] = bvalid && (r0 + rr < KW);
             }
         }
-        if (!fail) fail = poll_words<float, NWR, FRNN_BWD_PD>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
+        if (!fail) fail = poll_words_staggered<float, NWR>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
 #pragma unroll
         for (int rr = 0; rr < RC; ++rr)
           if (r0 + rr < KW) {
