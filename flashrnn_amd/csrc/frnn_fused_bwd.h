@@ -199,7 +199,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     constexpr bool cut = decltype(CUT)::value;
     T* const gb = (t & 1) ? gbuf1 : gbuf0;
     FRNN_STAMP(c0);
-    load_pre(pn, max(t - 1, 0));
+    // (readfirstlane: the compiler otherwise forms max(t - 1, 0) with a saturating VALU subtract and
+    // then wraps a buffer load that uses it as a scalar offset into a waterfall loop)
+    load_pre(pn, __builtin_amdgcn_readfirstlane(t > 0 ? t - 1 : 0));
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
