@@ -10,12 +10,13 @@
 // alternate by step parity: a workgroup can only write step t+2 after it has read all of step
 // t+1, which every workgroup wrote only after reading step t, so slot (t & 1) is never
 // overwritten while still in use.  Accesses are agent scope: workgroup-scope loads are served
-// from the per-CU L1 and never see another compute unit's store (measured), and agent scope
-// costs the same ~0.45 us per hop whether or not the two workgroups share an XCD.
+// from the per-CU L1 and never see another compute unit's store (measured).  One all-to-all step
+// between 4 workgroups costs ~1700 cycles when they share an XCD and ~2300 when they do not
+// (measured), which is why the launch maps the workgroups of a head to one XCD.
 //
 // Ownership.  The 16x16 MFMA result gives lane l the 4 rows 4*(l/16)..+3 of column l%16, i.e.
 // (with A = weight rows, B = streamed vector) 4 consecutive units of batch row l%16.
-//   FULL: a lane keeps its 4 elements.
+//   16-row tiles: a lane keeps its 4 elements.
 //   8-row tiles: columns 8..15 are padding, so lanes 8..15 of every 16-lane row take elements
 //   2,3 of the lane 8 below them (one DPP move each) and every lane does the gate math of 2
 //   elements instead of 4.
