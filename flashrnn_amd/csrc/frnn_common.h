@@ -228,6 +228,29 @@ __device__ __forceinline__ unsigned ll_payload(bf16_t*, u64 w) { return ll_paylo
 __device__ __forceinline__ unsigned ll_payload(half_t*, u64 w) { return ll_payload16(w); }
 __device__ __forceinline__ unsigned ll_payload(float*, u64 w) { return (unsigned)w; }
 
+// Partial sums of the backward exchange.  fp32 storage: (tag32 << 32 | f32 bits) as above.  16-bit
+// storage: one 32-bit word (tag8 << 24 | the sum rounded to sign, 8 exponent and 15 mantissa bits):
+// the operands of the sum carry 8 or 11 mantissa bits, and the exchange costs by the byte (measured:
+// -18 % per step against 8-byte words).  Tag of step t is never 0 and differs from that of step
+// t +- 2, the only older content a slot can hold.
+struct Part64 { typedef u64 Word; };
+struct Part32 { typedef unsigned Word; };
+__device__ __forceinline__ u64 part_pack(Part64*, float a, int t) { return (u64)__float_as_uint(a) | ((u64)(unsigned)(t + 1) << 32); }
+__device__ __forceinline__ bool ll_ok(Part64*, u64 w, int t) { return (unsigned)(w >> 32) == (unsigned)(t + 1); }
+__device__ __forceinline__ float part_value(Part64*, u64 w) { return __uint_as_float((unsigned)w); }
+__device__ __forceinline__ unsigned tag8(int t) { return (unsigned)(t % 255) + 1u; }
+__device__ __forceinline__ unsigned part_pack(Part32*, float a, int t) {
+  return (tag8(t) << 24) | ((__float_as_uint(a) + 0x80u) >> 8);
+}
+__device__ __forceinline__ bool ll_ok(Part32*, unsigned w, int t) { return (w >> 24) == tag8(t); }
+__device__ __forceinline__ float part_value(Part32*, unsigned w) { return __uint_as_float(w << 8); }
+__device__ __forceinline__ unsigned ll_load(const unsigned* p) {
+  return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void ll_store(unsigned* p, unsigned v) {
+  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+
 __device__ __forceinline__ void ll_store32(unsigned* p, unsigned v) {
   __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }

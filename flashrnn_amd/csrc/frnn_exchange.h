@@ -131,11 +131,11 @@ __device__ __forceinline__ bool poll_words(const u64* base, const int* off, cons
 // and the first missing one sends the next probe at once, while the tail of the last one is still
 // in flight.  Measured 3 % faster than the straight-line form for the 3-word sets of the backward
 // exchange (and 4 % slower for the 2-word sets of the forward one).
-template <typename TAG, int NW>
-__device__ __forceinline__ bool poll_words_staggered(const u64* base, const int* off, const bool* need, int t, u64* out,
+template <typename TAG, int NW, typename W>
+__device__ __forceinline__ bool poll_words_staggered(const W* base, const int* off, const bool* need, int t, W* out,
                                                      int* status, int spin_limit, int first_delay) {
   for (int i = 0; i < first_delay; ++i) __builtin_amdgcn_s_sleep(1);
-  u64 v[NW];
+  W v[NW];
 #pragma unroll
   for (int i = 0; i < NW; ++i) v[i] = ll_load(base + off[i]);
   for (int spins = 0;; ++spins) {

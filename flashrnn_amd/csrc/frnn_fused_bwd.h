@@ -52,7 +52,8 @@ struct BwdArgs {
   long long* trace;  // phase cycle sums per wave; only written by -DFRNN_TRACE builds
 };
 
-// 64-bit words of one inbox area of one group: [dst wg][wave][tile][src wg][element 4][lane 64]
+// words (64-bit for fp32 storage, 32-bit otherwise) of one inbox area of one group:
+// [dst wg][wave][tile][src wg][element 4][lane 64]
 constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) * 256; }
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_at(const T* p);
@@ -162,7 +163,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     }
 
   // per group: area 0, area 1 (by step parity) and a third that swallows padded lanes' stores
-  u64* const inbox = a.ll + (size_t)grp * 3 * INW;
+  // partial sums travel as 32-bit words for 16-bit storage types, as 64-bit words for fp32
+  typedef typename std::conditional<sizeof(T) == 2, Part32, Part64>::type PT;
+  typedef typename PT::Word IW;
+  IW* const inbox = reinterpret_cast<IW*>(a.ll) + (size_t)grp * 3 * INW;
 
   struct Pre { Dw<ND_> cache[UTW][NCA], sp[UTW][S], sn[UTW][S], dso[UTW][S]; };
   Pre pa, pb;
@@ -302,7 +306,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     FRNN_STAMP(c3);
     if constexpr (KW > 1) {
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
-      u64* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
+      IW* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
 #pragma unroll
       for (int r = 1; r < KW; ++r) {
         const int x = (slice + r) % KW;
@@ -310,17 +314,17 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         for (int u = 0; u < UTW; ++u) {
           float part[E];
           own_elems<TR>(acc[r][u], part);
-          u64* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
+          IW* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
 #pragma unroll
-          for (int e = 0; e < E; ++e) ll_store(dst + e * 64, ll_pack((float*)0, part[e], t));
+          for (int e = 0; e < E; ++e) ll_store(dst + e * 64, part_pack((PT*)0, part[e], t));
         }
       }
       // receive: KW-1 partial sums of the own tiles, RC sources at a time
-      const u64* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
+      const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
 #pragma unroll
       for (int r0 = 1; r0 < KW; r0 += RC) {
         constexpr int NWR = RC * UTW * E;
-        int off[NWR]; bool need[NWR]; u64 v[NWR];
+        int off[NWR]; bool need[NWR]; IW v[NWR];
 #pragma unroll
         for (int rr = 0; rr < RC; ++rr) {
           const int src = (slice + (r0 + rr < KW ? r0 + rr : 1)) % KW;
@@ -332,14 +336,14 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
               need[(rr * UTW + u) * E + e] = bvalid && (r0 + rr < KW);
             }
         }
-        if (!fail) fail = poll_words_staggered<float, NWR>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
+        if (!fail) fail = poll_words_staggered<PT, NWR>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
 #pragma unroll
         for (int rr = 0; rr < RC; ++rr)
           if (r0 + rr < KW) {
 #pragma unroll
             for (int u = 0; u < UTW; ++u)
 #pragma unroll
-              for (int e = 0; e < E; ++e) ds[u][e][0] += __uint_as_float((unsigned)v[(rr * UTW + u) * E + e]);
+              for (int e = 0; e < E; ++e) ds[u][e][0] += part_value((PT*)0, v[(rr * UTW + u) * E + e]);
           }
       }
     }
