@@ -81,10 +81,12 @@ template <int E> __device__ __forceinline__ void ll_write(float*, u64* slot, int
   for (int i = 0; i < E; ++i) ll_store(slot + ST<float>::frag_elem(row, k0 + i), ll_pack((float*)0, v[i], t));
 }
 
-// The words thread `tid` of NT polls, for a [rows_valid x KDIM] vector; -1 = none.
+// The words thread `tid` of NT polls, for a [rows_valid x KDIM] vector without the `own` columns
+// starting at `own0` (the workgroup's own slice, which it has in LDS already); -1 = none.
 template <typename T, int NP, int NT>
-__device__ __forceinline__ void ll_plan(int tid, int rows_valid, int kdim, int* q) {
-  const int tot = rows_valid * kdim / ST<T>::EPW;
+__device__ __forceinline__ void ll_plan(int tid, int rows_valid, int kdim, int own0, int own, int* q) {
+  constexpr int CG = ST<T>::EPW == 2 ? 8 : 1;  // columns per enumerated group (bf16/f16: 4 words of 2)
+  const int tot = rows_valid * (kdim - own) / ST<T>::EPW;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
     const int qc = tid + i * NT;
@@ -92,9 +94,11 @@ __device__ __forceinline__ void ll_plan(int tid, int rows_valid, int kdim, int* 
     if (ST<T>::EPW == 2) {
       const int jj = r & 3; r >>= 2;
       const int b = r % rows_valid; r /= rows_valid;
+      if (r >= own0 / CG) r += own / CG;
       word = (((r >> 2) * 64 + (r & 3) * 16 + b) << 2) + jj;
     } else {
       const int b = r % rows_valid; r /= rows_valid;
+      if (r >= own0 / CG) r += own / CG;
       word = (r >> 2) * 64 + (r & 3) * 16 + b;
     }
     q[i] = qc < tot ? word : -1;

@@ -64,7 +64,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
   constexpr int LLW = 16 * D / X::EPW;  // 64-bit words per exchange slot
-  constexpr int NP = (LLW * TR / 16 + NT - 1) / NT;  // words a thread polls per step: only the TR rows of the tile
+  // words a thread polls per step: the TR rows of the tile, without the workgroup's own slice
+  // (polled 16 at a time: longer lists are padded to whole rounds with entries that wait for nothing)
+  constexpr int NP_ = (LLW * TR / 16 * (KW > 1 ? KW - 1 : 1) / KW + NT - 1) / NT;
+  constexpr int NP = NP_ <= 16 ? NP_ : (NP_ + 15) / 16 * 16;
   constexpr int NCA = NC > 0 ? NC : 1;
   constexpr int GX = GT - GR > 0 ? GT - GR : 1;
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
@@ -162,7 +165,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   }
 
   int qpoll[NP];
-  if (KW > 1) ll_plan<T, NP, NT>(tid, rows_valid, D, qpoll);
+  if (KW > 1) ll_plan<T, NP, NT>(tid, rows_valid, D, slice * (D / KW), D / KW, qpoll);
   // per group: slot 0, slot 1, and a third area that swallows the stores of padded lanes
   u64* const llbase = a.ll + (size_t)grp * 3 * LLW;
 
@@ -279,8 +282,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         for (int k = 0; k < S; ++k) so[k][e] = s[u][e][k];
       }
       // the new h first: it is what the next step (of every workgroup of the head) waits for
-      if (KW == 1) lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
-      else ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
+      // (the own slice goes straight to the LDS buffer of the next step: the workgroup does not poll it)
+      if (KW > 1) ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
+      lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
