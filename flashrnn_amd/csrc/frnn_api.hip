@@ -62,6 +62,7 @@ static int prof_slot(int i) {  // i-th oldest entry still held -> ring slot, or 
 #define FRNN_ROW(Dv, VAR, W, U, K) {Dv, VAR, W, U, K},
 static const Plan kFwd4B[] = {FRNN_PLANS_GR4_BF16(FRNN_ROW)};
 static const Plan kFwd4F[] = {FRNN_PLANS_GR4_F32(FRNN_ROW)};
+static const Plan kFwdSB[] = {FRNN_PLANS_SLSTM_BF16(FRNN_ROW)};
 static const Plan kFwd3B[] = {FRNN_PLANS_GR3_BF16(FRNN_ROW)};
 static const Plan kFwd3F[] = {FRNN_PLANS_GR3_F32(FRNN_ROW)};
 static const Plan kFwd1B[] = {FRNN_PLANS_GR1_BF16(FRNN_ROW)};
@@ -74,12 +75,13 @@ static const Plan kBwd1B[] = {FRNN_BWD_PLANS_GR1_BF16(FRNN_ROW)};
 static const Plan kBwd1F[] = {FRNN_BWD_PLANS_GR1_F32(FRNN_ROW)};
 #undef FRNN_ROW
 
-bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out) {
+bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* out) {
+  const int GR = cell_dims(function).GR;
   const Plan* tab = nullptr;
   size_t n = 0;
 #define PICK(T) { tab = T; n = sizeof(T) / sizeof(Plan); }
   if (!backward) {
-    if (GR == 4) { if (dtype != FRNN_F32) PICK(kFwd4B) else PICK(kFwd4F) }
+    if (GR == 4) { if (dtype == FRNN_F32) PICK(kFwd4F) else if (function == FRNN_SLSTM) PICK(kFwdSB) else PICK(kFwd4B) }
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kFwd3B) else PICK(kFwd3F) }
     else { if (dtype != FRNN_F32) PICK(kFwd1B) else PICK(kFwd1F) }
   } else {
@@ -291,8 +293,7 @@ int frnn_fused_supported(int function, int dtype, int B, int N, int D) {
   int e = check_problem(function, dtype, B, 1, N, D);
   if (e) return e;
   Plan pf, pb;
-  const int GR = cell_dims(function).GR;
-  if (!find_plan(GR, dtype, D, 0, 0, &pf) || !find_plan(GR, dtype, D, 0, 1, &pb))
+  if (!find_plan(function, dtype, D, 0, 0, &pf) || !find_plan(function, dtype, D, 0, 1, &pb))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   return 0;
 }
@@ -302,7 +303,7 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
   int e = check_problem(function, dtype, B, 1, N, D);
   if (e) return e;
   Plan p;
-  if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p))
+  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   if (waves) *waves = p.waves;
   if (tiles_per_wave) *tiles_per_wave = p.utw;
@@ -320,7 +321,7 @@ size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int 
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
   Plan p;
-  if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p)) return 0;
+  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p)) return 0;
   return backward ? carve_fused_bwd(nullptr, function, dtype, B, T, N, D, p).total
                   : carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
 }
@@ -343,7 +344,7 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
   e = parse_opts(opt, function, true, &o);
   if (e) return e;
   Plan p;
-  if (!find_plan(cell_dims(function).GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
+  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   e = check_fused_sizes(function, dtype, B, T, N, D);
   if (e) return e;
@@ -414,7 +415,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   if (e) return e;
   const CellDims c = cell_dims(function);
   Plan p;
-  if (!find_plan(c.GR, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
+  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   e = check_fused_sizes(function, dtype, B, T, N, D);
   if (e) return e;

@@ -14,8 +14,8 @@ struct BwdArgs;
 template <int F, int DT> int fused_fwd_launch(const Plan& p, const FwdArgs& a, hipStream_t st);
 template <int F, int DT> int fused_bwd_launch(const Plan& p, const BwdArgs& a, hipStream_t st);
 
-// plan table lookup: gate rows per unit (4/3/1), dtype, D, variant -> plan; false if none
-bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out);
+// plan table lookup: function, dtype, D, variant -> plan; false if none
+bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* out);
 
 }  // namespace frnn
 
@@ -28,7 +28,10 @@ bool find_plan(int GR, int dtype, int D, int variant, int backward, Plan* out);
 #define FRNN_TU_T float
 #endif
 #if FRNN_F == 0 || FRNN_F == 1
-#if FRNN_DT != 1
+#if FRNN_DT != 1 && FRNN_F == 1
+#define FRNN_TU_PLANS FRNN_PLANS_SLSTM_BF16
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16
+#elif FRNN_DT != 1
 #define FRNN_TU_PLANS FRNN_PLANS_GR4_BF16
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16
 #else
