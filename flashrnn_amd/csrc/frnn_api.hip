@@ -371,7 +371,10 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
-  a.poll_delay = env_int("FRNN_POLL_DELAY", 4);  // s_sleep units before the first probe of a step (measured best: 4)
+  // s_sleep units before the first probe of a step (an early probe only adds traffic).  Measured
+  // best on MI355X: none for up to 4 workgroups per head; for 8, 4 with 4 waves per workgroup
+  // (LSTM D = 512) and 12 with 8 waves (Elman D = 1024)
+  a.poll_delay = env_int("FRNN_POLL_DELAY", p.kw > 4 ? (p.waves > 4 ? 12 : 4) : 0);
   a.h_clip = o.h_clip;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
@@ -446,7 +449,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   a.ll = w.ll; a.status = w.status;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
-  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", 4);  // ~0.12 us: measured best on MI355X
+  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6);  // measured best, as in the forward call
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
