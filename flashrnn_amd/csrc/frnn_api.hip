@@ -315,7 +315,9 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
 
 size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int D) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
-  return (size_t)T * N * ((B + 15) / 16) * 16 * D * cell_dims(function).NC * dtype_size(dtype);
+  // NC values per element, padded to whole dwords (CacheBlk in frnn_common.h)
+  const int nc = cell_dims(function).NC, ncp = dtype_size(dtype) == 2 ? (nc + 1) / 2 * 2 : nc;
+  return (size_t)T * N * ((B + 15) / 16) * 16 * D * ncp * dtype_size(dtype);
 }
 
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
@@ -372,9 +374,9 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   // s_sleep units before the first probe of a step (an early probe only adds traffic).  Measured
-  // best on MI355X: none for up to 4 workgroups per head; for 8, 4 with 4 waves per workgroup
+  // best on MI355X: 2 for up to 4 workgroups per head; for 8, 4 with 4 waves per workgroup
   // (LSTM D = 512) and 12 with 8 waves (Elman D = 1024)
-  a.poll_delay = env_int("FRNN_POLL_DELAY", p.kw > 4 ? (p.waves > 4 ? 12 : 4) : 0);
+  a.poll_delay = env_int("FRNN_POLL_DELAY", p.kw > 4 ? (p.waves > 4 ? 12 : 4) : 2);
   a.h_clip = o.h_clip;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

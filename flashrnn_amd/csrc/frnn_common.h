@@ -190,6 +190,70 @@ template <int N, bool SUB = false> __device__ __forceinline__ void buf_store(con
   else { static_assert(N == 4, "1, 2 or 4 dwords"); __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[0], d.v[1], d.v[2], d.v[3]}, r, voff, soff, 0); }
 }
 
+// N dwords per lane with as few instructions as possible (pieces of 4, then 3, 2 or 1 dwords):
+// every vector memory instruction costs a wave some 30 cycles of issue time, whatever its width
+typedef unsigned u32x3 __attribute__((ext_vector_type(3)));
+template <int N> __device__ __forceinline__ Dw<N> buf_load_wide(rsrc_t r, unsigned voff, unsigned soff) {
+  Dw<N> d;
+  constexpr int Q = N / 4 * 4, R = N % 4;
+#pragma unroll
+  for (int i = 0; i < Q; i += 4) {
+    const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff + i * 4, soff, 0);
+    d.v[i] = t.x; d.v[i + 1] = t.y; d.v[i + 2] = t.z; d.v[i + 3] = t.w;
+  }
+  if constexpr (R == 3) { const u32x3 t = __builtin_amdgcn_raw_buffer_load_b96(r, voff + Q * 4, soff, 0); d.v[Q] = t.x; d.v[Q + 1] = t.y; d.v[Q + 2] = t.z; }
+  else if constexpr (R == 2) { const u32x2 t = __builtin_amdgcn_raw_buffer_load_b64(r, voff + Q * 4, soff, 0); d.v[Q] = t.x; d.v[Q + 1] = t.y; }
+  else if constexpr (R == 1) { d.v[Q] = __builtin_amdgcn_raw_buffer_load_b32(r, voff + Q * 4, soff, 0); }
+  return d;
+}
+template <int N> __device__ __forceinline__ void buf_store_wide(const Dw<N>& d, rsrc_t r, unsigned voff, unsigned soff) {
+  constexpr int Q = N / 4 * 4, R = N % 4;
+#pragma unroll
+  for (int i = 0; i < Q; i += 4)
+    __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[i], d.v[i + 1], d.v[i + 2], d.v[i + 3]}, r, voff + i * 4, soff, 0);
+  if constexpr (R == 3) __builtin_amdgcn_raw_buffer_store_b96(u32x3{d.v[Q], d.v[Q + 1], d.v[Q + 2]}, r, voff + Q * 4, soff, 0);
+  else if constexpr (R == 2) __builtin_amdgcn_raw_buffer_store_b64(u32x2{d.v[Q], d.v[Q + 1]}, r, voff + Q * 4, soff, 0);
+  else if constexpr (R == 1) __builtin_amdgcn_raw_buffer_store_b32(d.v[Q], r, voff + Q * 4, soff, 0);
+}
+
+// Gate cache of the fused kernels: the NC cached values of one (batch row, unit) are adjacent
+// (padded to NCP, a whole number of dwords), units are the next index, so a lane moves all cached
+// values of its E consecutive units with one or two instructions.
+template <typename T, int NC> struct CacheBlk {
+  static constexpr int NCP = sizeof(T) == 2 ? (NC + 1) / 2 * 2 : NC;
+  template <int E> struct Words { static constexpr int value = E * NCP * (int)sizeof(T) / 4 > 0 ? E * NCP * (int)sizeof(T) / 4 : 1; };
+};
+// v[c][e] -> dwords, element (e, c) at flat index e*NCP + c
+template <typename T, int NC, int E> __device__ __forceinline__ Dw<CacheBlk<T, NC>::template Words<E>::value>
+cache_pack(const float (*v)[E]) {
+  constexpr int NCP = CacheBlk<T, NC>::NCP, NW = CacheBlk<T, NC>::template Words<E>::value;
+  Dw<NW> d;
+  if constexpr (sizeof(T) == 4) {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) d.v[i] = __float_as_uint(v[i % NCP][i / NCP]);
+  } else {
+#pragma unroll
+    for (int i = 0; i < NW; ++i) {
+      const int i0 = 2 * i, i1 = 2 * i + 1;
+      const float a = (i0 % NCP) < NC ? v[i0 % NCP][i0 / NCP] : 0.f, b = (i1 % NCP) < NC ? v[i1 % NCP][i1 / NCP] : 0.f;
+      d.v[i] = H16<T>::pack2(a, b);
+    }
+  }
+  return d;
+}
+template <typename T, int NC, int E> __device__ __forceinline__ void
+cache_unpack(const Dw<CacheBlk<T, NC>::template Words<E>::value>& d, float (*v)[E]) {
+  constexpr int NCP = CacheBlk<T, NC>::NCP;
+#pragma unroll
+  for (int e = 0; e < E; ++e)
+#pragma unroll
+    for (int c = 0; c < NC; ++c) {
+      const int i = e * NCP + c;
+      if constexpr (sizeof(T) == 4) v[c][e] = __uint_as_float(d.v[i]);
+      else v[c][e] = (i & 1) ? H16<T>::hi(d.v[i / 2]) : H16<T>::lo(d.v[i / 2]);
+    }
+}
+
 // 4 consecutive elements <-> 4 floats (vector form, used outside the time loops)
 template <typename T> __device__ __forceinline__ void unpack4(uint2 v, float* o) {
   o[0] = H16<T>::lo(v.x); o[1] = H16<T>::hi(v.x); o[2] = H16<T>::lo(v.y); o[3] = H16<T>::hi(v.y);

@@ -113,7 +113,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
   const rsrc_t rS0 = make_rsrc(a.s0, (size_t)S * B * ND * ES);
   const rsrc_t rDs = make_rsrc(a.dstates, (size_t)S * B * Tn * ND * ES);
-  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * NC * ES);
+  constexpr int NCP = CacheBlk<T, NCA>::NCP, NWC = CacheBlk<T, NCA>::template Words<E>::value;
+  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * (NC ? NCP : 0) * ES);
   const rsrc_t rDw = make_rsrc(a.dWx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rDx = make_rsrc(a.dgx, (size_t)B * Tn * ND * ES);
 
@@ -126,7 +127,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
     st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
     s0_v[u] = bvalid ? ((unsigned)bg * ND + d0) * ES : kInvalidOff;
-    ca_v[u] = bvalid ? (((unsigned)(ub[u] >> 4) * NC * Bpad + bg) * 16 + (esub & 15)) * ES : kInvalidOff;
+    ca_v[u] = bvalid ? ((((unsigned)(ub[u] >> 4) * Bpad + bg) * 16 + (esub & 15)) * NCP) * ES : kInvalidOff;
   }
 
   // rtf[r][u][ks]: rows p of the tiles at this wave's position in workgroup (slice + r) % KW,
@@ -168,26 +169,31 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   typedef typename PT::Word IW;
   IW* const inbox = reinterpret_cast<IW*>(a.ll) + (size_t)grp * 3 * INW;
 
-  struct Pre { Dw<ND_> cache[UTW][NCA], sp[UTW][S], sn[UTW][S], dso[UTW][S]; };
+  // operands of one step.  s_t is not among them: it is the s_(t-1) of the step before (kept in
+  // registers, `sn` below), so only the first step loads it
+  struct Pre { Dw<NWC> cache[UTW]; Dw<ND_> sp[UTW][S], dso[UTW][S]; };
   Pre pa, pb;
   auto load_pre = [&](Pre& p, int t) __attribute__((always_inline)) {
     const bool first = t == 0;
     const rsrc_t rPrev = first ? rS0 : rSt;
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-#pragma unroll
-      for (int c = 0; c < NC; ++c)
-        p.cache[u][c] = buf_load<ND_, SB>(rCa, ca_v[u], ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
+      if constexpr (NC > 0)
+        p.cache[u] = buf_load_wide<NWC>(rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
         const unsigned so = ((unsigned)k * B * Tn + t) * ND * ES;
-        p.sn[u][k] = buf_load<ND_, SB>(rSt, st_v[u], so);
         p.dso[u][k] = buf_load<ND_, SB>(rDs, st_v[u], so);
         p.sp[u][k] = buf_load<ND_, SB>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * B * ND * ES : so - ND * ES);
       }
     }
   };
   load_pre(pa, Tn - 1);
+  Dw<ND_> sn[UTW][S];
+#pragma unroll
+  for (int u = 0; u < UTW; ++u)
+#pragma unroll
+    for (int k = 0; k < S; ++k) sn[u][k] = buf_load<ND_, SB>(rSt, st_v[u], ((unsigned)k * B * Tn + (Tn - 1)) * ND * ES);
   __syncthreads();
 
 #ifdef FRNN_TRACE
@@ -209,11 +215,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
-#pragma unroll
-      for (int c = 0; c < NC; ++c) unpack<E>(pc.cache[u][c], cv[c], (T*)0);
+      if constexpr (NC > 0) cache_unpack<T, NCA, E>(pc.cache[u], cv);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
-        unpack<E>(pc.sp[u][k], spv[k], (T*)0); unpack<E>(pc.sn[u][k], snv[k], (T*)0); unpack<E>(pc.dso[u][k], dsov[k], (T*)0);
+        unpack<E>(pc.sp[u][k], spv[k], (T*)0); unpack<E>(sn[u][k], snv[k], (T*)0); unpack<E>(pc.dso[u][k], dsov[k], (T*)0);
+        sn[u][k] = pc.sp[u][k];  // s_(t-1) is the s_t of the next step
       }
       float dgr[GR][E], dgw[GW][E];
 #pragma unroll

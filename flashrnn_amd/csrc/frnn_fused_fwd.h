@@ -97,7 +97,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 
   const rsrc_t rWx = make_rsrc(a.Wx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
-  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * NC * ES);
+  constexpr int NCP = CacheBlk<T, NCA>::NCP, NWC = CacheBlk<T, NCA>::template Words<E>::value;
+  const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * (NC ? NCP : 0) * ES);
 
   int ub[UTW];
   unsigned wx_v[UTW], st_v[UTW], ca_v[UTW];  // per-lane byte offsets; out of range for padded rows
@@ -107,7 +108,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     const unsigned d0 = n * D + ub[u] + esub;
     wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
     st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
-    ca_v[u] = (bvalid && a.training) ? (((unsigned)(ub[u] >> 4) * NC * Bpad + bg) * 16 + (esub & 15)) * ES : kInvalidOff;
+    ca_v[u] = (bvalid && a.training) ? ((((unsigned)(ub[u] >> 4) * Bpad + bg) * 16 + (esub & 15)) * NCP) * ES : kInvalidOff;
   }
 
   // ---- resident operands ----------------------------------------------------------------
@@ -288,11 +289,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
-      // private cache layout [t][head][unit tile][value][batch row][16 units]
-#pragma unroll
-      for (int c = 0; c < NC; ++c)
-        buf_store<ND_, SB>(pack<E>(cv[c], (T*)0), rCa, ca_v[u],
-                       ((((unsigned)t * N + n) * (D / 16)) * NC + c) * Bpad * 16 * ES);
+      // private cache layout [t][head][unit tile][batch row][16 units][value]: one store per tile
+      if constexpr (NC > 0)
+        buf_store_wide<NWC>(cache_pack<T, NCA, E>(cv), rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
     }
 #ifdef FRNN_TRACE
     FRNN_STAMP(c3);
