@@ -158,12 +158,17 @@ static int check_problem(int function, int dtype, int B, int T, int N, int D) {
   if ((long)B * T >= (1L << 31)) return fail(FRNN_E_ARG, "B*T too large");
   return 0;
 }
+// gate cache of the fused kernels: NC values per element, padded to whole dwords (CacheBlk in frnn_common.h)
+static size_t fused_cache_bytes_of(int function, int dtype, int B, int T, int N, int D) {
+  const int nc = cell_dims(function).NC, ncp = dtype_size(dtype) == 2 ? (nc + 1) / 2 * 2 : nc;
+  return (size_t)T * N * B * D * ncp * dtype_size(dtype);
+}
 // the fused kernels address each tensor with 32-bit byte offsets
 static int check_fused_sizes(int function, int dtype, int B, int T, int N, int D) {
   const CellDims c = cell_dims(function);
   const size_t es = dtype_size(dtype), btnd = (size_t)B * T * N * D;
   const size_t gmax = (size_t)(c.GW > c.S ? c.GW : c.S);
-  const size_t cache = (size_t)T * N * ((B + 15) / 16) * 16 * D * c.NC * es;  // rows padded to 16
+  const size_t cache = fused_cache_bytes_of(function, dtype, B, T, N, D);
   if (btnd * gmax * es >= ((size_t)1 << 31) || cache >= ((size_t)1 << 31))
     return fail(FRNN_E_ARG, "a tensor of this problem reaches 2 GiB; split the batch (fused kernels use 32-bit offsets)");
   return 0;
@@ -315,9 +320,7 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
 
 size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int D) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
-  // NC values per element, padded to whole dwords (CacheBlk in frnn_common.h)
-  const int nc = cell_dims(function).NC, ncp = dtype_size(dtype) == 2 ? (nc + 1) / 2 * 2 : nc;
-  return (size_t)T * N * ((B + 15) / 16) * 16 * D * ncp * dtype_size(dtype);
+  return fused_cache_bytes_of(function, dtype, B, T, N, D);
 }
 
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {

@@ -105,7 +105,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const int r16 = lane & 15, q4 = lane >> 4;
   const int brow = O::row(r16), esub = O::sub(r16, q4);
   const int bg = bt * TR + brow;
-  const unsigned Bpad = (unsigned)((a.B + 15) / 16) * 16;
+  const unsigned Bpad = (unsigned)a.B;  // rows of the gate cache: padded rows are never read or written
   const bool bvalid = bg < B;
   const T* __restrict__ Rt = static_cast<const T*>(a.Rt);
   const unsigned ND = (unsigned)N * D;

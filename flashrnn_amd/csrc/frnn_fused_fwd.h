@@ -88,7 +88,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   const int bg = bt * TR + brow;  // batch row this lane does the gate math for
   const bool bvalid = bg < B;
   const int rows_valid = min(TR, B - bt * TR);
-  const unsigned Bpad = (unsigned)((B + 15) / 16) * 16;  // rows of the gate cache
+  const unsigned Bpad = (unsigned)B;  // rows of the gate cache: padded rows are never read or written
   const T* __restrict__ R = static_cast<const T*>(a.R);
   const T* __restrict__ bias_g = static_cast<const T*>(a.b);
   const T* __restrict__ s0 = static_cast<const T*>(a.s0);

@@ -119,3 +119,33 @@ def test_repeated_calls_are_deterministic(gpu):
     for _ in range(3):
         c = _run(gpu, "lstm", inp, "hip_fused")[0]
         assert torch.equal(a, c)
+
+
+def test_sequence_longer_than_the_tag_period(gpu):
+    """T = 66000 steps: the step tags of the workgroup exchange (16 bits forward, 8 bits backward)
+    wrap around; the fused kernels must still agree with the alternating backend, which has no
+    exchange, in every state and in dWx."""
+    from flashrnn_amd import flashrnn
+
+    function, B, T, N, D = "lstm", 2, 66000, 1, 256
+    print(f"case tag-wrap {function} B{B} T{T} N{N} D{D}", flush=True)
+    inp = make_inputs(function, B, T, N, D, 77, init="zeros", round_to=torch.bfloat16)
+    g = torch.Generator(device="cpu").manual_seed(78)
+    dst = (torch.randn((2, B, T, N, D), generator=g) * 0.1).to(gpu, torch.bfloat16)
+    out = {}
+    for backend in ("hip_fused", "hip"):
+        Wx = inp["Wx"].to(gpu, torch.bfloat16).requires_grad_(True)
+        st, _ = flashrnn(Wx, inp["R"].to(gpu, torch.bfloat16), inp["b"].to(gpu, torch.bfloat16), None,
+                         function=function, backend=backend, dtype="bfloat16")
+        (dWx,) = torch.autograd.grad(st, [Wx], grad_outputs=dst)
+        out[backend] = (st.detach().float(), dWx.float())
+    torch.cuda.synchronize()
+    for k, name in enumerate(("states", "dWx")):
+        f, a = out["hip_fused"][k], out["hip"][k]
+        assert torch.isfinite(f).all() and torch.isfinite(a).all(), name
+        err = (f - a).abs()
+        # two bf16 trajectories of the same recurrence, as in test_fused_and_alternating_agree
+        assert not bool((err > 4e-2 * torch.clamp(a.abs(), min=1.0)).any()), (name, float(err.max()))
+        # and the last steps (forward) / first steps (backward) are as close as the others: no drift after the wrap
+        tail = err[:, :, -256:] if name == "states" else err[:, :256]
+        assert float(tail.max()) <= 4e-2 * max(1.0, float(a.abs().max())), (name, float(tail.max()))
