@@ -172,7 +172,14 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   // operands of one step.  s_t is not among them: it is the s_(t-1) of the step before (kept in
   // registers, `sn` below), so only the first step loads it
   struct Pre { Dw<NWC> cache[UTW]; Dw<ND_> sp[UTW][S], dso[UTW][S]; };
-  Pre pa, pb;
+  // operands are fetched PD steps ahead into a ring of PD + 1 register sets: a head that
+  // exchanges nothing (KW = 1) has steps shorter than a fetch from HBM takes
+#ifdef FRNN_PD
+  constexpr int PD = KW == 1 ? FRNN_PD : 1;
+#else
+  constexpr int PD = KW > 1 || WAVES >= 8 ? 1 : 3;  // measured: with 8 waves and more, other waves hide the fetch
+#endif
+  Pre pre[PD + 1];
   auto load_pre = [&](Pre& p, int t) __attribute__((always_inline)) {
     const bool first = t == 0;
     const rsrc_t rPrev = first ? rS0 : rSt;
@@ -188,7 +195,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
     }
   };
-  load_pre(pa, Tn - 1);
+#pragma unroll
+  for (int i = 0; i < PD; ++i) load_pre(pre[i], Tn - 1 - i > 0 ? Tn - 1 - i : 0);
   Dw<ND_> sn[UTW][S];
 #pragma unroll
   for (int u = 0; u < UTW; ++u)
@@ -209,9 +217,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     constexpr bool cut = decltype(CUT)::value;
     T* const gb = (t & 1) ? gbuf1 : gbuf0;
     FRNN_STAMP(c0);
-    // (readfirstlane: the compiler otherwise forms max(t - 1, 0) with a saturating VALU subtract and
-    // then wraps a buffer load that uses it as a scalar offset into a waterfall loop)
-    load_pre(pn, __builtin_amdgcn_readfirstlane(t > 0 ? t - 1 : 0));
+    // (readfirstlane: the compiler otherwise forms max(t - PD, 0) with a saturating VALU subtract
+    // and then wraps a buffer load that uses it as a scalar offset into a waterfall loop)
+    load_pre(pn, __builtin_amdgcn_readfirstlane(t >= PD ? t - PD : 0));
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
@@ -359,20 +367,37 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #endif
   };
 
+  // the time loop, unrolled over the ring: step t - j consumes set j and refills the set that the
+  // step before it consumed
   int t = Tn - 1;
   if (a.cut) {
-    for (; t >= 1; t -= 2) {
-      step(std::true_type{}, t, pa, pb);
-      step(std::true_type{}, t - 1, pb, pa);
+    for (; t >= PD; t -= PD + 1) {
+#pragma unroll
+      for (int j = 0; j <= PD; ++j) step(std::true_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
     }
-    if (t == 0) step(std::true_type{}, 0, pa, pb);
-  } else {
+#pragma unroll
+    for (int j = 0; j < PD; ++j)
+      if (t - j >= 0) step(std::true_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
+  } else if constexpr (PD == 1) {
+    // (written out: in the general form below the register allocation of the largest kernels,
+    // which sit at the 256-register limit, comes out with spills)
     for (; t >= 1 && !dead; t -= 2) {
-      step(std::false_type{}, t, pa, pb);
+      step(std::false_type{}, t, pre[0], pre[1]);
       if (dead) break;
-      step(std::false_type{}, t - 1, pb, pa);
+      step(std::false_type{}, t - 1, pre[1], pre[0]);
     }
-    if (!dead && t == 0) step(std::false_type{}, 0, pa, pb);
+    if (!dead && t == 0) step(std::false_type{}, 0, pre[0], pre[1]);
+  } else {
+    for (; t >= PD && !dead; t -= PD + 1) {
+#pragma unroll
+      for (int j = 0; j <= PD; ++j) {
+        step(std::false_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
+        if (dead) break;
+      }
+    }
+#pragma unroll
+    for (int j = 0; j < PD; ++j)
+      if (!dead && t - j >= 0) step(std::false_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
   }
   if (!dead && barrier_or(fail, dead_flag)) dead = true;
 #ifdef FRNN_TRACE

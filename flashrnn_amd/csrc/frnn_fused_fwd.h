@@ -170,14 +170,25 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   // per group: slot 0, slot 1, and a third area that swallows the stores of padded lanes
   u64* const llbase = a.ll + (size_t)grp * 3 * LLW;
 
-  Dw<ND_> wxA[UTW][GW], wxB[UTW][GW];
+  // Wx is fetched PD steps ahead into a ring of PD + 1 register sets.  A head that exchanges
+  // nothing (KW = 1) has steps shorter than a fetch from HBM takes (D = 64: 1100 cycles against
+  // ~1900), so it looks further ahead and issues the loads behind its MFMAs; with an exchange the
+  // loads must stay well clear of the poll, whose wait counts every load in flight.
+#ifdef FRNN_PD
+  constexpr int PD = KW == 1 ? FRNN_PD : 1;
+#else
+  constexpr int PD = KW > 1 || WAVES >= 16 ? 1 : (D <= 64 ? 3 : 2);  // measured; 16 waves have no registers to spare
+#endif
+  constexpr bool WX_LATE = KW == 1;
+  Dw<ND_> wx[PD + 1][UTW][GW];
   auto load_wx = [&](Dw<ND_> (&dst)[UTW][GW], int t) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
       for (int g = 0; g < GW; ++g) dst[u][g] = buf_load<ND_, SB>(rWx, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
   };
-  load_wx(wxA, 0);
+#pragma unroll
+  for (int i = 0; i < PD; ++i) load_wx(wx[i], min(i, Tn - 1));
   __syncthreads();
 
 #ifdef FRNN_TRACE
@@ -185,7 +196,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   const long long tr_begin = clock64();
 #endif
   bool dead = false;
-  // one time step: consumes `wc` (Wx of step t), prefetches Wx of step t+1 into `wn`
+  // one time step: consumes `wc` (Wx of step t), prefetches Wx of step t+PD into `wn`
   auto step = [&](const int t, Dw<ND_> (&wc)[UTW][GW], Dw<ND_> (&wn)[UTW][GW]) __attribute__((always_inline)) {
     const int cur = t & 1;
     FRNN_STAMP(c0);
@@ -198,7 +209,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       }
     }
     FRNN_STAMP(c1);
-    load_wx(wn, min(t + 1, Tn - 1));
+    if constexpr (!WX_LATE) load_wx(wn, min(t + PD, Tn - 1));
 
     // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once
     // NACC accumulators per (tile, gate), used round robin over the k-steps, so that at least ~4
@@ -244,6 +255,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         for (int j = 1; j < NACC; ++j) acc[u][g] += accp[j][u][g];
       }
 
+    if constexpr (WX_LATE) {
+      load_wx(wn, min(t + PD, Tn - 1));
+      __builtin_amdgcn_sched_barrier(0);
+    }
 #ifdef FRNN_TRACE
     { float sink = 0.f;
 #pragma unroll
@@ -299,13 +314,30 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #endif
   };
 
+  // the time loop, unrolled over the ring: step t + j consumes set j and refills the set that the
+  // step before it consumed
   int t = 0;
-  for (; t + 1 < Tn && !dead; t += 2) {
-    step(t, wxA, wxB);
-    if (dead) break;
-    step(t + 1, wxB, wxA);
+  if constexpr (PD == 1) {
+    // (written out: the general form below changes the register allocation of kernels that sit
+    // at the register limit)
+    for (; t + 1 < Tn && !dead; t += 2) {
+      step(t, wx[0], wx[1]);
+      if (dead) break;
+      step(t + 1, wx[1], wx[0]);
+    }
+    if (!dead && t < Tn) step(t, wx[0], wx[1]);
+    t = Tn;
   }
-  if (!dead && t < Tn) step(t, wxA, wxB);
+  for (; t + PD < Tn && !dead; t += PD + 1) {
+#pragma unroll
+    for (int j = 0; j <= PD; ++j) {
+      step(t + j, wx[j], wx[(j + PD) % (PD + 1)]);
+      if (dead) break;
+    }
+  }
+#pragma unroll
+  for (int j = 0; j < PD; ++j)
+    if (!dead && t + j < Tn) step(t + j, wx[j], wx[(j + PD) % (PD + 1)]);
 
 #ifdef FRNN_TRACE
   if (lane == 0 && a.trace) {
