@@ -5,7 +5,9 @@
 // X(D, VARIANT, WAVES, UTW, KW):  D = 16 * UTW * WAVES * KW.
 //   R registers per lane = UTW * G_r * D / 8 (bf16) or UTW * G_r * D / 4 (f32); a workgroup of
 //   4 waves (one per SIMD) may use up to 512 VGPRs per lane, one of 8 waves 256, of 16 waves 128.
-// VARIANT 0 is the default; others are alternatives selectable with FRNN_FUSED_VARIANT for tuning.
+// VARIANT 0 is the default; to try another tiling add an X(D, 1, ...) entry and run with
+// FRNN_FUSED_VARIANT=1.  The alternatives that were measured and lost (4 waves x 2 tiles for
+// D = 128, 2 x 8 waves or 8 x 2 waves for D = 256, ...) are not compiled in.
 // Forward and backward tile independently (the gate cache layout does not depend on the plan).
 #pragma once
 
@@ -19,38 +21,38 @@ struct Plan { int D, variant, waves, utw, kw; };
 // beat fewer, fuller workgroups (the step is a dependency chain, not a throughput problem).
 // ---- 4 recurrent gate rows per unit (lstm, slstm) --------------------------------------------
 #define FRNN_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 1, 3) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 2, 2, 1, 8) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8)
 #define FRNN_BWD_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 4, 1, 3) X(192, 1, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 2, 2, 1, 8) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 4, 1, 3) \
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8)
 // slstm: its heavier gate math tips D = 192 forward to 3 workgroups of 4 waves (1.19 against 1.26 ms)
 #define FRNN_PLANS_SLSTM_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 4, 1, 3) X(192, 1, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 2, 2, 1, 8) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 4, 1, 3) \
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8)
 #define FRNN_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(128, 1, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
 #define FRNN_BWD_PLANS_GR4_F32 FRNN_PLANS_GR4_F32
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8)
 #define FRNN_BWD_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 1, 3) \
-  X(256, 0, 4, 1, 4) X(256, 1, 4, 2, 2) X(256, 3, 8, 1, 2) X(512, 0, 4, 1, 8)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8)
 #define FRNN_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
 #define FRNN_BWD_PLANS_GR3_F32 FRNN_PLANS_GR3_F32
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
-  X(256, 0, 16, 1, 1) X(256, 1, 4, 4, 1) X(512, 0, 4, 2, 4) X(512, 1, 8, 1, 4) X(512, 2, 16, 1, 2) \
-  X(1024, 0, 8, 1, 8) X(1024, 1, 4, 1, 16)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
+  X(256, 0, 16, 1, 1) X(384, 0, 8, 3, 1) X(512, 0, 4, 2, 4) \
+  X(1024, 0, 8, 1, 8)
 #define FRNN_BWD_PLANS_GR1_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 8, 1, 1) X(128, 1, 4, 2, 1) X(192, 0, 12, 1, 1) X(192, 1, 4, 3, 1) \
-  X(256, 0, 16, 1, 1) X(256, 1, 4, 4, 1) X(512, 0, 16, 1, 2) X(512, 1, 4, 2, 4) X(512, 2, 8, 1, 4) \
-  X(1024, 0, 8, 1, 8) X(1024, 1, 4, 1, 16)
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
+  X(256, 0, 16, 1, 1) X(384, 0, 8, 1, 3) X(512, 0, 16, 1, 2) \
+  X(1024, 0, 8, 1, 8)
 #define FRNN_PLANS_GR1_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) X(256, 0, 4, 4, 1) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) X(256, 0, 4, 4, 1) \
   X(512, 0, 4, 2, 4) X(1024, 0, 4, 1, 16)
 #define FRNN_BWD_PLANS_GR1_F32 FRNN_PLANS_GR1_F32

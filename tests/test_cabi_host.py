@@ -49,11 +49,12 @@ def test_function_dims_mirror_the_registry(lib):
 def test_supported_table(lib):
     L, S, G, E = (_lib.FUNCTION_IDS[k] for k in ("lstm", "slstm", "gru", "elman"))
     for f in (L, S, G, E):
-        for D in (32, 64, 128, 192, 256, 512):
+        for D in (32, 64, 96, 128, 192, 256, 384, 512):
             assert lib.frnn_fused_supported(f, 0, 8, 3, D) == 0, (f, D)
     assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == _lib.E_UNSUPPORTED  # too large to keep on chip
     assert lib.frnn_fused_supported(L, 1, 8, 1, 512) == _lib.E_UNSUPPORTED   # fp32 R is twice the size
+    assert lib.frnn_fused_supported(L, 1, 8, 1, 96) == 0 and lib.frnn_fused_supported(L, 1, 8, 1, 384) == _lib.E_UNSUPPORTED
     assert lib.frnn_fused_supported(L, 0, 8, 1, 48) == _lib.E_UNSUPPORTED
     assert b"head dim" in lib.frnn_last_error()
     assert lib.frnn_alt_supported(L, 0, 8, 1, 1024) == 0

@@ -32,6 +32,15 @@ FUSED_SMALL = [
     ("slstm", 16, 12, 2, 192, "bfloat16"),   # D not a power of two, 3 workgroups per head
     ("slstm", 5, 8, 1, 192, "float32"),
     ("slstm", 12, 5, 2, 256, "bfloat16"),
+    ("lstm", 7, 6, 2, 96, "bfloat16"),       # 6 waves, 3 k-steps
+    ("lstm", 5, 5, 1, 96, "float32"),
+    ("gru", 9, 5, 1, 96, "bfloat16"),
+    ("slstm", 6, 7, 1, 96, "bfloat16"),
+    ("elman", 10, 6, 2, 96, "bfloat16"),
+    ("lstm", 9, 7, 1, 384, "bfloat16"),      # 6 workgroups per head
+    ("gru", 6, 5, 1, 384, "bfloat16"),
+    ("slstm", 5, 6, 1, 384, "bfloat16"),
+    ("elman", 12, 6, 1, 384, "bfloat16"),    # 3 workgroups of 8 waves
 ]
 
 
