@@ -168,6 +168,9 @@ def main():
     roofline = dict(kernel=dom, bound="mfma", achieved=achieved, peak=peak, unit="TFLOP/s", frac=achieved / peak,
                     traffic=TRAFFIC_BYTES.get((args.workload, dom)), avg_launch_ms=dom_ms, launches_per_step=cand[dom][1],
                     us_per_time_step=dom_ms * 1e3 / w["T"])
+    # the whole step against the same peak: 3 contractions of flops_scan each when there is a backward pass
+    step_flops = flops_scan * (3.0 if w["bwd"] else 1.0)
+    roofline.update(whole_step_tflops=step_flops / (ms * 1e-3) / 1e12, whole_step_frac=step_flops / (ms * 1e-3) / 1e12 / peak)
     try:
         from flashrnn_amd import fused_plan
 
