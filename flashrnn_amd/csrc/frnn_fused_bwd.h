@@ -220,6 +220,16 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     // (readfirstlane: the compiler otherwise forms max(t - PD, 0) with a saturating VALU subtract
     // and then wraps a buffer load that uses it as a scalar offset into a waterfall loop)
     load_pre(pn, __builtin_amdgcn_readfirstlane(t >= PD ? t - PD : 0));
+    // dWx_t (and the GRU's g-gate cotangent).  With an exchange the stores are issued after the
+    // partial sums are sent, where they fill the wait for the other workgroups instead of delaying
+    // the barrier (a vector memory instruction costs ~30 cycles to issue)
+    constexpr bool DW_LATE = KW > 1 && GW > 1;  // (a single store, Elman, measured no better behind the send)
+    Dw<ND_> dwp[UTW][GW], dxp[UTW];
+    auto store_dw = [&](int u) __attribute__((always_inline)) {
+#pragma unroll
+      for (int g = 0; g < GW; ++g) buf_store<ND_, SB>(dwp[u][g], rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
+      if (F == FRNN_GRU) buf_store<ND_, SB>(dxp[u], rDx, st_v[u], (unsigned)t * ND * ES);
+    };
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
@@ -249,10 +259,16 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
         for (int k = 0; k < S; ++k) ds[u][e][k] = bvalid ? ds[u][e][k] : 0.f;
       }
+      if constexpr (DW_LATE && !cut) {
 #pragma unroll
-      for (int g = 0; g < GW; ++g)
-        buf_store<ND_, SB>(pack<E>(dgw[g], (T*)0), rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
-      if (F == FRNN_GRU) buf_store<ND_, SB>(pack<E>(dgr[0], (T*)0), rDx, st_v[u], (unsigned)t * ND * ES);
+        for (int g = 0; g < GW; ++g) dwp[u][g] = pack<E>(dgw[g], (T*)0);
+        if (F == FRNN_GRU) dxp[u] = pack<E>(dgr[0], (T*)0);
+      } else {
+#pragma unroll
+        for (int g = 0; g < GW; ++g)
+          buf_store<ND_, SB>(pack<E>(dgw[g], (T*)0), rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
+        if (F == FRNN_GRU) buf_store<ND_, SB>(pack<E>(dgr[0], (T*)0), rDx, st_v[u], (unsigned)t * ND * ES);
+      }
       if constexpr (!cut) {
 #pragma unroll
         for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
@@ -332,6 +348,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
           for (int e = 0; e < E; ++e) ll_store(dst + e * 64, part_pack((PT*)0, part[e], t));
         }
+      }
+      if constexpr (DW_LATE) {
+#pragma unroll
+        for (int u = 0; u < UTW; ++u) store_dw(u);
       }
       // receive: KW-1 partial sums of the own tiles, RC sources at a time
       const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
