@@ -457,7 +457,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   // measured best, as in the forward call; the cells with several dWx stores issue them between
   // the send and the first probe, which is part of their delay
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", function == FRNN_ELMAN ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
-                                                                        : (p.kw > 4 ? 6 : 4));
+                                                                        : 4);
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

@@ -283,6 +283,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     // one accumulator per tile: splitting a lone chain over several accumulators (as the forward
     // kernel does) measured 3-8 % slower here, before and after the barrier was made LDS-only
     constexpr int NACC = 1;
+    // With 3 and more workgroups per head the products that other workgroups wait for come first
+    // and are sent at once; the product for the own tiles follows while those words travel (it
+    // needs all fragments still in registers: one chunk)
+    constexpr bool OWN_LAST = KW >= 3 && KS == chunk_of(KS);
     f32x4 accp[NACC][KW][UTW];
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;
     constexpr int KC = chunk_of(KS);
@@ -303,28 +307,27 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       for (int k = 0; k < KC; ++k) {
         const int ks = kc * KC + k, j = ks % NACC;
 #pragma unroll
-        for (int r = 0; r < KW; ++r)
+        for (int r = OWN_LAST ? 1 : 0; r < KW; ++r)
 #pragma unroll
           for (int u = 0; u < UTW; ++u)
             accp[j][r][u] = X::mfma(rtf[r][u][ks], gq[kc & 1][k], ks < NACC ? f32x4{0.f, 0.f, 0.f, 0.f} : accp[j][r][u]);
         if (j == NACC - 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
+    static_assert(NACC == 1, "one accumulator per tile");
     f32x4 acc[KW][UTW];
 #pragma unroll
-    for (int r = 0; r < KW; ++r)
+    for (int r = OWN_LAST ? 1 : 0; r < KW; ++r)
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) acc[r][u] = accp[0][r][u];
+    if constexpr (!OWN_LAST) {
 #pragma unroll
       for (int u = 0; u < UTW; ++u) {
-        acc[r][u] = accp[0][r][u];
+        float own[E];
+        own_elems<TR>(acc[0][u], own);
 #pragma unroll
-        for (int j = 1; j < NACC; ++j) acc[r][u] += accp[j][r][u];
+        for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
       }
-#pragma unroll
-    for (int u = 0; u < UTW; ++u) {
-      float own[E];
-      own_elems<TR>(acc[0][u], own);
-#pragma unroll
-      for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
     }
 
 #ifdef FRNN_TRACE
@@ -352,6 +355,21 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       if constexpr (DW_LATE) {
 #pragma unroll
         for (int u = 0; u < UTW; ++u) store_dw(u);
+      }
+      if constexpr (OWN_LAST) {
+        // the product for the own tiles, while the words just sent travel
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks)
+#pragma unroll
+          for (int u = 0; u < UTW; ++u)
+            accp[0][0][u] = X::mfma(rtf[0][u][ks], gq[0][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : accp[0][0][u]);
+#pragma unroll
+        for (int u = 0; u < UTW; ++u) {
+          float own[E];
+          own_elems<TR>(accp[0][0][u], own);
+#pragma unroll
+          for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
+        }
       }
       // receive: KW-1 partial sums of the own tiles, RC sources at a time
       const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
