@@ -105,6 +105,21 @@ static int env_int(const char* name, int dflt) {
   return (v && *v) ? atoi(v) : dflt;
 }
 
+// s_sleep units before the first probe of a forward step.  A probe that reaches memory before the
+// data costs a whole extra round trip and adds traffic, one that comes late costs its lateness; where
+// the data arrives depends on how long the other workgroups' gate math and stores take, so the best
+// value differs by cell and tiling.  Measured on MI355X (bf16, T = 1024; a unit off costs 1-3 %):
+//   lstm  D=256 (4 workgroups) 3, D=384 (6) 6, D=512 (8) 3;  gru D=256 5;  slstm D=192 (3) 2;
+//   elman D=512 (4 workgroups, 2 tiles per wave) 6, D=1024 (8 workgroups of 8 waves) 12.
+static int fwd_poll_delay_default(int function, const Plan& p) {
+  if (p.kw <= 1) return 0;
+  if (function == FRNN_ELMAN) return p.waves > 4 ? 12 : 6;
+  if (p.kw == 3) return 2;
+  if (p.kw == 6) return 6;
+  if (p.kw == 4 && function == FRNN_GRU) return 5;
+  return 3;
+}
+
 // compute units of the current device; 256 (MI355X) if no device can be queried
 static int device_cus() {
   static int cached[64] = {0};
@@ -376,10 +391,7 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
-  // s_sleep units before the first probe of a step (an early probe only adds traffic).  Measured
-  // best on MI355X: 2 for up to 4 workgroups per head; for 8, 4 with 4 waves per workgroup
-  // (LSTM D = 512) and 12 with 8 waves (Elman D = 1024)
-  a.poll_delay = env_int("FRNN_POLL_DELAY", p.kw > 4 ? (p.waves > 4 ? 12 : 4) : 2);
+  a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(function, p));
   a.h_clip = o.h_clip;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

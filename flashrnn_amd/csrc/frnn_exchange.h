@@ -83,13 +83,15 @@ template <int E> __device__ __forceinline__ void ll_write(float*, u64* slot, int
 
 // The words thread `tid` of NT polls, for a [rows_valid x KDIM] vector without the `own` columns
 // starting at `own0` (the workgroup's own slice, which it has in LDS already); -1 = none.
-template <typename T, int NP, int NT>
+// PAIRS: entries 2j and 2j+1 of a thread are two adjacent words (16 bytes, fetched with one load).
+template <typename T, int NP, int NT, bool PAIRS = false>
 __device__ __forceinline__ void ll_plan(int tid, int rows_valid, int kdim, int own0, int own, int* q) {
   constexpr int CG = ST<T>::EPW == 2 ? 8 : 1;  // columns per enumerated group (bf16/f16: 4 words of 2)
+  static_assert(!PAIRS || (ST<T>::EPW == 2 && NP % 2 == 0), "pairs: 16-bit types, an even number of words");
   const int tot = rows_valid * (kdim - own) / ST<T>::EPW;
 #pragma unroll
   for (int i = 0; i < NP; ++i) {
-    const int qc = tid + i * NT;
+    const int qc = PAIRS ? 2 * tid + (i & 1) + (i >> 1) * 2 * NT : tid + i * NT;
     int r = qc, word;
     if (ST<T>::EPW == 2) {
       const int jj = r & 3; r >>= 2;
@@ -161,6 +163,55 @@ __device__ __forceinline__ bool poll_words_staggered(const W* base, const int* o
   }
 }
 constexpr int probe_depth(int) { return 1; }
+
+// The same wait for pairs of adjacent words, each pair fetched with one 16-byte agent-scope load
+// (raw buffer load, cache policy sc1): half the memory instructions per probe.  A 16-byte load is
+// not one atomic access, which the protocol does not need: every 32-bit half carries its own tag.
+template <typename TAG, int NW>
+__device__ __forceinline__ bool poll_pairs(rsrc_t slot, unsigned soff, const int* off, const bool* need, int t, u64* out,
+                                           int* status, int spin_limit, int first_delay) {
+  static_assert(NW % 2 == 0, "pairs");
+  if (spin_limit < -1) return true;  // host-side test hook: every wait gives up at once
+  for (int i = 0; i < first_delay; ++i) __builtin_amdgcn_s_sleep(1);
+  for (int spins = 0;; ++spins) {
+#pragma unroll
+    for (int i = 0; i < NW; i += 2) {
+      const u32x4 v = __builtin_amdgcn_raw_buffer_load_b128(slot, (unsigned)off[i] * 8u, soff, 16 /* sc1 */);
+      out[i] = (u64)v.x | ((u64)v.y << 32);
+      out[i + 1] = (u64)v.z | ((u64)v.w << 32);
+    }
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) ok = ok & (!need[i] | ll_ok((TAG*)0, out[i], t));
+    if (__all(ok)) return false;
+    if (spins > spin_limit) return true;
+    if ((spins & 63) == 63 &&
+        __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
+  }
+}
+template <typename T, int NP>
+__device__ __forceinline__ bool ll_gather_pairs(rsrc_t slots, unsigned soff, const int* q, int t, T* lds_dst,
+                                                int* status, int spin_limit, int first_delay) {
+  constexpr int CH = NP < 16 ? NP : 16;  // words polled together
+  static_assert(NP % CH == 0 && CH % 2 == 0, "poll list must split into whole chunks of pairs");
+  bool fail = false;
+#pragma unroll
+  for (int c0 = 0; c0 < NP; c0 += CH) {
+    int off[CH]; bool need[CH]; u64 v[CH];
+#pragma unroll
+    for (int i = 0; i < CH; ++i) { need[i] = q[c0 + i] >= 0; off[i] = need[i] ? q[c0 + i] : 0; }
+    fail = fail || poll_pairs<T, CH>(slots, soff, off, need, t, v, status, spin_limit, c0 == 0 ? first_delay : 0);
+    if (!fail) {
+      // (the list is a whole number of pairs: its length, rows x columns / 2, is even)
+#pragma unroll
+      for (int i = 0; i < CH; i += 2)
+        if (need[i])
+          *reinterpret_cast<uint2*>(reinterpret_cast<unsigned*>(lds_dst) + off[i]) =
+              make_uint2(ll_payload((T*)0, v[i]), ll_payload((T*)0, v[i + 1]));
+    }
+  }
+  return fail;
+}
 
 // Forward gather: poll the planned words of slot, then copy their payloads to LDS.
 template <typename T, int NP>

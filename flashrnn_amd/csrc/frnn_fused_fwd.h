@@ -67,7 +67,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   // words a thread polls per step: the TR rows of the tile, without the workgroup's own slice
   // (polled 16 at a time: longer lists are padded to whole rounds with entries that wait for nothing)
   constexpr int NP_ = (LLW * TR / 16 * (KW > 1 ? KW - 1 : 1) / KW + NT - 1) / NT;
-  constexpr int NP = NP_ <= 16 ? NP_ : (NP_ + 15) / 16 * 16;
+  // 16-bit types fetch two adjacent words with one 16-byte load when a thread polls more than one
+  constexpr bool PAIRS = X::EPW == 2 && NP_ > 1;
+  constexpr int NP = NP_ <= 16 ? (PAIRS ? (NP_ + 1) / 2 * 2 : NP_) : (NP_ + 15) / 16 * 16;
   constexpr int NCA = NC > 0 ? NC : 1;
   constexpr int GX = GT - GR > 0 ? GT - GR : 1;
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
@@ -166,9 +168,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   }
 
   int qpoll[NP];
-  if (KW > 1) ll_plan<T, NP, NT>(tid, rows_valid, D, slice * (D / KW), D / KW, qpoll);
+  if (KW > 1) ll_plan<T, NP, NT, PAIRS>(tid, rows_valid, D, slice * (D / KW), D / KW, qpoll);
   // per group: slot 0, slot 1, and a third area that swallows the stores of padded lanes
   u64* const llbase = a.ll + (size_t)grp * 3 * LLW;
+  const rsrc_t rLL = make_rsrc(llbase, (size_t)2 * LLW * 8);  // the two slots that are read
 
   // Wx is fetched PD steps ahead into a ring of PD + 1 register sets.  A head that exchanges
   // nothing (KW = 1) has steps shorter than a fetch from HBM takes (D = 64: 1100 cycles against
@@ -202,7 +205,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     FRNN_STAMP(c0);
     if (t > 0) {
       if (KW > 1) {
-        const bool fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
+        bool fail;
+        if constexpr (PAIRS) fail = ll_gather_pairs<T, NP>(rLL, (unsigned)((t - 1) & 1) * LLW * 8u, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
+        else fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
         if (barrier_or(fail, &dead_flag)) { dead = true; return; }
       } else {
         lds_barrier();
