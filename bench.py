@@ -98,21 +98,36 @@ def run_gpu(w, backend, steps, warmup, device):
 
 
 def run_cpu_baseline(w, budget_s=20.0):
-    """The CPU oracle (a port of the reference's vanilla backend) on the host cores, fp32."""
+    """The CPU oracle (a port of the reference's vanilla backend) on the host cores, fp32, on a bounded
+    sample: the first T_cpu time steps of the workload, T_cpu chosen from a 32-step probe so that one
+    pass takes about 8 s (the whole sequence if that is shorter: C1, C2)."""
     import torch
     from oracle import flashrnn_oracle, make_inputs
 
     torch.set_num_threads(os.cpu_count() or 1)
     rt = torch.bfloat16 if w["dtype"] == "bfloat16" else None
-    inp = make_inputs(w["function"], w["B"], w["T"], w["N"], w["D"], w["seed"], init=w["init"], round_to=rt,
-                      grad_on=w["grad_on"], forget_bias_linspace=w.get("forget_bias_linspace", False))
+    T_full = w["T"]
 
-    def one():
-        leaves = [inp[k].clone().requires_grad_(w["bwd"]) for k in ("Wx", "R", "b", "states")]
-        out, _ = flashrnn_oracle(*leaves, function=w["function"], slstm_per_element_first_step=True)
-        if w["bwd"]:
-            torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"])
+    def make(T):
+        wc = dict(w, T=T)
+        inp = make_inputs(wc["function"], wc["B"], T, wc["N"], wc["D"], wc["seed"], init=wc["init"], round_to=rt,
+                          grad_on=wc["grad_on"], forget_bias_linspace=wc.get("forget_bias_linspace", False))
 
+        def one():
+            leaves = [inp[k].clone().requires_grad_(w["bwd"]) for k in ("Wx", "R", "b", "states")]
+            out, _ = flashrnn_oracle(*leaves, function=w["function"], slstm_per_element_first_step=True)
+            if w["bwd"]:
+                torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"])
+        return one
+
+    probe_T = min(T_full, 32)
+    probe = make(probe_T)
+    probe()
+    t0 = time.perf_counter()
+    probe()
+    per_step = (time.perf_counter() - t0) / probe_T
+    T_cpu = max(probe_T, min(T_full, int(8.0 / max(per_step, 1e-6))))
+    one = make(T_cpu)
     t0 = time.perf_counter()
     one()  # warm-up, also tells us how many repetitions fit the budget
     first = time.perf_counter() - t0
@@ -123,8 +138,9 @@ def run_cpu_baseline(w, budget_s=20.0):
         one()
         times.append(time.perf_counter() - t0)
     med = sorted(times)[len(times) // 2]
-    return dict(value=w["B"] * w["T"] / med, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
-                sample=f"full workload ({describe(w)}), fp32 torch CPU, median of {reps} after 1 warm-up",
+    sample = "full workload" if T_cpu == T_full else f"first {T_cpu} of {T_full} time steps"
+    return dict(value=w["B"] * T_cpu / med, unit="tokens/s", cores=torch.get_num_threads(), kind="port",
+                sample=f"{sample} ({describe(w)}), fp32 torch CPU, median of {reps} after 1 warm-up",
                 ms=med * 1e3)
 
 
