@@ -110,12 +110,13 @@ static int env_int(const char* name, int dflt) {
 // the data arrives depends on how long the other workgroups' gate math and stores take, so the best
 // value differs by cell and tiling.  Measured on MI355X (bf16, T = 1024; a unit off costs 1-3 %):
 //   lstm  D=256 (4 workgroups) 3, D=384 (6) 6, D=512 (8) 3;  gru D=256 5;  slstm D=192 (3) 2;
+//   lstm D=768 (12 workgroups) 6;
 //   elman D=512 (4 workgroups, 2 tiles per wave) 6, D=1024 (8 workgroups of 8 waves) 12.
 static int fwd_poll_delay_default(int function, const Plan& p) {
   if (p.kw <= 1) return 0;
   if (function == FRNN_ELMAN) return p.waves > 4 ? 12 : 6;
   if (p.kw == 3) return 2;
-  if (p.kw == 6) return 6;
+  if (p.kw == 6 || p.kw == 12) return 6;
   if (p.kw == 4 && function == FRNN_GRU) return 5;
   return 3;
 }
@@ -469,7 +470,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   // measured best, as in the forward call; the cells with several dWx stores issue them between
   // the send and the first probe, which is part of their delay
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", function == FRNN_ELMAN ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
-                                                                        : 4);
+                                                                        : (p.kw >= 12 ? 8 : 4));
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

@@ -56,6 +56,22 @@ struct BwdArgs {
 // [dst wg][wave][tile][src wg][element 4][lane 64]
 constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) * 256; }
 
+// Resident operand of the reverse product: a wave holds KW*UTW*KS fragments of the transposed R (all
+// destination tiles at its position, its workgroup's gate rows).  At 4 waves per workgroup a wave has
+// 512 registers; when the fragments alone would take more than 320 of them (LSTM D = 768: 384), those
+// of the last RLD destination tiles (as many as bring the rest down to 256) live in LDS instead (the reverse kernel needs little LDS otherwise)
+// and are read back, one k-step ahead, as the A operand of their MFMAs.
+constexpr int bwd_lds_tiles(int GR, int D, int WAVES, int UTW, int KW, int esize) {
+  const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4;
+  const int KS = GR * (D / KW) / KM, regs = KW * UTW * KS * FR, per = UTW * KS * FR;
+  return (WAVES == 4 && regs > 320) ? (regs - 256 + per - 1) / per : 0;
+}
+constexpr size_t bwd_lds_bytes(int GR, int D, int WAVES, int UTW, int KW, int esize) {
+  const int KM = esize == 4 ? 4 : 32, FRB = esize == 4 ? 4 : 16;
+  const int KS = GR * (D / KW) / KM;
+  return (size_t)2 * 16 * GR * (D / KW) * esize + (size_t)WAVES * bwd_lds_tiles(GR, D, WAVES, UTW, KW, esize) * UTW * KS * 64 * FRB;
+}
+
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_at(const T* p);
 template <> __device__ __forceinline__ bf16x8 load_frag_at<bf16_t>(const bf16_t* p) { return *reinterpret_cast<const bf16x8*>(p); }
 template <> __device__ __forceinline__ f16x8 load_frag_at<half_t>(const half_t* p) { return *reinterpret_cast<const f16x8*>(p); }
@@ -90,6 +106,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);
   T* const gbuf1 = gbuf0 + 16 * KDL;
+  constexpr int RLD = bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)), KWR = KW - RLD;
+  // this lane's fragments of the last RLD destination tiles: [wave][tile][u][ks][lane]
+  Frag* const rl = reinterpret_cast<Frag*>(smem_raw + (size_t)2 * 16 * KDL * sizeof(T)) +
+                   (size_t)(threadIdx.x >> 6) * RLD * UTW * KS * 64 + (threadIdx.x & 63);
   // a static LDS word, not a slice of the dynamic array: through a pointer computed from the
   // dynamic array the compiler reads the flag with a flat load, which has to wait for every global
   // load in flight (measured: the operand prefetch's full HBM latency, once per step)
@@ -132,7 +152,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 
   // rtf[r][u][ks]: rows p of the tiles at this wave's position in workgroup (slice + r) % KW,
   // columns = the own gate rows, local index kk = g*DL + (d - slice*DL)
-  Frag rtf[KW][UTW][KS];
+  Frag rtf[KWR][UTW][KS];
 #pragma unroll
   for (int r = 0; r < KW; ++r) {
     const int x = (slice + r) % KW;
@@ -142,7 +162,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int kk0 = ks * X::KM + q4 * KE;
-        rtf[r][u][ks] = load_frag_at<T>(row + (kk0 / DL) * D + (kk0 % DL));
+        const Frag f = load_frag_at<T>(row + (kk0 / DL) * D + (kk0 % DL));
+        if (r < KWR) rtf[r < KWR ? r : 0][u][ks] = f;
+        else rl[(((r - KWR) * UTW + u) * KS + ks) * 64] = f;
       }
     }
   }
@@ -294,6 +316,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     Frag gq[2][KC];
 #pragma unroll
     for (int k = 0; k < KC; ++k) gq[0][k] = gf[k * 64];
+    Frag la_next[RLD > 0 ? RLD : 1][UTW];
+    if constexpr (RLD > 0) {
+#pragma unroll
+      for (int rr = 0; rr < RLD; ++rr)
+#pragma unroll
+        for (int u = 0; u < UTW; ++u) la_next[rr][u] = rl[((rr * UTW + u) * KS) * 64];
+    }
     // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -306,11 +335,27 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
       for (int k = 0; k < KC; ++k) {
         const int ks = kc * KC + k, j = ks % NACC;
+        // fragments kept in LDS: those of the next k-step are requested before this one's MFMAs
+        Frag la[RLD > 0 ? RLD : 1][UTW];
+        if constexpr (RLD > 0) {
+#pragma unroll
+          for (int rr = 0; rr < RLD; ++rr)
+#pragma unroll
+            for (int u = 0; u < UTW; ++u) la[rr][u] = la_next[rr][u];
+          if (ks + 1 < KS) {
+#pragma unroll
+            for (int rr = 0; rr < RLD; ++rr)
+#pragma unroll
+              for (int u = 0; u < UTW; ++u) la_next[rr][u] = rl[((rr * UTW + u) * KS + ks + 1) * 64];
+          }
+          __builtin_amdgcn_sched_barrier(0);
+        }
 #pragma unroll
         for (int r = OWN_LAST ? 1 : 0; r < KW; ++r)
 #pragma unroll
           for (int u = 0; u < UTW; ++u)
-            accp[j][r][u] = X::mfma(rtf[r][u][ks], gq[kc & 1][k], ks < NACC ? f32x4{0.f, 0.f, 0.f, 0.f} : accp[j][r][u]);
+            accp[j][r][u] = X::mfma(r < KWR ? rtf[r < KWR ? r : 0][u][ks] : la[r < KWR ? 0 : r - KWR][u], gq[kc & 1][k],
+                                    ks < NACC ? f32x4{0.f, 0.f, 0.f, 0.f} : accp[j][r][u]);
         if (j == NACC - 1) __builtin_amdgcn_sched_barrier(0);
       }
     }

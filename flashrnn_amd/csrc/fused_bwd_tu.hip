@@ -8,7 +8,7 @@ namespace frnn {
 template <>
 int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
-  const size_t lds = (size_t)2 * 16 * Cell<FRNN_F>::GR * (p.D / p.kw) * sizeof(FRNN_TU_T) + 16;
+  const size_t lds = bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T)) + 16;
 #define FRNN_CASE(Dv, VAR, W, U, K)                                                                     \
   if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                            \
     auto kern = a.tile_rows == 4 ? fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4>                   \

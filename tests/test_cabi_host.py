@@ -51,6 +51,8 @@ def test_supported_table(lib):
     for f in (L, S, G, E):
         for D in (32, 64, 96, 128, 192, 256, 384, 512):
             assert lib.frnn_fused_supported(f, 0, 8, 3, D) == 0, (f, D)
+    for f in (L, S, G, E):
+        assert lib.frnn_fused_supported(f, 0, 8, 1, 768) == 0, f
     assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == _lib.E_UNSUPPORTED  # too large to keep on chip
     assert lib.frnn_fused_supported(L, 1, 8, 1, 512) == _lib.E_UNSUPPORTED   # fp32 R is twice the size

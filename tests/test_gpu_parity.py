@@ -41,6 +41,11 @@ FUSED_SMALL = [
     ("gru", 6, 5, 1, 384, "bfloat16"),
     ("slstm", 5, 6, 1, 384, "bfloat16"),
     ("elman", 12, 6, 1, 384, "bfloat16"),    # 3 workgroups of 8 waves
+    ("lstm", 6, 7, 1, 768, "bfloat16"),      # 12 workgroups per head; backward keeps part of R^T in LDS
+    ("gru", 9, 5, 1, 768, "bfloat16"),
+    ("slstm", 5, 6, 1, 768, "bfloat16"),
+    ("lstm", 17, 4, 1, 768, "float16"),
+    ("elman", 11, 6, 1, 768, "bfloat16"),
 ]
 
 
