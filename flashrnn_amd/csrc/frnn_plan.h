@@ -36,10 +36,10 @@ struct Plan { int D, variant, waves, utw, kw; };
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8) X(768, 0, 4, 1, 12)
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8) X(768, 0, 4, 1, 12) X(1024, 0, 4, 1, 16)
 #define FRNN_BWD_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8) X(768, 0, 4, 1, 12)
+  X(256, 0, 4, 1, 4) X(384, 0, 4, 1, 6) X(512, 0, 4, 1, 8) X(768, 0, 4, 1, 12) X(1024, 0, 4, 1, 16)
 #define FRNN_PLANS_GR3_F32(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
 #define FRNN_BWD_PLANS_GR3_F32 FRNN_PLANS_GR3_F32

@@ -53,7 +53,7 @@ def test_supported_table(lib):
             assert lib.frnn_fused_supported(f, 0, 8, 3, D) == 0, (f, D)
     for f in (L, S, G, E):
         assert lib.frnn_fused_supported(f, 0, 8, 1, 768) == 0, f
-    assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0
+    assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0 and lib.frnn_fused_supported(G, 0, 32, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == _lib.E_UNSUPPORTED  # too large to keep on chip
     assert lib.frnn_fused_supported(L, 1, 8, 1, 512) == _lib.E_UNSUPPORTED   # fp32 R is twice the size
     assert lib.frnn_fused_supported(L, 1, 8, 1, 96) == 0 and lib.frnn_fused_supported(L, 1, 8, 1, 384) == _lib.E_UNSUPPORTED

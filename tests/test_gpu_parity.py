@@ -46,6 +46,7 @@ FUSED_SMALL = [
     ("slstm", 5, 6, 1, 768, "bfloat16"),
     ("lstm", 17, 4, 1, 768, "float16"),
     ("elman", 11, 6, 1, 768, "bfloat16"),
+    ("gru", 7, 5, 1, 1024, "bfloat16"),      # 16 workgroups per head
 ]
 
 
