@@ -240,5 +240,31 @@ def flashrnn(
     if tuple(states.shape) != (S, B, 1, N, D):
         raise ValueError(f"states must be [{S},{B},1,{N},{D}], got {tuple(states.shape)}")
     training = torch.is_grad_enabled() and any(x.requires_grad for x in (Wx, R, b, states))
-    out = _FlashRNNFunction.apply(Wx, R, b, states, config, training)
+    if D == 16:
+        out = _paired_heads(Wx, R, b, states, config, training)
+    else:
+        out = _FlashRNNFunction.apply(Wx, R, b, states, config, training)
     return out, out[:, :, -1:]
+
+
+def _paired_heads(Wx, R, b, states, config, training):
+    """Head dimension 16 (half a bf16 MFMA k-step; the reference's benchmark sweep has it): two heads
+    run as one head of 32 units whose recurrent matrix is block diagonal, so a unit still sees only the
+    h of its own head.  Wx, b and the states are views (adjacent heads are adjacent in memory); only
+    the small R is rebuilt, with differentiable ops, so its gradient arrives by autograd."""
+    B, T, Gw, N, D = Wx.shape
+    if N % 2:  # one all-zero head completes the last pair; its outputs are dropped
+        pad = lambda x: torch.nn.functional.pad(x, (0, 0, 0, 1))
+        Wx, b, states = pad(Wx), pad(b), pad(states)
+        R = torch.nn.functional.pad(R, (0, 0, 0, 0, 0, 1))
+    M = (N + 1) // 2
+    Gr = R.shape[0]
+    Rp = R.reshape(Gr, M, 2, 16, 16)
+    R2 = torch.cat([torch.cat([Rp[:, :, 0], torch.zeros_like(Rp[:, :, 0])], -1),
+                    torch.cat([torch.zeros_like(Rp[:, :, 1]), Rp[:, :, 1]], -1)], -2)
+    cfg2 = FlashRNNConfig(**{**{k: getattr(config, k) for k in ("function", "backend", "dtype", "forward_clipval",
+                                                                "gradient_recurrent_clipval", "gradient_recurrent_cut")},
+                             "head_dim": 32, "num_heads": M, "batch_size": B})
+    out = _FlashRNNFunction.apply(Wx.reshape(B, T, Gw, M, 32), R2, b.reshape(b.shape[0], M, 32),
+                                  states.reshape(states.shape[0], B, 1, M, 32), cfg2, training)
+    return out.reshape(out.shape[0], B, T, 2 * M, 16)[:, :, :, :N]

@@ -50,6 +50,18 @@ FUSED_SMALL = [
 ]
 
 
+@pytest.mark.parametrize("function,N,dtype,backend", [
+    ("lstm", 4, "bfloat16", "hip_fused"), ("lstm", 3, "float32", "hip_fused"), ("gru", 5, "bfloat16", "hip_fused"),
+    ("slstm", 2, "bfloat16", "hip_fused"), ("elman", 7, "float16", "hip_fused"), ("lstm", 3, "bfloat16", "hip"),
+])
+def test_head_dim_16_runs_as_paired_heads(gpu, function, N, dtype, backend):
+    """D = 16 (in the reference's benchmark sweep) is half a bf16 MFMA k-step: flashrnn() runs two heads
+    as one head of 32 units with a block-diagonal R; outputs and all gradients, dR included, must match
+    the oracle, which computes the heads separately."""
+    print(f"case paired heads {function} N{N} {dtype} {backend}", flush=True)
+    check_case(gpu, function, 6, 7, N, 16, dtype, backend, seed=23, init="randn")
+
+
 @pytest.mark.parametrize("function,B,T,N,D,dtype", FUSED_SMALL)
 @pytest.mark.parametrize("init", ["zeros", "randn"])
 def test_fused_matches_oracle(gpu, function, B, T, N, D, dtype, init):
