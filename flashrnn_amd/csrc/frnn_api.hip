@@ -117,6 +117,7 @@ static int fwd_poll_delay_default(int function, const Plan& p) {
   if (function == FRNN_ELMAN) return p.waves > 4 ? 12 : 6;
   if (p.kw == 3) return 2;
   if (p.kw == 6 || p.kw == 12) return 6;
+  if (p.kw == 10) return 5;
   if (p.kw >= 16) return 8;
   if (p.kw == 4 && function == FRNN_GRU) return 5;
   return 3;
@@ -471,7 +472,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   // measured best, as in the forward call; the cells with several dWx stores issue them between
   // the send and the first probe, which is part of their delay
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", function == FRNN_ELMAN ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
-                                                                        : (p.kw >= 12 ? 8 : 4));
+                                                                        : (p.kw >= 10 ? 8 : 4));
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

@@ -58,13 +58,13 @@ constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) *
 
 // Resident operand of the reverse product: a wave holds KW*UTW*KS fragments of the transposed R (all
 // destination tiles at its position, its workgroup's gate rows).  At 4 waves per workgroup a wave has
-// 512 registers; when the fragments alone would take more than 320 of them (LSTM D = 768: 384), those
+// 512 registers; when the fragments alone would take more than 288 of them (LSTM D = 768: 384), those
 // of the last RLD destination tiles (as many as bring the rest down to 256) live in LDS instead (the reverse kernel needs little LDS otherwise)
 // and are read back, one k-step ahead, as the A operand of their MFMAs.
 constexpr int bwd_lds_tiles(int GR, int D, int WAVES, int UTW, int KW, int esize) {
   const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4;
   const int KS = GR * (D / KW) / KM, regs = KW * UTW * KS * FR, per = UTW * KS * FR;
-  return (WAVES == 4 && regs > 320) ? (regs - 256 + per - 1) / per : 0;
+  return (WAVES == 4 && regs > 288) ? (regs - 256 + per - 1) / per : 0;
 }
 constexpr size_t bwd_lds_bytes(int GR, int D, int WAVES, int UTW, int KW, int esize) {
   const int KM = esize == 4 ? 4 : 32, FRB = esize == 4 ? 4 : 16;

@@ -49,7 +49,7 @@ def test_function_dims_mirror_the_registry(lib):
 def test_supported_table(lib):
     L, S, G, E = (_lib.FUNCTION_IDS[k] for k in ("lstm", "slstm", "gru", "elman"))
     for f in (L, S, G, E):
-        for D in (32, 64, 96, 128, 192, 256, 384, 512):
+        for D in (32, 64, 96, 128, 160, 192, 256, 320, 384, 448, 512, 640):
             assert lib.frnn_fused_supported(f, 0, 8, 3, D) == 0, (f, D)
     for f in (L, S, G, E):
         assert lib.frnn_fused_supported(f, 0, 8, 1, 768) == 0, f

@@ -47,6 +47,17 @@ FUSED_SMALL = [
     ("lstm", 17, 4, 1, 768, "float16"),
     ("elman", 11, 6, 1, 768, "bfloat16"),
     ("gru", 7, 5, 1, 1024, "bfloat16"),      # 16 workgroups per head
+    ("lstm", 6, 5, 2, 160, "bfloat16"),      # 10 waves
+    ("slstm", 9, 6, 1, 160, "bfloat16"),
+    ("gru", 5, 7, 1, 320, "bfloat16"),       # 5 workgroups per head
+    ("lstm", 10, 6, 1, 320, "float16"),
+    ("elman", 7, 5, 2, 320, "bfloat16"),
+    ("lstm", 5, 6, 1, 448, "bfloat16"),      # 7 workgroups per head
+    ("elman", 9, 5, 1, 448, "bfloat16"),
+    ("lstm", 7, 5, 1, 640, "bfloat16"),      # 10 workgroups per head
+    ("slstm", 4, 6, 1, 640, "bfloat16"),
+    ("gru", 6, 4, 1, 640, "bfloat16"),
+    ("elman", 12, 5, 1, 640, "bfloat16"),
 ]
 
 
