@@ -110,7 +110,7 @@ static int env_int(const char* name, int dflt) {
 // the data arrives depends on how long the other workgroups' gate math and stores take, so the best
 // value differs by cell and tiling.  Measured on MI355X (bf16, T = 1024; a unit off costs 1-3 %):
 //   lstm  D=256 (4 workgroups) 3, D=384 (6) 6, D=512 (8) 3;  gru D=256 5;  slstm D=192 (3) 2;
-//   lstm D=768 (12 workgroups) 6;  gru D=1024 (16 workgroups) 8;
+//   lstm D=320 (5) 3, D=448 (7) 3, D=640 (10) 5, D=768 (12) 6;  gru D=1024 (16 workgroups) 8;
 //   elman D=512 (4 workgroups, 2 tiles per wave) 6, D=1024 (8 workgroups of 8 waves) 12.
 static int fwd_poll_delay_default(int function, const Plan& p) {
   if (p.kw <= 1) return 0;
