@@ -118,7 +118,7 @@ static int fwd_poll_delay_default(int function, const Plan& p) {
   if (p.kw == 3) return 2;
   if (p.kw == 6 || p.kw == 12) return 6;
   if (p.kw == 10) return 5;
-  if (p.kw >= 16) return 8;
+  if (p.kw >= 16) return 8;  // (lstm D=1024, 32 workgroups of 2 waves: 8 as well)
   if (p.kw == 4 && function == FRNN_GRU) return 5;
   return 3;
 }

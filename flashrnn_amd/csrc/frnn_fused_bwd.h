@@ -64,7 +64,12 @@ constexpr size_t bwd_inbox_words(int D, int KW) { return (size_t)KW * (D / 16) *
 constexpr int bwd_lds_tiles(int GR, int D, int WAVES, int UTW, int KW, int esize) {
   const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4;
   const int KS = GR * (D / KW) / KM, regs = KW * UTW * KS * FR, per = UTW * KS * FR;
-  return (WAVES == 4 && regs > 288) ? (regs - 256 + per - 1) / per : 0;
+  if (!(WAVES <= 4 && regs > 288)) return 0;
+  const int want = (regs - 256 + per - 1) / per;
+  // what fits: 160 KB of LDS minus the two dg buffers and some slack
+  const int FRB = esize == 4 ? 4 : 16;
+  const int room = (160 * 1024 - 2 * 16 * GR * (D / KW) * esize - 2048) / (WAVES * UTW * KS * 64 * FRB);
+  return want < room ? want : room;
 }
 constexpr size_t bwd_lds_bytes(int GR, int D, int WAVES, int UTW, int KW, int esize) {
   const int KM = esize == 4 ? 4 : 32, FRB = esize == 4 ? 4 : 16;

@@ -41,6 +41,19 @@ struct FwdArgs {
 #define FRNN_STAMP(var)
 #endif
 
+// Resident operand of the forward product: a wave holds UTW*G_r*KS fragments of R.  When they alone
+// would take more than 400 of the 512 registers a wave has at one wave per SIMD (LSTM D = 1024: all
+// 512), those of the last RLK k-steps live in LDS instead (as many as bring the rest down to 352, and
+// as fit beside the two h buffers) and are read back one k-step ahead as the A operand of their MFMAs.
+constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
+  const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4, FRB = esize == 4 ? 4 : 16;
+  const int KS = D / KM, per = UTW * GR * FR, regs = per * KS;
+  if (!(WAVES <= 4 && regs > 400)) return 0;
+  const int want = (regs - 352 + per - 1) / per;
+  const int room = (160 * 1024 - 2 * 16 * D * esize - 1024) / (WAVES * UTW * GR * 64 * FRB);
+  return want < room ? want : room;
+}
+
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag(const T* row, int ks, int kq);
 template <> __device__ __forceinline__ bf16x8 load_frag<bf16_t>(const bf16_t* row, int ks, int kq) {
   return *reinterpret_cast<const bf16x8*>(row + ks * 32 + kq * 8);
@@ -78,6 +91,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
   __shared__ int dead_flag;
+  constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
+  // [wave][k-step][u][g][lane]: each lane reads back what it wrote
+  __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -114,14 +130,19 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   }
 
   // ---- resident operands ----------------------------------------------------------------
-  Frag rf[UTW][GR][KS];
+  Frag rf[UTW][GR][KSR];
+  Frag* const rl = rlds + (size_t)w * RLK * UTW * GR * 64 + lane;
 #pragma unroll
   for (int u = 0; u < UTW; ++u)
 #pragma unroll
     for (int g = 0; g < GR; ++g) {
       const T* row = R + ((size_t)(g * N + n) * D + ub[u] + r16) * D;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) rf[u][g][ks] = load_frag<T>(row, ks, q4);
+      for (int ks = 0; ks < KS; ++ks) {
+        const Frag f = load_frag<T>(row, ks, q4);
+        if (ks < KSR) rf[u][g][ks < KSR ? ks : 0] = f;
+        else rl[(((ks - KSR) * UTW + u) * GR + g) * 64] = f;
+      }
     }
   // bias of the recurrent gate slots: as the C operand of the first MFMA when a lane keeps all 4
   // elements of a tile (costs nothing), else added to the lane's own elements in the gate math
@@ -228,6 +249,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     Frag hq[2][KC];
 #pragma unroll
     for (int k = 0; k < KC; ++k) hq[0][k] = hf[k * 64];
+    Frag la_next[UTW][GR];
+    if constexpr (RLK > 0 && KSR == 0) {
+#pragma unroll
+      for (int u = 0; u < UTW; ++u)
+#pragma unroll
+        for (int g = 0; g < GR; ++g) la_next[u][g] = rl[(u * GR + g) * 64];
+    }
     // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
@@ -240,11 +268,28 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int k = 0; k < KC; ++k) {
         const int ks = kc * KC + k, j = ks % NACC;
+        // fragments kept in LDS: those of the next k-step are requested before this one's MFMAs
+        Frag la[UTW][GR];
+        if constexpr (RLK > 0) {
+          if (ks >= KSR) {
+#pragma unroll
+            for (int u = 0; u < UTW; ++u)
+#pragma unroll
+              for (int g = 0; g < GR; ++g) la[u][g] = la_next[u][g];
+          }
+          if (ks + 1 >= KSR && ks + 1 < KS) {
+#pragma unroll
+            for (int u = 0; u < UTW; ++u)
+#pragma unroll
+              for (int g = 0; g < GR; ++g) la_next[u][g] = rl[(((ks + 1 - KSR) * UTW + u) * GR + g) * 64];
+            __builtin_amdgcn_sched_barrier(0);
+          }
+        }
 #pragma unroll
         for (int u = 0; u < UTW; ++u)
 #pragma unroll
           for (int g = 0; g < GR; ++g)
-            accp[j][u][g] = X::mfma(rf[u][g][ks], hq[kc & 1][k],
+            accp[j][u][g] = X::mfma(ks < KSR ? rf[u][g][ks < KSR ? ks : 0] : la[u][g], hq[kc & 1][k],
                                     ks < NACC ? ((BIAS_C && ks == 0) ? biasc[u][g] : f32x4{0.f, 0.f, 0.f, 0.f}) : accp[j][u][g]);
         // group by group: consecutive MFMAs then never depend on each other
         if (j == NACC - 1) __builtin_amdgcn_sched_barrier(0);

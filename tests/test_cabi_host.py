@@ -54,7 +54,8 @@ def test_supported_table(lib):
     for f in (L, S, G, E):
         assert lib.frnn_fused_supported(f, 0, 8, 1, 768) == 0, f
     assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0 and lib.frnn_fused_supported(G, 0, 32, 1, 1024) == 0
-    assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == _lib.E_UNSUPPORTED  # too large to keep on chip
+    assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == 0
+    assert lib.frnn_fused_supported(L, 0, 8, 1, 2048) == _lib.E_UNSUPPORTED  # too large to keep on chip
     assert lib.frnn_fused_supported(L, 1, 8, 1, 512) == _lib.E_UNSUPPORTED   # fp32 R is twice the size
     assert lib.frnn_fused_supported(L, 1, 8, 1, 96) == 0 and lib.frnn_fused_supported(L, 1, 8, 1, 384) == _lib.E_UNSUPPORTED
     assert lib.frnn_fused_supported(L, 0, 8, 1, 48) == _lib.E_UNSUPPORTED
@@ -81,7 +82,7 @@ def test_plan_and_sizes(lib):
     assert lib.frnn_fused_cache_bytes(_lib.FUNCTION_IDS["elman"], 0, 8, 16, 3, 256) == 0
     assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 256, 0) >= 256
     assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 256, 1) > lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 256, 0)
-    assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 1024, 0) == 0  # unsupported
+    assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 2048, 0) == 0  # unsupported
 
 
 def _fwd(lib, entry, function=0, dtype=0, B=8, T=4, N=1, D=64, Wx=FAKE, R=FAKE, b=FAKE, s0=FAKE, states=FAKE,

@@ -47,6 +47,9 @@ FUSED_SMALL = [
     ("lstm", 17, 4, 1, 768, "float16"),
     ("elman", 11, 6, 1, 768, "bfloat16"),
     ("gru", 7, 5, 1, 1024, "bfloat16"),      # 16 workgroups per head
+    ("lstm", 6, 7, 1, 1024, "bfloat16"),     # 32 workgroups of 2 waves per head; part of R in LDS
+    ("slstm", 5, 5, 1, 1024, "bfloat16"),
+    ("lstm", 18, 4, 1, 1024, "float16"),
     ("lstm", 6, 5, 2, 160, "bfloat16"),      # 10 waves
     ("slstm", 9, 6, 1, 160, "bfloat16"),
     ("gru", 5, 7, 1, 320, "bfloat16"),       # 5 workgroups per head

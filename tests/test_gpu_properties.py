@@ -151,7 +151,7 @@ def test_sequence_longer_than_the_tag_period(gpu):
         assert float(tail.max()) <= 4e-2 * max(1.0, float(a.abs().max())), (name, float(tail.max()))
 
 
-@pytest.mark.parametrize("function,B,T,N,D", [("lstm", 16, 512, 1, 768), ("slstm", 8, 256, 1, 768), ("gru", 8, 256, 1, 1024),
+@pytest.mark.parametrize("function,B,T,N,D", [("lstm", 16, 512, 1, 768), ("slstm", 8, 256, 1, 768), ("gru", 8, 256, 1, 1024), ("lstm", 8, 256, 1, 1024),
                                               ("lstm", 8, 512, 3, 256)])
 def test_fused_and_alternating_gradients_agree(gpu, function, B, T, N, D):
     """Backward of long sequences on the largest tilings (12 and 16 workgroups per head, part of the
