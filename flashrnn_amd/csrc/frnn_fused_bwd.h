@@ -69,6 +69,8 @@ constexpr int bwd_lds_tiles(int GR, int D, int WAVES, int UTW, int KW, int esize
   // what fits: 160 KB of LDS minus the two dg buffers and some slack
   const int FRB = esize == 4 ? 4 : 16;
   const int room = (160 * 1024 - 2 * 16 * GR * (D / KW) * esize - 2048) / (WAVES * UTW * KS * 64 * FRB);
+  // more than 8 remote destinations are processed in groups of 4 (see the kernel): whole groups in LDS
+  if (KW - 1 > 8) return (want + 3) / 4 * 4 < room / 4 * 4 ? (want + 3) / 4 * 4 : room / 4 * 4;
   return want < room ? want : room;
 }
 constexpr size_t bwd_lds_bytes(int GR, int D, int WAVES, int UTW, int KW, int esize) {
@@ -314,7 +316,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     // and are sent at once; the product for the own tiles follows while those words travel (it
     // needs all fragments still in registers: one chunk)
     constexpr bool OWN_LAST = KW >= 3 && KS == chunk_of(KS);
-    f32x4 accp[NACC][KW][UTW];
+    // More than 8 remote destinations (10 and more workgroups per head): their products run in groups
+    // of 4 destinations (4 independent MFMA chains), each group sent as soon as it is complete, so that
+    // 16 accumulator registers are live instead of 4 per destination (128 at 32 workgroups per head).
+    constexpr bool GROUPED = OWN_LAST && KW - 1 > 8;
+    constexpr int RI = 4;
+    static_assert(!GROUPED || RLD % RI == 0, "LDS-resident destinations come in whole groups");
+    f32x4 accp[NACC][GROUPED ? 1 : KW][UTW];
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;
     constexpr int KC = chunk_of(KS);
     static_assert(KS % KC == 0, "k-steps must split into whole chunks");
@@ -322,7 +330,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
     for (int k = 0; k < KC; ++k) gq[0][k] = gf[k * 64];
     Frag la_next[RLD > 0 ? RLD : 1][UTW];
-    if constexpr (RLD > 0) {
+    if constexpr (RLD > 0 && !GROUPED) {
 #pragma unroll
       for (int rr = 0; rr < RLD; ++rr)
 #pragma unroll
@@ -330,8 +338,75 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     }
     // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
     __builtin_amdgcn_sched_barrier(0);
+    if constexpr (GROUPED) {
+      IW* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
+      auto send_group = [&](int r0, int nr, f32x4 (&ag)[RI][UTW]) __attribute__((always_inline)) {
 #pragma unroll
-    for (int kc = 0; kc < KS / KC; ++kc) {
+        for (int rr = 0; rr < RI; ++rr) {
+          if (rr >= nr) continue;
+          const int x = (slice + r0 + rr) % KW;
+#pragma unroll
+          for (int u = 0; u < UTW; ++u) {
+            float part[E];
+            own_elems<TR>(ag[rr][u], part);
+            IW* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
+#pragma unroll
+            for (int e = 0; e < E; ++e) ll_store(dst + e * 64, part_pack((PT*)0, part[e], t));
+          }
+        }
+      };
+      // destinations whose fragments are in registers
+#pragma unroll
+      for (int r0 = 1; r0 < KWR; r0 += RI) {
+        const int nr = KWR - r0 < RI ? KWR - r0 : RI;
+        f32x4 ag[RI][UTW];
+#pragma unroll
+        for (int ks = 0; ks < KS; ++ks) {
+#pragma unroll
+          for (int rr = 0; rr < RI; ++rr)
+#pragma unroll
+            for (int u = 0; u < UTW; ++u)
+              if (rr < nr) ag[rr][u] = X::mfma(rtf[r0 + rr < KWR ? r0 + rr : 0][u][ks], gq[0][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : ag[rr][u]);
+          __builtin_amdgcn_sched_barrier(0);
+        }
+        send_group(r0, nr, ag);
+      }
+      // destinations whose fragments are in LDS: those of the next (group, k-step) are requested before
+      // the MFMAs of the current one
+      if constexpr (RLD > 0) {
+        Frag lb[2][RI][UTW];
+#pragma unroll
+        for (int rr = 0; rr < RI; ++rr)
+#pragma unroll
+          for (int u = 0; u < UTW; ++u) lb[0][rr][u] = rl[((rr * UTW + u) * KS) * 64];
+        __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+        for (int gi = 0; gi < RLD / RI; ++gi) {
+          f32x4 ag[RI][UTW];
+#pragma unroll
+          for (int ks = 0; ks < KS; ++ks) {
+            const int m = gi * KS + ks, mn = m + 1;
+            if (mn < (RLD / RI) * KS) {
+              const int gn = mn / KS, kn = mn % KS;
+#pragma unroll
+              for (int rr = 0; rr < RI; ++rr)
+#pragma unroll
+                for (int u = 0; u < UTW; ++u) lb[mn & 1][rr][u] = rl[(((gn * RI + rr) * UTW + u) * KS + kn) * 64];
+              __builtin_amdgcn_sched_barrier(0);
+            }
+#pragma unroll
+            for (int rr = 0; rr < RI; ++rr)
+#pragma unroll
+              for (int u = 0; u < UTW; ++u)
+                ag[rr][u] = X::mfma(lb[m & 1][rr][u], gq[0][ks], ks == 0 ? f32x4{0.f, 0.f, 0.f, 0.f} : ag[rr][u]);
+            __builtin_amdgcn_sched_barrier(0);
+          }
+          send_group(KWR + gi * RI, RI, ag);
+        }
+      }
+    }
+#pragma unroll
+    for (int kc = 0; kc < (GROUPED ? 0 : KS / KC); ++kc) {
       if (kc + 1 < KS / KC) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) gq[(kc + 1) & 1][k] = gf[((kc + 1) * KC + k) * 64];
@@ -365,9 +440,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
     }
     static_assert(NACC == 1, "one accumulator per tile");
-    f32x4 acc[KW][UTW];
+    f32x4 acc[GROUPED ? 1 : KW][UTW];
 #pragma unroll
-    for (int r = OWN_LAST ? 1 : 0; r < KW; ++r)
+    for (int r = OWN_LAST ? 1 : 0; r < (GROUPED ? 0 : KW); ++r)
 #pragma unroll
       for (int u = 0; u < UTW; ++u) acc[r][u] = accp[0][r][u];
     if constexpr (!OWN_LAST) {
@@ -391,7 +466,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
       IW* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
 #pragma unroll
-      for (int r = 1; r < KW; ++r) {
+      for (int r = 1; r < (GROUPED ? 0 : KW); ++r) {
         const int x = (slice + r) % KW;
 #pragma unroll
         for (int u = 0; u < UTW; ++u) {
