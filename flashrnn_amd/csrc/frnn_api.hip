@@ -232,7 +232,7 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   w.Rt = bp.take((size_t)N * D * c.GR * D * es);
   w.dgx = bp.take(function == FRNN_GRU ? (size_t)B * T * N * D * es : 0);
   w.dbp = (float*)bp.take(bt * c.GT * N * D * 4);
-  w.splits = grad_gemm_splits(B, T, N, D, c.GR);
+  w.splits = grad_gemm_splits(dtype, B, T, N, D, c.GR);
   w.part = (float*)bp.take((size_t)w.splits * c.GR * N * D * D * 4);
   w.total = bp.off;
   return w;
@@ -524,7 +524,7 @@ AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, i
     const long rows = (long)B * T;
     w.bsplits = rows < 64 ? (int)rows : 64;
     w.dbp = (float*)bp.take((size_t)w.bsplits * c.GT * ND * 4);
-    w.splits = grad_gemm_splits(B, T, N, D, c.GR);
+    w.splits = grad_gemm_splits(dtype, B, T, N, D, c.GR);
     w.part = (float*)bp.take((size_t)w.splits * c.GR * ND * D * 4);
   }
   w.total = bp.off;

@@ -16,7 +16,7 @@ struct GradGemmArgs {
 };
 
 int launch_transpose_r(int dtype, const void* R, void* Rt, int N, int D, int GR, hipStream_t st);
-int grad_gemm_splits(int B, int T, int N, int D, int GR);
+int grad_gemm_splits(int dtype, int B, int T, int N, int D, int GR);
 int launch_grad_gemm(int dtype, GradGemmArgs a, int splits, hipStream_t st);
 int launch_grad_reduce(const float* part_r, int splits_r, size_t n_r, float* dR,
                        const float* part_b, int splits_b, size_t n_b, float* db, hipStream_t st);
