@@ -32,8 +32,8 @@ PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, publi
 # two `rocprofv3 --pmc` runs of this script; summary and commands in
 # profiles/fused_kernels_lstm_bf16_B8_T1024_N3_D256_hbm_traffic.txt.  Workloads not profiled: null.
 TRAFFIC_BYTES = {
-    ("C2", "fused_fwd_kernel"): (38976.3 + 98304.0) * 1024,
-    ("C2", "fused_bwd_kernel"): (81961.4 + 122928.0) * 1024,
+    ("C2", "fused_fwd_kernel"): (38977.1 + 98304.0) * 1024,
+    ("C2", "fused_bwd_kernel"): (81939.2 + 122928.0) * 1024,
 }
 
 
