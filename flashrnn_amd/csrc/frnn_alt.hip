@@ -244,18 +244,32 @@ struct AltBiasArgs {
   float* part;                     // [splits][G_t][N][D]
   int GT, N, D; long rows, rows_per_split;
 };
+// one thread sums 4 adjacent columns (one 8- or 16-byte load per row) over the rows of its split
 template <typename T>
 __global__ void __launch_bounds__(256) alt_bias_kernel(const AltBiasArgs a) {
-  const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
+  const size_t i4 = (size_t)blockIdx.x * 256 + threadIdx.x;
   const size_t nb = (size_t)a.GT * a.N * a.D;
-  if (i >= nb) return;
+  if (i4 * 4 >= nb) return;
+  const size_t i = i4 * 4;
   const int g = i / ((size_t)a.N * a.D);
   const size_t nd = i % ((size_t)a.N * a.D);
   const T* p = static_cast<const T*>(a.src[g]) + nd;
   const long r0 = (long)blockIdx.y * a.rows_per_split, r1 = min(a.rows, r0 + a.rows_per_split);
-  float s = 0.f;
-  for (long r = r0; r < r1; ++r) s += ld(p + (size_t)r * a.ld[g]);
-  a.part[(size_t)blockIdx.y * nb + i] = s;
+  float s[4] = {0.f, 0.f, 0.f, 0.f};
+  for (long r = r0; r < r1; ++r) {
+    float v[4];
+    if constexpr (sizeof(T) == 2) {
+      const uint2 w = *reinterpret_cast<const uint2*>(p + (size_t)r * a.ld[g]);
+      Dw<2> d; d.v[0] = w.x; d.v[1] = w.y;
+      unpack<4>(d, v, (T*)nullptr);
+    } else {
+      const float4 w = *reinterpret_cast<const float4*>(p + (size_t)r * a.ld[g]);
+      v[0] = w.x; v[1] = w.y; v[2] = w.z; v[3] = w.w;
+    }
+#pragma unroll
+    for (int e = 0; e < 4; ++e) s[e] += v[e];
+  }
+  *reinterpret_cast<float4*>(a.part + (size_t)blockIdx.y * nb + i) = make_float4(s[0], s[1], s[2], s[3]);
 }
 
 // ---------------------------------------------------------------------------------------------
@@ -317,7 +331,7 @@ int launch_bias_partial(int dtype, const void* const* src, const long* ld, int G
   AltBiasArgs a;
   for (int g = 0; g < 4; ++g) { a.src[g] = g < GT ? src[g] : nullptr; a.ld[g] = g < GT ? ld[g] : 0; }
   a.part = part; a.GT = GT; a.N = N; a.D = D; a.rows = rows; a.rows_per_split = (rows + splits - 1) / splits;
-  const dim3 grid((unsigned)(((size_t)GT * N * D + 255) / 256), splits);
+  const dim3 grid((unsigned)(((size_t)GT * N * D / 4 + 255) / 256), splits);  // D is a multiple of 16
   if (dtype == FRNN_BF16) hipLaunchKernelGGL(alt_bias_kernel<bf16_t>, grid, dim3(256), 0, st, a);
   else if (dtype == FRNN_F16) hipLaunchKernelGGL(alt_bias_kernel<half_t>, grid, dim3(256), 0, st, a);
   else hipLaunchKernelGGL(alt_bias_kernel<float>, grid, dim3(256), 0, st, a);

@@ -524,7 +524,7 @@ AltWs carve_alt(void* ws, int function, int dtype, int B, int T, int N, int D, i
     w.dg = bp.take(2 * BND * c.GR * es);
     w.dsr = (float*)bp.take((size_t)c.S * BND * 4);
     const long rows = (long)B * T;
-    w.bsplits = rows < 64 ? (int)rows : 64;
+    w.bsplits = rows < 256 ? (int)rows : 256;
     w.dbp = (float*)bp.take((size_t)w.bsplits * c.GT * ND * 4);
     w.splits = grad_gemm_splits(dtype, B, T, N, D, c.GR);
     w.part = (float*)bp.take((size_t)w.splits * c.GR * ND * D * 4);

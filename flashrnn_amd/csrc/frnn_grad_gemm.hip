@@ -316,11 +316,13 @@ __global__ void __launch_bounds__(256) grad_reduce_kernel(const float* __restric
   const size_t i = (size_t)blockIdx.x * 256 + threadIdx.x;
   if (i < n_r) {
     float s = 0.f;
+#pragma unroll 16
     for (int k = 0; k < splits_r; ++k) s += part_r[(size_t)k * n_r + i];
     dR[i] = s;
   } else if (i - n_r < n_b) {
     const size_t j = i - n_r;
     float s = 0.f;
+#pragma unroll 16
     for (int k = 0; k < splits_b; ++k) s += part_b[(size_t)k * n_b + j];
     db[j] = s;
   }
