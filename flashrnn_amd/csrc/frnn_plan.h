@@ -31,8 +31,9 @@ struct Plan { int D, variant, waves, utw, kw; };
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 4, 1, 3) \
   X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 2, 1, 32)
 #define FRNN_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
-#define FRNN_BWD_PLANS_GR4_F32 FRNN_PLANS_GR4_F32
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+#define FRNN_BWD_PLANS_GR4_F32(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
@@ -41,8 +42,9 @@ struct Plan { int D, variant, waves, utw, kw; };
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
   X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 4, 1, 16)
 #define FRNN_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
-#define FRNN_BWD_PLANS_GR3_F32 FRNN_PLANS_GR3_F32
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+#define FRNN_BWD_PLANS_GR3_F32(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
