@@ -176,20 +176,22 @@ def test_config2_alternating_full_size(gpu):
     check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", "hip", seed=1002, init="randn")
 
 
-def test_config3_gru_bf16_quarter_length(gpu):
-    print("case C3 T=512", flush=True)
-    check_case(gpu, "gru", 16, 512, 4, 128, "bfloat16", "hip_fused", seed=1003, init="zeros")
+@pytest.mark.parametrize("backend", ["hip_fused", "hip"])
+def test_config3_gru_bf16_full_size(gpu, backend):
+    print(f"case C3 full {backend}", flush=True)
+    check_case(gpu, "gru", 16, 2048, 4, 128, "bfloat16", backend, seed=1003, init="zeros")
 
 
-def test_config4_slstm_bf16_eighth_length(gpu):
-    print("case C4 T=512", flush=True)
-    check_case(gpu, "slstm", 16, 512, 4, 192, "bfloat16", "hip_fused", seed=1004, init="zeros",
+def test_config4_slstm_bf16_full_size(gpu):
+    print("case C4 full", flush=True)
+    check_case(gpu, "slstm", 16, 4096, 4, 192, "bfloat16", "hip_fused", seed=1004, init="zeros",
                forget_bias_linspace=True)
 
 
-def test_config5_elman_alternating_quarter_length(gpu):
-    print("case C5 T=256", flush=True)
-    check_case(gpu, "elman", 32, 256, 1, 1024, "bfloat16", "hip", seed=1005, init="zeros")
+@pytest.mark.parametrize("backend", ["hip", "hip_fused"])
+def test_config5_elman_full_size(gpu, backend):
+    print(f"case C5 full {backend}", flush=True)
+    check_case(gpu, "elman", 32, 1024, 1, 1024, "bfloat16", backend, seed=1005, init="zeros")
 
 
 @pytest.mark.parametrize("N,D", [(24, 32), (12, 64), (6, 128), (3, 256), (1, 512)])
