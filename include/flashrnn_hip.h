@@ -78,7 +78,8 @@ int frnn_function_dims(int function, int* G_r, int* G_w, int* G_t, int* S, int* 
 int frnn_fused_supported(int function, int dtype, int B, int N, int D);
 
 /* The launch plan: waves per workgroup, 16-unit tiles per wave, workgroups per head and the
- * number of workgroups that do work (= compute units used).  backward = 0/1. */
+ * number of workgroups that do work (= compute units used; heads that run as one workgroup of
+ * up to 4 waves may share a compute unit three at a time).  backward = 0/1. */
 int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
                     int* waves, int* tiles_per_wave, int* wgs_per_head, int* active_wgs);
 
