@@ -1,7 +1,7 @@
 """Shared helpers of the GPU parity tests: run the HIP path and the CPU oracle on the same seeded
 inputs and compare under the stated tolerances.
 
-Tolerances (the bar of the task: 1e-5 relative in fp32; 2e-2 max-abs in bf16 against an fp32 run
+Tolerances (the bar: 1e-5 relative in fp32; 2e-2 max-abs in bf16 against an fp32 run
 of the oracle fed the same bf16-rounded inputs):
   fp32   every output and gradient: max|err| <= 1e-5 * max(1, max|ref|)     (oracle run in fp64)
   bf16   h (state 0):       max|err| <= 2e-2
