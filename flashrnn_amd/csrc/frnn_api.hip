@@ -146,9 +146,12 @@ static int tile_rows_for(int B, int N, int kw, int waves) {
   const int forced = env_int("FRNN_TILE_ROWS", 0);
   if (forced == 4 || forced == 8 || forced == 16) return forced;
   const long room = (long)device_cus() * (kw == 1 && waves <= 4 ? 3 : 1);
-  for (int tr = 4; tr < 16; tr *= 2)
+  // one workgroup of 10 or 12 waves per head: 168 registers per wave, the 16-row variants spill
+  // (LSTM D = 192 B = 1024: 3.6 ms with 16-row tiles, 3.1 with 8-row tiles in two rounds)
+  const int largest = kw == 1 && waves > 8 ? 8 : 16;
+  for (int tr = 4; tr < largest; tr *= 2)
     if ((long)N * ((B + tr - 1) / tr) * kw <= room) return tr;
-  return 16;
+  return largest;
 }
 
 // Options as the kernels take them: a clip value of 0 switches the clamp off.
