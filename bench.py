@@ -2,6 +2,7 @@
 """Benchmark of the recurrent hot path on one MI355X.
 
     python bench.py [--gpus 1] [--steps K] [--warmup W] [--workload C2] [--backend hip_fused]
+    python bench.py --shape lstm:bfloat16:16:1024:1:768 --no-cpu      (any other shape: function:dtype:B:T:N:D)
 
 A step is one forward + backward pass of ``flashrnn()`` over one batch of synthetic input that is
 already resident in HBM.  Prints ONE JSON line: tokens/s (B*T per second) of the whole job, the
@@ -150,6 +151,8 @@ def main():
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
     ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--shape", default=None, help="function:dtype:B:T:N:D, e.g. lstm:bfloat16:16:1024:1:768 (fwd+bwd, "
+                    "zero initial state, cotangent on every state); replaces --workload")
     ap.add_argument("--backend", default=None, choices=["hip_fused", "hip"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-alt", action="store_true", help="skip the other-backend comparison leg")
@@ -165,6 +168,11 @@ def main():
         print("bench.py needs a GPU (flashrnn_amd has no CPU path)", file=sys.stderr)
         sys.exit(2)
     device = torch.device("cuda:0")
+    if args.shape:
+        f, dt, B, T, N, D = args.shape.split(":")
+        args.workload = "shape " + args.shape
+        WORKLOADS[args.workload] = dict(function=f, dtype=dt, B=int(B), T=int(T), N=int(N), D=int(D), init="zeros",
+                                        grad_on="all", bwd=True, seed=2000)
     w = WORKLOADS[args.workload]
     backend = args.backend or ("hip" if args.workload == "C5" else "hip_fused")
     tokens = w["B"] * w["T"]
