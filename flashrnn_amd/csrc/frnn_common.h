@@ -21,7 +21,7 @@ typedef unsigned long long u64;
 // Cell descriptors.  Gate-slot rule of the reference (flashrnn/flashrnn/flashrnn.py:148-158):
 // R fills the first GR of the GI interacting slots, Wx the last GW, b covers all GT.
 // NC = values cached per element for the backward pass (private layout; LSTM: the four activated
-// gates, GRU: g, r, z and the raw recurrent part of n, sLSTM: i', f', tanh z, sigmoid o, sigmoid(-f)).
+// gates, GRU: g, r, z and the candidate n, sLSTM: i', f', tanh z, sigmoid o, sigmoid(-f)).
 // ---------------------------------------------------------------------------------------
 template <int F> struct Cell;
 template <> struct Cell<FRNN_LSTM>  { static constexpr int GR = 4, GW = 4, GT = 4, S = 2, NC = 4; };

@@ -112,15 +112,14 @@ template <bool FAST> struct CellMath<FRNN_GRU, FAST> {
     const float g = ry[0];
     const float r = M::sigmoid(wx[0] + ry[1]);
     const float z = M::sigmoid(wx[1] + ry[2]);
-    const float nr = wx[2] + b[0];
-    s[0] = z * s[0] + (1.0f - z) * M::tanh(nr + r * g);
-    cache[0] = g; cache[1] = r; cache[2] = z; cache[3] = nr;
+    const float nv = M::tanh(wx[2] + b[0] + r * g);
+    s[0] = z * s[0] + (1.0f - z) * nv;
+    cache[0] = g; cache[1] = r; cache[2] = z; cache[3] = nv;  // the candidate itself: the adjoint needs no tanh
   }
   static __device__ __forceinline__ void bwd(const float* cache, const float* sp, const float* sn, const float* dso,
                                              float* ds, float* dgr, float* dgw, float* dgb) {
-    const float g = cache[0], r = cache[1], z = cache[2], nr = cache[3];
+    const float g = cache[0], r = cache[1], z = cache[2], nv = cache[3];
     const float dy = dso[0] + ds[0];
-    const float nv = M::tanh(nr + r * g);
     const float dz = z * (1.0f - z) * dy * (sp[0] - nv);
     const float dn = dy * (1.0f - z) * (1.0f - nv * nv);
     const float dr = dn * g * r * (1.0f - r);
