@@ -14,7 +14,7 @@ from __future__ import annotations
 
 import os
 from dataclasses import dataclass
-from typing import Optional
+from typing import Optional, Sequence, Union
 
 import torch
 
@@ -57,6 +57,16 @@ class FlashRNNConfig:
     num_gates_i: int = 0
     num_gates_t: int = 0
     simple_agg: bool = True
+    # layouts of the tensors the caller hands over and gets back (flashrnn.py:163-173; B batch, T time,
+    # G gate, H head, D unit, P previous unit, S state).  The kernels read the defaults as they are;
+    # any other layout is permuted on the way in and out (the reference permutes every layout to an
+    # internal one, flashrnn.py:892-924)
+    input_shape: str = "BTGHD"
+    output_shape: str = "SBTHD"
+    recurrent_shape: str = "GHDP"
+    bias_shape: str = "GHD"
+    # value of the default initial state, one number or one per state (flashrnn.py:204, :946-953)
+    initial_val: Union[float, Sequence[float]] = 0.0
 
     def __post_init__(self):
         if self.function not in rnn_function_registry:
@@ -67,6 +77,10 @@ class FlashRNNConfig:
                 "'vanilla' loop is the test oracle and is not part of the package")
         if self.dtype not in DTYPE_DICT:
             raise ValueError(f"dtype {self.dtype} not supported (bfloat16, float16, float32)")
+        for name, canon in (("input_shape", "BTGHD"), ("output_shape", "SBTHD"), ("recurrent_shape", "GHDP"),
+                            ("bias_shape", "GHD")):
+            if sorted(getattr(self, name)) != sorted(canon):
+                raise ValueError(f"{name} must be a permutation of {canon}, got {getattr(self, name)}")
         for name in ("gradient_recurrent_clipval", "forward_clipval"):
             v = getattr(self, name)
             if v is not None and not v > 0:
@@ -204,10 +218,31 @@ def _get_config(Wx, R, b, function, backend, dtype) -> FlashRNNConfig:
                           dtype=dtype if dtype is not None else "bfloat16")
 
 
+def permute_to(input_shape: str, output_shape: str):
+    """Axis permutation that takes a tensor laid out as `input_shape` to `output_shape`, None if they
+    are equal (flashrnn.py:100-110): permute_to("ABC", "BAC") == (1, 0, 2)."""
+    if input_shape == output_shape:
+        return None
+    return tuple(input_shape.index(x) for x in output_shape)
+
+
+def _permuted(x: torch.Tensor, have: str, want: str) -> torch.Tensor:
+    p = permute_to(have, want)
+    return x if p is None else x.permute(p)
+
+
 def _zero_state(config: FlashRNNConfig, Wx: torch.Tensor) -> torch.Tensor:
-    """[S,B,1,N,D] zeros like the reference's _zero_state (flashrnn.py:927-954)."""
+    """Default initial state [S,B,1,N,D] for a Wx in the kernels' layout [B,T,G,N,D]: `initial_val`
+    everywhere, or one value per state (flashrnn.py:927-954)."""
     B, _, _, N, D = Wx.shape
-    return torch.zeros((config.num_states, B, 1, N, D), dtype=Wx.dtype, device=Wx.device)
+    state = torch.zeros((config.num_states, B, 1, N, D), dtype=Wx.dtype, device=Wx.device)
+    if isinstance(config.initial_val, (int, float)):
+        if config.initial_val != 0.0:
+            state += float(config.initial_val)
+    else:
+        for i in range(config.num_states):
+            state[i] += float(config.initial_val[i])
+    return state
 
 
 def flashrnn(
@@ -222,11 +257,19 @@ def flashrnn(
 ):
     """Same call as the reference's ``flashrnn`` (flashrnn.py:1114-1135).
 
-    Returns ``(all_states [S,B,T,N,D], last_states [S,B,1,N,D])`` in the kernel dtype ``dtype``.
+    Returns ``(all_states [S,B,T,N,D], last_states [S,B,1,N,D])`` in the kernel dtype ``dtype``
+    (shapes as named by ``config.input_shape`` / ``output_shape`` / ``recurrent_shape`` / ``bias_shape``
+    when a config with other layouts is given).
     Differentiable w.r.t. Wx, R, b and states.  Raises ValueError if the chosen backend has no
     kernel for the head dimension (as the reference does when no tiling exists)."""
     if config is None:
         config = _get_config(Wx, R, b, function, backend, dtype)
+    # to the layouts the kernels read (views; nothing is copied for the default layouts)
+    Wx = _permuted(Wx, config.input_shape, "BTGHD")
+    R = _permuted(R, config.recurrent_shape, "GHDP")
+    b = _permuted(b, config.bias_shape, "GHD")
+    if states is not None:
+        states = _permuted(states, config.output_shape, "SBTHD")
     Gr, Gw, _, Gt, S = rnn_function_registry[config.function]["gates_states"]
     if Wx.dim() != 5 or Wx.shape[2] != Gw:
         raise ValueError(f"Wx must be [B,T,{Gw},N,D], got {tuple(Wx.shape)}")
@@ -244,7 +287,7 @@ def flashrnn(
         out = _paired_heads(Wx, R, b, states, config, training)
     else:
         out = _FlashRNNFunction.apply(Wx, R, b, states, config, training)
-    return out, out[:, :, -1:]
+    return _permuted(out, "SBTHD", config.output_shape), _permuted(out[:, :, -1:], "SBTHD", config.output_shape)
 
 
 def _paired_heads(Wx, R, b, states, config, training):

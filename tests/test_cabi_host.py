@@ -183,3 +183,29 @@ def test_options_are_validated_before_launch(lib):
         o = _lib.Options(0.0, -2.0, 0)
         assert getattr(lib, entry)(0, 0, 8, 4, 1, 64, *([FAKE] * 11), 0, None, ctypes.byref(o)) == _lib.E_ARG
         assert getattr(lib, entry)(0, 0, 8, 4, 1, 64, *([FAKE] * 11), 0, None, None) == _lib.E_WORKSPACE
+
+
+def test_layout_options_and_initial_state():
+    """The reference's public layout options (flashrnn.py:163-173, permute_to :100-110) and the default
+    initial state with `initial_val` (:927-954), checked on CPU tensors (no kernel involved)."""
+    from flashrnn_amd.flashrnn import _permuted, _zero_state, permute_to
+
+    assert permute_to("ABC", "BAC") == (1, 0, 2) and permute_to("GHD", "GHD") is None
+    cfg = FlashRNNConfig(function="slstm", head_dim=4, num_heads=2, input_shape="TBGHD", output_shape="STBHD",
+                         recurrent_shape="HPGD", bias_shape="HDG", initial_val=[0.0, 1.0, 2.0, 3.0])
+    Wx = torch.arange(5 * 3 * 4 * 2 * 4, dtype=torch.float32).reshape(5, 3, 4, 2, 4)      # T B G H D
+    x = _permuted(Wx, cfg.input_shape, "BTGHD")
+    assert x.shape == (3, 5, 4, 2, 4) and x[1, 2, 3, 1, 0] == Wx[2, 1, 3, 1, 0]
+    R = torch.arange(2 * 4 * 4 * 4, dtype=torch.float32).reshape(2, 4, 4, 4)               # H P G D
+    r = _permuted(R, cfg.recurrent_shape, "GHDP")
+    assert r.shape == (4, 2, 4, 4) and r[3, 1, 2, 0] == R[1, 0, 3, 2]
+    z = _zero_state(cfg, x)
+    assert z.shape == (4, 3, 1, 2, 4) and [float(z[k].unique()) for k in range(4)] == [0.0, 1.0, 2.0, 3.0]
+    z = _zero_state(FlashRNNConfig(function="lstm", head_dim=4, num_heads=2, initial_val=0.5), x)
+    assert z.shape == (2, 3, 1, 2, 4) and float(z.unique()) == 0.5
+    back = _permuted(_permuted(z, "SBTHD", "STBHD"), "STBHD", "SBTHD")
+    assert torch.equal(back, z)
+    with pytest.raises(ValueError):
+        FlashRNNConfig(input_shape="BTGH")
+    with pytest.raises(ValueError):
+        FlashRNNConfig(output_shape="SBTHX")

@@ -178,3 +178,39 @@ def test_fused_and_alternating_gradients_agree(gpu, function, B, T, N, D):
         # dWx: per element as in test_fused_and_alternating_agree; dR: a sum over B*T tokens, bf16-rounded on return
         tol = 4e-2 * torch.clamp(a.abs(), min=1.0) if name == "dWx" else torch.full_like(a, max(4e-2, 2e-2 * scale))
         assert not bool((err > tol).any()), (name, float(err.max()), scale)
+
+
+def test_layout_options_equal_the_default_layouts(gpu):
+    """A call that declares other public layouts (time-major input, head-major R and bias, time-major
+    output) returns the default call's result in the declared output layout, gradients included."""
+    from flashrnn_amd import FlashRNNConfig, flashrnn
+
+    print("case layouts", flush=True)
+    B, T, N, D = 5, 7, 2, 64
+    inp = make_inputs("lstm", B, T, N, D, 77, init="randn", round_to=torch.bfloat16)
+    leaves = [inp[k].to(gpu, torch.bfloat16).requires_grad_(True) for k in ("Wx", "R", "b", "states")]
+    ds = inp["dstates"].to(gpu, torch.bfloat16)
+    out, last = flashrnn(*leaves, function="lstm", backend="hip_fused")
+    g = torch.autograd.grad(out, leaves, grad_outputs=ds)
+    cfg = FlashRNNConfig(function="lstm", backend="hip_fused", head_dim=D, num_heads=N, batch_size=B,
+                         input_shape="TBGHD", recurrent_shape="HPGD", bias_shape="HDG", output_shape="STBHD")
+    Wx2 = leaves[0].detach().permute(1, 0, 2, 3, 4).contiguous().requires_grad_(True)     # T B G H D
+    R2 = leaves[1].detach().permute(1, 3, 0, 2).contiguous().requires_grad_(True)         # H P G D
+    b2 = leaves[2].detach().permute(1, 2, 0).contiguous().requires_grad_(True)            # H D G
+    s2 = leaves[3].detach().permute(0, 2, 1, 3, 4).contiguous().requires_grad_(True)      # S T B H D
+    out2, last2 = flashrnn(Wx2, R2, b2, s2, config=cfg)
+    g2 = torch.autograd.grad(out2, [Wx2, R2, b2, s2], grad_outputs=ds.permute(0, 2, 1, 3, 4))
+    torch.cuda.synchronize()
+    assert out2.shape == (2, T, B, N, D) and last2.shape == (2, 1, B, N, D)
+    assert torch.equal(out2.permute(0, 2, 1, 3, 4), out) and torch.equal(last2.permute(0, 2, 1, 3, 4), last)
+    assert torch.equal(g2[0].permute(1, 0, 2, 3, 4), g[0])
+    assert torch.equal(g2[1].permute(2, 0, 3, 1), g[1])
+    assert torch.equal(g2[2].permute(2, 0, 1), g[2])
+    assert torch.equal(g2[3].permute(0, 2, 1, 3, 4), g[3])
+    # default initial state from initial_val
+    cfg0 = FlashRNNConfig(function="lstm", backend="hip_fused", head_dim=D, num_heads=N, batch_size=B, initial_val=0.25)
+    a, _ = flashrnn(leaves[0].detach(), leaves[1].detach(), leaves[2].detach(), None, config=cfg0)
+    s_const = torch.full((2, B, 1, N, D), 0.25, device=gpu, dtype=torch.bfloat16)
+    c, _ = flashrnn(leaves[0].detach(), leaves[1].detach(), leaves[2].detach(), s_const, function="lstm", backend="hip_fused")
+    torch.cuda.synchronize()
+    assert torch.equal(a, c)
