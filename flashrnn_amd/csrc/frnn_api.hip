@@ -399,6 +399,7 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  p.cooperative = env_int("FRNN_COOPERATIVE", 0);
   a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(function, p));
   a.h_clip = o.h_clip;
   a.trace = nullptr;
@@ -474,6 +475,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   a.ll = w.ll; a.status = w.status;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  p.cooperative = env_int("FRNN_COOPERATIVE", 0);
   // measured best, as in the forward call; the cells with several dWx stores issue them between
   // the send and the first probe, which is part of their delay
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", function == FRNN_ELMAN ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)

@@ -12,7 +12,10 @@
 #pragma once
 
 namespace frnn {
-struct Plan { int D, variant, waves, utw, kw; };
+struct Plan {
+  int D, variant, waves, utw, kw;
+  int cooperative = 0;  // host side only: launch the kernel as a cooperative one (see fused_*_tu.hip)
+};
 }
 
 // Measured on MI355X (T = 1024, bf16): when the head fits one workgroup, one tile per wave and

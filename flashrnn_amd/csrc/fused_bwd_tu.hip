@@ -18,6 +18,11 @@ int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
       if (e != hipSuccess) return (int)e;                                                                \
     }                                                                                                    \
+    if (K > 1 && p.cooperative) { /* see fused_fwd_tu.hip */                                             \
+      BwdArgs aa = a;                                                                                    \
+      void* args[] = {(void*)&aa};                                                                       \
+      return (int)hipLaunchCooperativeKernel((const void*)kern, grid, dim3(W * 64), args, lds, st);      \
+    }                                                                                                    \
     hipLaunchKernelGGL(kern, grid, dim3(W * 64), lds, st, a);                                            \
     return (int)hipGetLastError();                                                                       \
   }

@@ -94,9 +94,10 @@ size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, 
 
 /* Concurrency: when a head spans several workgroups (frnn_fused_plan: wgs_per_head > 1) they wait for
  * each other inside the kernel and a launch may fill the device, so run one such call at a time per
- * device (calls on one stream are; the reference's cooperative launch has the same property).  Calls
- * that overlap anyway cannot hang: every wait is bounded and a wait that runs out is reported in the
- * status word. */
+ * device (calls on one stream are; the reference's cooperative launch has the same property), or set
+ * FRNN_COOPERATIVE=1 in the environment: the kernels are then launched as cooperative kernels, which
+ * the runtime runs one at a time (about 15 us more per launch).  Calls that overlap anyway cannot
+ * hang: every wait is bounded and a wait that runs out is reported in the status word. */
 
 /* Forward over the whole sequence.  Replaces FlashRNNFuncFused::forward (fused/flashrnn.cc:68-144)
  * + ForwardPass::Run (fused/flashrnn_fused_forward.cu:772-975).

@@ -214,3 +214,27 @@ def test_layout_options_equal_the_default_layouts(gpu):
     c, _ = flashrnn(leaves[0].detach(), leaves[1].detach(), leaves[2].detach(), s_const, function="lstm", backend="hip_fused")
     torch.cuda.synchronize()
     assert torch.equal(a, c)
+
+
+@pytest.mark.parametrize("function,B,T,N,D", [("lstm", 8, 24, 3, 256), ("gru", 16, 8, 1, 768)])
+def test_cooperative_launch_gives_the_same_result(gpu, function, B, T, N, D, monkeypatch):
+    """FRNN_COOPERATIVE=1 launches the kernels whose workgroups wait for each other as cooperative
+    kernels (one at a time per device, for callers that overlap fused calls on several streams):
+    same bits as the plain launch."""
+    print(f"case cooperative {function} B{B} T{T} N{N} D{D}", flush=True)
+    inp = make_inputs(function, B, T, N, D, 31, init="randn", round_to=torch.bfloat16)
+
+    def run():
+        from flashrnn_amd import flashrnn
+
+        leaves = [inp[k].to(gpu, torch.bfloat16).requires_grad_(True) for k in ("Wx", "R", "b", "states")]
+        out, _ = flashrnn(*leaves, function=function, backend="hip_fused")
+        g = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(gpu, torch.bfloat16))
+        torch.cuda.synchronize()
+        return (out,) + g
+
+    plain = run()
+    monkeypatch.setenv("FRNN_COOPERATIVE", "1")
+    coop = run()
+    for a, b in zip(plain, coop):
+        assert torch.equal(a, b)
