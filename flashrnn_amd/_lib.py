@@ -51,6 +51,8 @@ _SIGNATURES = {
     "frnn_fused_backward_opt": (c_int, _BWD + [POINTER(Options)]),
     "frnn_alt_forward_opt": (c_int, _FWD + [POINTER(Options)]),
     "frnn_alt_backward_opt": (c_int, _BWD + [POINTER(Options)]),
+    "frnn_fused_forward_static_max_bytes": (c_size_t, []),
+    "frnn_fused_forward_static": (c_int, [c_int] * 7 + [c_void_p] * 7 + [POINTER(Options)]),
 }
 EXPORTED_SYMBOLS = tuple(_SIGNATURES)
 

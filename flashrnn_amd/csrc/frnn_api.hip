@@ -6,6 +6,8 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <mutex>
+
 #include "frnn_alt.h"
 #include "frnn_fused_bwd.h"
 #include "frnn_fused_fwd.h"
@@ -283,6 +285,31 @@ static int weight_grads(int function, int dtype, int B, int T, int N, int D, con
   return 0;
 }
 
+// ---- static scratch of frnn_fused_forward_static ------------------------------------------------------
+// Workspace (status word + the exchange slots between the workgroups of a head) for callers that cannot
+// allocate.  Every device the library runs on holds its own copy of the array until the process ends; in
+// host code the array's name is only a handle for hipGetSymbolAddress, the address itself is looked up
+// once per device (with that device current) and kept.
+static constexpr size_t kStaticScratchBytes = (size_t)4 << 20;
+static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
+static std::mutex g_scratch_mu;
+static void* g_scratch_ptr[64] = {nullptr};
+static int static_scratch(void** out) {
+  int dev = 0;
+  hipError_t e = hipGetDevice(&dev);
+  if (e != hipSuccess) return fail(FRNN_E_DEVICE, "hipGetDevice: %s", hipGetErrorString(e));
+  if (dev < 0 || dev >= 64) return fail(FRNN_E_DEVICE, "device index %d out of range", dev);
+  std::lock_guard<std::mutex> lk(g_scratch_mu);
+  if (!g_scratch_ptr[dev]) {
+    void* p = nullptr;
+    e = hipGetSymbolAddress(&p, HIP_SYMBOL(g_static_scratch));
+    if (e != hipSuccess || !p) return fail(FRNN_E_DEVICE, "hipGetSymbolAddress(static scratch): %s", hipGetErrorString(e));
+    g_scratch_ptr[dev] = p;
+  }
+  *out = g_scratch_ptr[dev];
+  return 0;
+}
+
 }  // namespace frnn
 
 using namespace frnn;
@@ -361,10 +388,11 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
                                 workspace_bytes, stream, nullptr);
 }
 
-int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
-                           const void* Wx, const void* R, const void* b, const void* s0,
-                           void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream,
-                           const frnn_options* opt) {
+// The forward call proper; `workspace` is the caller's buffer or this library's static scratch array.
+static int fused_forward_impl(int function, int dtype, int training, int B, int T, int N, int D,
+                              const void* Wx, const void* R, const void* b, const void* s0,
+                              void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream,
+                              const frnn_options* opt) {
   g_err[0] = 0;
   int e = check_problem(function, dtype, B, T, N, D);
   if (e) return e;
@@ -419,6 +447,37 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
     if (e) return hip_fail(e, "fused forward launch");
   }
   return 0;
+}
+
+int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
+                           const void* Wx, const void* R, const void* b, const void* s0,
+                           void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream,
+                           const frnn_options* opt) {
+  return fused_forward_impl(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, workspace,
+                            workspace_bytes, stream, opt);
+}
+
+size_t frnn_fused_forward_static_max_bytes(void) { return kStaticScratchBytes; }
+
+int frnn_fused_forward_static(int function, int dtype, int training, int B, int T, int N, int D,
+                              const void* Wx, const void* R, const void* b, const void* s0,
+                              void* states, void* cache, void* stream, const frnn_options* opt) {
+  g_err[0] = 0;
+  // refuse what does not fit before anything else, so that the message names the limit
+  int e = check_problem(function, dtype, B, T, N, D);
+  if (e) return e;
+  Plan p;
+  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
+    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  const size_t need = carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
+  if (need > kStaticScratchBytes)
+    return fail(FRNN_E_WORKSPACE, "this problem needs %zu bytes of workspace, the static scratch array holds %zu: "
+                "use frnn_fused_forward_opt with a workspace of the caller", need, kStaticScratchBytes);
+  void* ws = nullptr;
+  e = static_scratch(&ws);
+  if (e) return e;
+  return fused_forward_impl(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, ws,
+                            kStaticScratchBytes, stream, opt);
 }
 
 int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,

@@ -185,6 +185,21 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
                           void* workspace, size_t workspace_bytes, void* stream,
                           const frnn_options* opt);
 
+/* Forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose forward allocates its
+ * outputs and scratch on every call (fused/flashrnn.cc:97-118).  Same computation and same kernels as
+ * frnn_fused_forward_opt, but the workspace (status word + the exchange slots between the workgroups of a
+ * head) is a static array in device memory that belongs to the library: 4 MiB per device, held until the
+ * process ends (frnn_fused_forward_static_max_bytes()).  The call allocates and frees nothing.  A
+ * problem whose frnn_fused_workspace_bytes(..., backward = 0) exceeds that is refused with
+ * FRNN_E_WORKSPACE.  All calls on one device share the one array (each call clears the part it uses): two
+ * such calls that overlap on a device (different streams or threads) race, so keep them on one stream.
+ * The status word cannot be read by the caller; a bounded wait that ran out still shows as NaN in h. */
+size_t frnn_fused_forward_static_max_bytes(void);
+int frnn_fused_forward_static(int function, int dtype, int training, int B, int T, int N, int D,
+                              const void* Wx, const void* R, const void* b, const void* s0,
+                              void* states, void* cache, void* stream, const frnn_options* opt);
+
 #ifdef __cplusplus
 }
 #endif
