@@ -6,12 +6,16 @@ There is no CPU path: calls fail loudly without the HIP library or a GPU.
 """
 from .flashrnn import (  # noqa: F401
     FlashRNNConfig,
+    check_status,
     flashrnn,
+    flashrnn_step,
     fused_plan,
     last_status,
+    make_carry,
     rnn_function_registry,
 )
 from ._lib import build_library, library_path, load_library  # noqa: F401
 
-__all__ = ["flashrnn", "FlashRNNConfig", "rnn_function_registry", "fused_plan", "last_status",
+__all__ = ["flashrnn", "flashrnn_step", "make_carry", "FlashRNNConfig", "rnn_function_registry", "fused_plan",
+           "last_status", "check_status",
            "load_library", "library_path", "build_library"]

@@ -51,6 +51,10 @@ _SIGNATURES = {
     "frnn_fused_backward_opt": (c_int, _BWD + [POINTER(Options)]),
     "frnn_alt_forward_opt": (c_int, _FWD + [POINTER(Options)]),
     "frnn_alt_backward_opt": (c_int, _BWD + [POINTER(Options)]),
+    "frnn_fused_cache_bytes_opt": (c_size_t, _P6 + [POINTER(Options)]),
+    "frnn_alt_cache_bytes_opt": (c_size_t, _P6 + [POINTER(Options)]),
+    "frnn_fused_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),
+    "frnn_alt_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),
     "frnn_fused_forward_static_max_bytes": (c_size_t, []),
     "frnn_fused_forward_static": (c_int, [c_int] * 7 + [c_void_p] * 7 + [POINTER(Options)]),
 }

@@ -6,12 +6,15 @@
 
 namespace frnn {
 
-struct AltProblem { int function, dtype, B, T, N, D, training; float h_clip, g_clip; int cut; };
+struct AltProblem {
+  int function, dtype, B, T, N, D, training; float h_clip, g_clip; int cut;
+  int use_carry;  // forward: the first step takes its state from the fp32 side buffer, not from s0 (single-step calls)
+};
 
 struct AltFwdBuffers {
   const void* Wx; const void* R; const void* b; const void* s0;
   void* states; void* cache;
-  float* sfp;  // [S][B][N][D]
+  float* sfp;  // [S][B][N][D] fp32 running state; may be null for a single step without carry
 };
 
 struct AltBwdBuffers {

@@ -38,6 +38,8 @@ struct AltStepFwdArgs {
                     // that feeds the product is read back in the storage type), as in the fused path
   int B, T, N, D, t, training;
   float h_clip;     // > 0: new h clamped to [-h_clip, h_clip]
+  int from_sfp;     // this step takes s_{t-1} from sfp (every step but the first; the first too when the
+                    // caller carries the state of an earlier call in sfp)
 };
 
 template <int F, typename T>
@@ -75,7 +77,7 @@ __global__ void __launch_bounds__(256) alt_step_fwd_kernel(const AltStepFwdArgs 
   for (int g = GR; g < GT; ++g) bb[g - GR] = ld(bias + (size_t)(g * N + n) * D + d);
 #pragma unroll
   for (int k = 0; k < S; ++k)
-    s[k] = t > 0 ? a.sfp[(size_t)k * BND + idx] : ld(s0 + ((size_t)k * B + be) * ND + (size_t)n * D + d);
+    s[k] = a.from_sfp ? a.sfp[(size_t)k * BND + idx] : ld(s0 + ((size_t)k * B + be) * ND + (size_t)n * D + d);
 
   // ---- R h_{t-1} of the tile: acc[g] = rows (g, n, d0..d0+15) x batch rows bt*16..+15 ----
   {
@@ -122,7 +124,7 @@ __global__ void __launch_bounds__(256) alt_step_fwd_kernel(const AltStepFwdArgs 
 #pragma unroll
   for (int k = 0; k < S; ++k) {
     st_(states + (((size_t)k * B + b) * Tn + t) * ND + (size_t)n * D + d, s[k]);
-    a.sfp[(size_t)k * BND + idx] = s[k];
+    if (a.sfp) a.sfp[(size_t)k * BND + idx] = s[k];
   }
   if (a.training && NC > 0) {
     T* cache = static_cast<T*>(a.cache) + (((size_t)t * B + b) * N + n) * NC * D + d;
@@ -279,7 +281,8 @@ template <int F, typename T>
 static int alt_forward_t(const AltProblem& p, const AltFwdBuffers& bf, hipStream_t st) {
   const dim3 grid(p.D / 16, p.N, (p.B + 15) / 16);
   for (int t = 0; t < p.T; ++t) {
-    AltStepFwdArgs a{bf.Wx, bf.R, bf.b, bf.s0, bf.states, bf.cache, bf.sfp, p.B, p.T, p.N, p.D, t, p.training, p.h_clip};
+    AltStepFwdArgs a{bf.Wx, bf.R, bf.b, bf.s0, bf.states, bf.cache, bf.sfp, p.B, p.T, p.N, p.D, t, p.training, p.h_clip,
+                     (t > 0 || p.use_carry) ? 1 : 0};
     hipLaunchKernelGGL((alt_step_fwd_kernel<F, T>), grid, dim3(256), 0, st, a);
     const int e = (int)hipGetLastError();
     if (e) return e;
@@ -320,6 +323,9 @@ static int alt_backward_t(const AltProblem& p, const AltBwdBuffers& bf, hipStrea
     case FRNN_ELMAN * 3 + FRNN_BF16: return NAME<FRNN_ELMAN, bf16_t>(__VA_ARGS__);       \
     case FRNN_ELMAN * 3 + FRNN_F32:  return NAME<FRNN_ELMAN, float>(__VA_ARGS__);        \
     case FRNN_ELMAN * 3 + FRNN_F16:  return NAME<FRNN_ELMAN, half_t>(__VA_ARGS__);       \
+    case FRNN_ELMAN_CLIP * 3 + FRNN_BF16: return NAME<FRNN_ELMAN_CLIP, bf16_t>(__VA_ARGS__); \
+    case FRNN_ELMAN_CLIP * 3 + FRNN_F32:  return NAME<FRNN_ELMAN_CLIP, float>(__VA_ARGS__);  \
+    case FRNN_ELMAN_CLIP * 3 + FRNN_F16:  return NAME<FRNN_ELMAN_CLIP, half_t>(__VA_ARGS__); \
   }                                                                                      \
   return FRNN_E_ARG;
 

@@ -116,7 +116,7 @@ static int env_int(const char* name, int dflt) {
 //   elman D=512 (4 workgroups, 2 tiles per wave) 6, D=1024 (8 workgroups of 8 waves) 12.
 static int fwd_poll_delay_default(int function, const Plan& p) {
   if (p.kw <= 1) return 0;
-  if (function == FRNN_ELMAN) return p.waves > 4 ? 12 : 6;
+  if (function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP) return p.waves > 4 ? 12 : 6;
   if (p.kw == 3) return 2;
   if (p.kw == 6 || p.kw == 12) return 6;
   if (p.kw == 10) return 5;
@@ -138,6 +138,12 @@ static int device_cus() {
   return cached[dev];
 }
 
+// Groups (head, batch tile) of KW > 1 workgroups that one launch may hold.  The workgroups of a group wait
+// for each other, so all of them must be resident, and a group is pinned to one XCD (decode_block): what
+// counts is the room of an XCD (an eighth of the compute units, one such workgroup per compute unit), not
+// of the device: with KW = 12 an XCD of 32 compute units holds 2 groups, the device 16, not 256 / 12 = 21.
+static int groups_per_launch(int kw) { return 8 * ((device_cus() / 8) / kw); }
+
 // Batch rows per group: 4, 8 or 16.  Fewer rows per tile mean less gate math per lane and fewer
 // words to poll per step (the larger costs of a step) at the price of more workgroups and copies
 // of R, so the smallest tile is used for which every workgroup of the call still gets a compute
@@ -147,27 +153,68 @@ static int device_cus() {
 static int tile_rows_for(int B, int N, int kw, int waves) {
   const int forced = env_int("FRNN_TILE_ROWS", 0);
   if (forced == 4 || forced == 8 || forced == 16) return forced;
-  const long room = (long)device_cus() * (kw == 1 && waves <= 4 ? 3 : 1);
+  const long room = kw > 1 ? groups_per_launch(kw) : (long)device_cus() * (waves <= 4 ? 3 : 1);
   // one workgroup of 10 or 12 waves per head: 168 registers per wave, the 16-row variants spill
   // (LSTM D = 192 B = 1024: 3.6 ms with 16-row tiles, 3.1 with 8-row tiles in two rounds)
   const int largest = kw == 1 && waves > 8 ? 8 : 16;
   for (int tr = 4; tr < largest; tr *= 2)
-    if ((long)N * ((B + tr - 1) / tr) * kw <= room) return tr;
+    if ((long)N * ((B + tr - 1) / tr) <= room) return tr;
   return largest;
 }
 
-// Options as the kernels take them: a clip value of 0 switches the clamp off.
-struct Opts { float h_clip, g_clip; int cut; };
-static int parse_opts(const frnn_options* o, int function, bool forward, Opts* out) {
-  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0;
+// ---- one multi-workgroup launch at a time per device ------------------------------------------------
+// The workgroups of a head that spans several of them wait for each other, and a launch is sized to hold
+// all its groups on the device at once.  Two such kernels that ran at the same time (calls on different
+// streams) could each get a part of the device and starve each other until the bounded waits run out, so
+// the library orders them: per device it remembers the stream of the last such launch, and a launch on
+// another stream first waits (hipStreamWaitEvent, on the device, nothing blocks on the host) for an event
+// recorded on that stream.  Calls on one stream, the normal case, pay nothing.  The reference gets the same
+// guarantee from its cooperative launch (fused/flashrnn_fused_forward.cu:893-911).  Streams under graph
+// capture are left alone (a captured launch is replayed later, when this order means nothing): overlapping
+// replays are the caller's to order.  Kernels of other processes are not seen; there the bounded waits and
+// the status word remain the safety net.
+struct LaunchGate { std::mutex mu; hipEvent_t ev = nullptr; hipStream_t last = nullptr; bool have = false; };
+static LaunchGate g_gate[64];
+static bool stream_capturing(hipStream_t st) {
+  hipStreamCaptureStatus cs = hipStreamCaptureStatusNone;
+  if (hipStreamIsCapturing(st, &cs) != hipSuccess) { (void)hipGetLastError(); return false; }
+  return cs != hipStreamCaptureStatusNone;
+}
+// Locks the device's gate and orders `st` behind the last multi-workgroup launch; returns the gate to pass to
+// gate_leave, or null when there is nothing to do (one workgroup per head, capture, no device).
+static LaunchGate* gate_enter(int kw, hipStream_t st) {
+  if (kw <= 1) return nullptr;
+  int dev = 0;
+  if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return nullptr;
+  if (stream_capturing(st)) return nullptr;
+  LaunchGate* g = &g_gate[dev];
+  g->mu.lock();
+  if (g->have && g->last != st && !stream_capturing(g->last)) {
+    if (!g->ev && hipEventCreateWithFlags(&g->ev, hipEventDisableTiming) != hipSuccess) { g->ev = nullptr; (void)hipGetLastError(); }
+    // (a stream that no longer exists has no work left to wait for: errors are dropped)
+    if (g->ev && hipEventRecord(g->ev, g->last) == hipSuccess) (void)hipStreamWaitEvent(st, g->ev, 0);
+    (void)hipGetLastError();
+  }
+  return g;
+}
+static void gate_leave(LaunchGate* g, hipStream_t st) {
+  if (!g) return;
+  g->last = st; g->have = true;
+  g->mu.unlock();
+}
+
+// fx is the cell the kernels are instantiated for: the function itself, except that an Elman cell under
+// forward_clipval runs as FRNN_ELMAN_CLIP (one cached value per element: the unclamped h).
+struct Opts { float h_clip, g_clip; int cut; int fx; };
+static int parse_opts(const frnn_options* o, int function, Opts* out) {
+  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0; out->fx = function;
   if (!o) return 0;
   if (o->forward_clipval != o->forward_clipval || o->gradient_recurrent_clipval != o->gradient_recurrent_clipval ||
       o->forward_clipval < 0.f || o->gradient_recurrent_clipval < 0.f)
     return fail(FRNN_E_ARG, "clip values must be positive, or 0 for none (got %g, %g)", (double)o->forward_clipval,
                 (double)o->gradient_recurrent_clipval);
-  if (forward && o->forward_clipval > 0.f && function == FRNN_ELMAN)
-    return fail(FRNN_E_UNSUPPORTED, "forward_clipval is not available for elman: its backward pass rebuilds tanh' from the stored h");
   out->h_clip = o->forward_clipval; out->g_clip = o->gradient_recurrent_clipval; out->cut = o->gradient_recurrent_cut != 0;
+  if (function == FRNN_ELMAN && out->h_clip > 0.f) out->fx = FRNN_ELMAN_CLIP;
   return 0;
 }
 
@@ -373,6 +420,12 @@ size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int 
   return fused_cache_bytes_of(function, dtype, B, T, N, D);
 }
 
+size_t frnn_fused_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt) {
+  Opts o;
+  if (check_problem(function, dtype, B, T, N, D) || parse_opts(opt, function, &o)) return 0;
+  return fused_cache_bytes_of(o.fx, dtype, B, T, N, D);
+}
+
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
   Plan p;
@@ -388,65 +441,78 @@ int frnn_fused_forward(int function, int dtype, int training, int B, int T, int 
                                 workspace_bytes, stream, nullptr);
 }
 
-// The forward call proper; `workspace` is the caller's buffer or this library's static scratch array.
+// The forward call proper.  `workspace` is the caller's buffer or this library's static scratch array.
+// step != 0: one time step with carried state (frnn_fused_step): T = 1, no training, no workspace clear
+// (the one step neither waits for nor reads anything in the workspace; its exchange stores land in one
+// area shared by all groups), optional fp32 carry.
 static int fused_forward_impl(int function, int dtype, int training, int B, int T, int N, int D,
                               const void* Wx, const void* R, const void* b, const void* s0,
                               void* states, void* cache, void* workspace, size_t workspace_bytes, void* stream,
-                              const frnn_options* opt) {
+                              const frnn_options* opt, int step = 0, float* carry = nullptr) {
   g_err[0] = 0;
   int e = check_problem(function, dtype, B, T, N, D);
   if (e) return e;
   Opts o;
-  e = parse_opts(opt, function, true, &o);
+  e = parse_opts(opt, function, &o);
   if (e) return e;
+  const int fx = o.fx;
   Plan p;
-  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
+  if (!find_plan(fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
-  e = check_fused_sizes(function, dtype, B, T, N, D);
+  e = check_fused_sizes(fx, dtype, B, T, N, D);
   if (e) return e;
   CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
-  const bool need_cache = training && cell_dims(function).NC > 0;
+  const bool need_cache = training && cell_dims(fx).NC > 0;
   if (need_cache) CHECK_PTR(cache)
-  const FusedFwdWs w = carve_fused_fwd(workspace, dtype, B, N, D, p);
-  if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
-  prof_begin("fill_zero_kernel", st);
-  e = launch_fill_zero(workspace, w.zero_bytes, st);
-  prof_end(st);
-  if (e) return hip_fail(e, "workspace clear");
+  FusedFwdWs w = carve_fused_fwd(workspace, dtype, B, N, D, p);
+  if (!step) {
+    if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
+    prof_begin("fill_zero_kernel", st);
+    e = launch_fill_zero(workspace, w.zero_bytes, st);
+    prof_end(st);
+    if (e) return hip_fail(e, "workspace clear");
+  } else {
+    const size_t one_group = 256 + (p.kw > 1 ? (size_t)3 * 16 * D / (dtype == FRNN_F32 ? 1 : 2) * 8 : 0);
+    if (workspace_bytes < one_group) return fail(FRNN_E_WORKSPACE, "step scratch %zu < %zu bytes", workspace_bytes, one_group);
+  }
   const int tr = tile_rows_for(B, N, p.kw, p.waves);
   const int groups = N * ((B + tr - 1) / tr);
   int per_launch = groups;
   if (p.kw > 1) {  // workgroups that wait for each other must all be resident
-    per_launch = device_cus() / p.kw;
-    if (per_launch < 1) return fail(FRNN_E_DEVICE, "device has fewer compute units than the %d workgroups of one head", p.kw);
+    per_launch = groups_per_launch(p.kw);
+    if (per_launch < 1) return fail(FRNN_E_DEVICE, "an eighth of the device has fewer compute units than the %d workgroups of one head", p.kw);
   }
   FwdArgs a;
   a.Wx = Wx; a.R = R; a.b = b; a.s0 = s0; a.states = states; a.cache = cache;
   a.ll = w.ll; a.status = w.status;
+  a.carry = carry; a.step = step;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
-  a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(function, p));
+  a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(fx, p));
   a.h_clip = o.h_clip;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);
 #endif
+  LaunchGate* gate = gate_enter(step ? 1 : p.kw, st);  // (the workgroups of a single step never wait for each other)
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
     prof_begin("fused_fwd_kernel", st);
-    switch (function) {
+    switch (fx) {
       case FRNN_LSTM:  e = fused_fwd_dispatch<FRNN_LSTM>(dtype, p, a, st); break;
       case FRNN_SLSTM: e = fused_fwd_dispatch<FRNN_SLSTM>(dtype, p, a, st); break;
       case FRNN_GRU:   e = fused_fwd_dispatch<FRNN_GRU>(dtype, p, a, st); break;
-      default:         e = fused_fwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
+      case FRNN_ELMAN: e = fused_fwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
+      default:         e = fused_fwd_dispatch<FRNN_ELMAN_CLIP>(dtype, p, a, st); break;
     }
     prof_end(st);
-    if (e) return hip_fail(e, "fused forward launch");
+    if (e) break;
   }
-  return 0;
+  gate_leave(gate, st);
+  return e ? hip_fail(e, "fused forward launch") : 0;
 }
 
 int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
@@ -499,18 +565,19 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   int e = check_problem(function, dtype, B, T, N, D);
   if (e) return e;
   Opts o;
-  e = parse_opts(opt, function, false, &o);
+  e = parse_opts(opt, function, &o);
   if (e) return e;
-  const CellDims c = cell_dims(function);
+  const int fx = o.fx;
+  const CellDims c = cell_dims(fx);
   Plan p;
-  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
+  if (!find_plan(fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
-  e = check_fused_sizes(function, dtype, B, T, N, D);
+  e = check_fused_sizes(fx, dtype, B, T, N, D);
   if (e) return e;
   CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
   CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
   if (c.NC > 0) CHECK_PTR(cache)
-  const FusedBwdWs w = carve_fused_bwd(workspace, function, dtype, B, T, N, D, p);
+  const FusedBwdWs w = carve_fused_bwd(workspace, fx, dtype, B, T, N, D, p);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
   prof_begin("fill_zero_kernel", st);
@@ -525,8 +592,8 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   const int bt = (B + tr - 1) / tr, groups = N * bt;
   int per_launch = groups;
   if (p.kw > 1) {
-    per_launch = device_cus() / p.kw;
-    if (per_launch < 1) return fail(FRNN_E_DEVICE, "device has fewer compute units than the %d workgroups of one head", p.kw);
+    per_launch = groups_per_launch(p.kw);
+    if (per_launch < 1) return fail(FRNN_E_DEVICE, "an eighth of the device has fewer compute units than the %d workgroups of one head", p.kw);
   }
   BwdArgs a;
   a.Rt = w.Rt; a.s0 = s0; a.states = states; a.cache = cache; a.dstates = dstates;
@@ -537,26 +604,30 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
   // measured best, as in the forward call; the cells with several dWx stores issue them between
   // the send and the first probe, which is part of their delay
-  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", function == FRNN_ELMAN ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
-                                                                        : (p.kw >= 10 ? 8 : 4));
+  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", c.GR == 1 ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
+                                                                   : (p.kw >= 10 ? 8 : 4));
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);
 #endif
+  LaunchGate* gate = gate_enter(a.cut ? 1 : p.kw, st);  // (the truncated reverse scan exchanges nothing)
   for (int g0 = 0; g0 < groups; g0 += per_launch) {
     a.grp0 = g0; a.groups = groups - g0 < per_launch ? groups - g0 : per_launch;
     prof_begin("fused_bwd_kernel", st);
-    switch (function) {
+    switch (fx) {
       case FRNN_LSTM:  e = fused_bwd_dispatch<FRNN_LSTM>(dtype, p, a, st); break;
       case FRNN_SLSTM: e = fused_bwd_dispatch<FRNN_SLSTM>(dtype, p, a, st); break;
       case FRNN_GRU:   e = fused_bwd_dispatch<FRNN_GRU>(dtype, p, a, st); break;
-      default:         e = fused_bwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
+      case FRNN_ELMAN: e = fused_bwd_dispatch<FRNN_ELMAN>(dtype, p, a, st); break;
+      default:         e = fused_bwd_dispatch<FRNN_ELMAN_CLIP>(dtype, p, a, st); break;
     }
     prof_end(st);
-    if (e) return hip_fail(e, "fused backward launch");
+    if (e) break;
   }
-  return weight_grads(function, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, bt, dR, db, st);
+  gate_leave(gate, st);
+  if (e) return hip_fail(e, "fused backward launch");
+  return weight_grads(fx, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, bt, dR, db, st);
 }
 
 // ---- alternating --------------------------------------------------------------------------------------
@@ -570,6 +641,12 @@ int frnn_alt_supported(int function, int dtype, int B, int N, int D) {
 size_t frnn_alt_cache_bytes(int function, int dtype, int B, int T, int N, int D) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
   return (size_t)T * B * N * D * cell_dims(function).NC * dtype_size(dtype);
+}
+
+size_t frnn_alt_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt) {
+  Opts o;
+  if (check_problem(function, dtype, B, T, N, D) || parse_opts(opt, function, &o)) return 0;
+  return (size_t)T * B * N * D * cell_dims(o.fx).NC * dtype_size(dtype);
 }
 
 namespace {
@@ -618,20 +695,54 @@ int frnn_alt_forward_opt(int function, int dtype, int training, int B, int T, in
   int e = frnn_alt_supported(function, dtype, B, N, D);
   if (e) return e;
   Opts o;
-  e = parse_opts(opt, function, true, &o);
+  e = parse_opts(opt, function, &o);
   if (e) return e;
   if (T <= 0) return fail(FRNN_E_ARG, "non-positive T=%d", T);
   CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
-  const bool need_cache = training && cell_dims(function).NC > 0;
+  const bool need_cache = training && cell_dims(o.fx).NC > 0;
   if (need_cache) CHECK_PTR(cache)
-  const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 0);
+  const AltWs w = carve_alt(workspace, o.fx, dtype, B, T, N, D, 0);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
-  AltProblem p{function, dtype, B, T, N, D, need_cache ? 1 : 0, o.h_clip, 0.f, 0};
+  AltProblem p{o.fx, dtype, B, T, N, D, need_cache ? 1 : 0, o.h_clip, 0.f, 0, 0};
   AltFwdBuffers bf{Wx, R, b, s0, states, cache, w.sfp};
   prof_begin("alt_forward_steps", (hipStream_t)stream);
   e = alt_forward(p, bf, (hipStream_t)stream);
   prof_end((hipStream_t)stream);
   return e ? hip_fail(e, "alternating forward launch") : 0;
+}
+
+// ---- single step with carried state -----------------------------------------------------------------
+int frnn_fused_step(int function, int dtype, int B, int N, int D,
+                    const void* Wx_t, const void* R, const void* b, const void* s_in, void* s_out,
+                    float* carry, void* stream, const frnn_options* opt) {
+  g_err[0] = 0;
+  if (s_in == s_out && s_in) return fail(FRNN_E_ARG, "s_out must not be s_in: every workgroup of a head reads all of h");
+  if (carry && (((uintptr_t)carry) & 15)) return fail(FRNN_E_ALIGN, "carry is not 16-byte aligned");
+  void* ws = nullptr;
+  int e = static_scratch(&ws);
+  if (e) return e;
+  return fused_forward_impl(function, dtype, 0, B, 1, N, D, Wx_t, R, b, s_in, s_out, nullptr, ws, kStaticScratchBytes,
+                            stream, opt, 1, carry);
+}
+
+int frnn_alt_step(int function, int dtype, int B, int N, int D,
+                  const void* Wx_t, const void* R, const void* b, const void* s_in, void* s_out,
+                  float* carry, void* stream, const frnn_options* opt) {
+  g_err[0] = 0;
+  int e = frnn_alt_supported(function, dtype, B, N, D);
+  if (e) return e;
+  Opts o;
+  e = parse_opts(opt, function, &o);
+  if (e) return e;
+  CHECK_PTR(Wx_t) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s_in) CHECK_PTR(s_out)
+  if (s_in == s_out) return fail(FRNN_E_ARG, "s_out must not be s_in: every workgroup of a head reads all of h");
+  if (carry && (((uintptr_t)carry) & 15)) return fail(FRNN_E_ALIGN, "carry is not 16-byte aligned");
+  AltProblem p{o.fx, dtype, B, 1, N, D, 0, o.h_clip, 0.f, 0, carry ? 1 : 0};
+  AltFwdBuffers bf{Wx_t, R, b, s_in, s_out, nullptr, carry};
+  prof_begin("alt_forward_steps", (hipStream_t)stream);
+  e = alt_forward(p, bf, (hipStream_t)stream);
+  prof_end((hipStream_t)stream);
+  return e ? hip_fail(e, "alternating step launch") : 0;
 }
 
 int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
@@ -653,19 +764,20 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
   int e = frnn_alt_supported(function, dtype, B, N, D);
   if (e) return e;
   Opts o;
-  e = parse_opts(opt, function, false, &o);
+  e = parse_opts(opt, function, &o);
   if (e) return e;
   if (T <= 0) return fail(FRNN_E_ARG, "non-positive T=%d", T);
-  const CellDims c = cell_dims(function);
+  const int fx = o.fx;
+  const CellDims c = cell_dims(fx);
   CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
   CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
   if (c.NC > 0) CHECK_PTR(cache)
-  const AltWs w = carve_alt(workspace, function, dtype, B, T, N, D, 1);
+  const AltWs w = carve_alt(workspace, fx, dtype, B, T, N, D, 1);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   if (e) return hip_fail(e, "R transpose");
-  AltProblem p{function, dtype, B, T, N, D, 1, 0.f, o.g_clip, o.cut};
+  AltProblem p{fx, dtype, B, T, N, D, 1, 0.f, o.g_clip, o.cut, 0};
   AltBwdBuffers bf{w.Rt, s0, states, cache, dstates, dWx, w.dgx, ds0, w.dg, w.dsr};
   prof_begin("alt_backward_steps", st);
   e = alt_backward_scan(p, bf, st);
@@ -676,7 +788,7 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
   const void* src[4];
   long ld[4];
   for (int g = 0; g < c.GT; ++g) {
-    if (function == FRNN_GRU) {
+    if (fx == FRNN_GRU) {
       if (g == 0) { src[g] = w.dgx; ld[g] = (long)ND; }
       else { src[g] = (const char*)dWx + (size_t)(g - 1) * ND * es; ld[g] = (long)(c.GW * ND); }
     } else {
@@ -687,7 +799,7 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
   e = launch_bias_partial(dtype, src, ld, c.GT, N, D, (long)B * T, w.bsplits, w.dbp, st);
   prof_end(st);
   if (e) return hip_fail(e, "bias partial sums");
-  return weight_grads(function, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, w.bsplits, dR, db, st);
+  return weight_grads(fx, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, w.bsplits, dR, db, st);
 }
 
 }  // extern "C"

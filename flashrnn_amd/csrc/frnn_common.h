@@ -28,6 +28,11 @@ template <> struct Cell<FRNN_LSTM>  { static constexpr int GR = 4, GW = 4, GT = 
 template <> struct Cell<FRNN_SLSTM> { static constexpr int GR = 4, GW = 4, GT = 4, S = 4, NC = 5; };
 template <> struct Cell<FRNN_GRU>   { static constexpr int GR = 3, GW = 3, GT = 4, S = 1, NC = 4; };
 template <> struct Cell<FRNN_ELMAN> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 0; };
+// Internal variant of the Elman cell for forward_clipval: the stored h is clamped, so the adjoint cannot
+// rebuild tanh' from it and the forward pass caches the unclamped value, as the reference does
+// (flashrnn/flashrnn/fused/elman_fused_pointwise.cuh:34-60).  Not a function id of the C ABI.
+enum { FRNN_ELMAN_CLIP = 4 };
+template <> struct Cell<FRNN_ELMAN_CLIP> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 1; };
 
 struct CellDims { int GR, GW, GT, S, NC; };
 inline CellDims cell_dims(int f) {
@@ -36,6 +41,7 @@ inline CellDims cell_dims(int f) {
     case FRNN_SLSTM: return {4, 4, 4, 4, 5};
     case FRNN_GRU:   return {3, 3, 4, 1, 4};
     case FRNN_ELMAN: return {1, 1, 1, 1, 0};
+    case FRNN_ELMAN_CLIP: return {1, 1, 1, 1, 1};
   }
   return {0, 0, 0, 0, 0};
 }
@@ -305,7 +311,10 @@ __device__ __forceinline__ bool ll_ok(Part64*, u64 w, int t) { return (unsigned)
 __device__ __forceinline__ float part_value(Part64*, u64 w) { return __uint_as_float((unsigned)w); }
 __device__ __forceinline__ unsigned tag8(int t) { return (unsigned)(t % 255) + 1u; }
 __device__ __forceinline__ unsigned part_pack(Part32*, float a, int t) {
-  return (tag8(t) << 24) | ((__float_as_uint(a) + 0x80u) >> 8);
+  // round to nearest on the 8 dropped bits; a NaN is left as it is (the rounding add would carry a large
+  // NaN payload out of the word and turn the NaN into a zero)
+  const unsigned bits = __float_as_uint(a);
+  return (tag8(t) << 24) | ((a != a ? bits : bits + 0x80u) >> 8);
 }
 __device__ __forceinline__ bool ll_ok(Part32*, unsigned w, int t) { return (w >> 24) == tag8(t); }
 __device__ __forceinline__ float part_value(Part32*, unsigned w) { return __uint_as_float(w << 8); }

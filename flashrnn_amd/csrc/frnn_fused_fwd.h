@@ -29,8 +29,14 @@ struct FwdArgs {
   u64* ll; int* status;
   int B, T, N;
   int grp0, groups, groups_total;  // this launch handles groups [grp0, grp0 + groups)
-  int tile_rows;                   // batch rows per group: 8 (half-tile ownership) or 16
+  int tile_rows;                   // batch rows per group: 4, 8 or 16
   int training, spin_limit, poll_delay;
+  // single-step calls (T == 1, state carried from call to call): `carry` [S][B][N][D] fp32, if not null,
+  // holds the unrounded state: it is read instead of s0 for the gate math and rewritten at the end, so that
+  // a sequence of steps computes bit for bit what one call over the sequence does (which carries the state in
+  // fp32 registers); h for the recurrent product still comes from s0, in the storage type, as in the time loop.
+  // step != 0: all groups send their (unread) exchange words to one area
+  float* carry; int step;
   float h_clip;      // > 0: new h clamped to [-h_clip, h_clip] (forward_clipval)
   long long* trace;  // phase cycle sums per workgroup; only written by -DFRNN_TRACE builds
 };
@@ -171,7 +177,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       for (int g = GR; g < GT; ++g) bx[u][e][g - GR] = (float)bias_g[(size_t)(g * N + n) * D + ub[u] + esub + e];
 #pragma unroll
       for (int k = 0; k < S; ++k)
-        s[u][e][k] = bvalid ? (float)s0[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e] : 0.f;
+        s[u][e][k] = !bvalid ? 0.f : a.carry ? a.carry[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e]
+                                              : (float)s0[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e];
     }
   }
 
@@ -191,7 +198,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   int qpoll[NP];
   if (KW > 1) ll_plan<T, NP, NT, PAIRS>(tid, rows_valid, D, slice * (D / KW), D / KW, qpoll);
   // per group: slot 0, slot 1, and a third area that swallows the stores of padded lanes
-  u64* const llbase = a.ll + (size_t)grp * 3 * LLW;
+  u64* const llbase = a.ll + (size_t)(a.step ? 0 : grp) * 3 * LLW;
   const rsrc_t rLL = make_rsrc(llbase, (size_t)2 * LLW * 8);  // the two slots that are read
 
   // Wx is fetched PD steps ahead into a ring of PD + 1 register sets.  A head that exchanges
@@ -395,6 +402,14 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     o[0] = tr[0]; o[1] = tr[1]; o[2] = tr[2]; o[3] = clock64() - tr_begin;
   }
 #endif
+  if (a.carry && bvalid) {
+#pragma unroll
+    for (int u = 0; u < UTW; ++u)
+#pragma unroll
+      for (int e = 0; e < E; ++e)
+#pragma unroll
+        for (int k = 0; k < S; ++k) a.carry[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e] = s[u][e][k];
+  }
   if (dead) {
     // bounded wait ran out: report, and make the damage visible (NaN in every h of this
     // workgroup's units; the step that failed is not known exactly, so all steps are marked)

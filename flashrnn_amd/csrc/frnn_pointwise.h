@@ -145,4 +145,20 @@ template <bool FAST> struct CellMath<FRNN_ELMAN, FAST> {
   }
 };
 
+// Elman under forward_clipval: cache[0] is the unclamped tanh (the caller clamps s[0] after fwd)
+template <bool FAST> struct CellMath<FRNN_ELMAN_CLIP, FAST> {
+  typedef Math<FAST> M;
+  static __device__ __forceinline__ void fwd(const float* ry, const float* wx, const float* b, float* s, float* cache) {
+    s[0] = M::tanh(wx[0] + ry[0]);
+    cache[0] = s[0];
+  }
+  static __device__ __forceinline__ void bwd(const float* cache, const float*, const float*, const float* dso,
+                                             float* ds, float* dgr, float* dgw, float* dgb) {
+    const float dy = dso[0] + ds[0];
+    dgr[0] = (1.0f - cache[0] * cache[0]) * dy;
+    dgw[0] = dgr[0]; dgb[0] = dgr[0];
+    ds[0] = 0.0f;
+  }
+};
+
 }  // namespace frnn

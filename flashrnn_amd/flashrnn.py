@@ -67,6 +67,20 @@ class FlashRNNConfig:
     bias_shape: str = "GHD"
     # value of the default initial state, one number or one per state (flashrnn.py:204, :946-953)
     initial_val: Union[float, Sequence[float]] = 0.0
+    # per-tensor types of the reference (flashrnn.py:190-197: biases, recurrent matrix, inputs, gates,
+    # states, internal accumulation).  The kernels take every tensor in the one storage type `dtype`,
+    # accumulate in fp32 and compute the gates in fp32, so each may only be None or `dtype`
+    # (dtype_acc and dtype_a also "float32", which is what happens)
+    dtype_acc: Optional[str] = "float32"
+    dtype_b: Optional[str] = None
+    dtype_r: Optional[str] = None
+    dtype_w: Optional[str] = None
+    dtype_g: Optional[str] = None
+    dtype_s: Optional[str] = None
+    dtype_a: Optional[str] = None
+    # True: inputs of any floating type are cast to `dtype` on the way in (the reference's
+    # custom_fwd(cast_inputs=...), flashrnn.py:690-695); False: they must arrive in `dtype`
+    enable_automatic_mixed_precision: bool = True
 
     def __post_init__(self):
         if self.function not in rnn_function_registry:
@@ -81,6 +95,19 @@ class FlashRNNConfig:
                             ("bias_shape", "GHD")):
             if sorted(getattr(self, name)) != sorted(canon):
                 raise ValueError(f"{name} must be a permutation of {canon}, got {getattr(self, name)}")
+        for name in ("dtype_b", "dtype_r", "dtype_w", "dtype_g", "dtype_s"):
+            v = getattr(self, name)
+            if v is None:
+                setattr(self, name, self.dtype)
+            elif v != self.dtype:
+                raise ValueError(f"{name}={v}: the HIP kernels take every tensor in the one storage type "
+                                 f"dtype={self.dtype} (accumulation and gate math are fp32 whatever it is)")
+        for name in ("dtype_acc", "dtype_a"):
+            v = getattr(self, name)
+            if v is None:
+                setattr(self, name, "float32")
+            elif v not in ("float32", self.dtype):
+                raise ValueError(f"{name}={v}: accumulation and gate math are fp32")
         for name in ("gradient_recurrent_clipval", "forward_clipval"):
             v = getattr(self, name)
             if v is not None and not v > 0:
@@ -117,14 +144,82 @@ def _raise(code: int, what: str):
     raise RuntimeError(msg)
 
 
-_last_workspace = {}
+class _StatusLog:
+    """Status words of the fused calls, checked without a device-wide synchronisation.
+
+    A fused kernel whose bounded wait between workgroups ran out fills its outputs with NaN and sets the
+    status word at the head of its workspace.  Every fused call copies that word to pinned host memory
+    behind the kernels (4 bytes, asynchronous) and records an event; the entries whose event has
+    completed are read at the start of every later call (forward or backward, any stream), and a non-zero
+    one raises RuntimeError there.  ``check_status()`` waits for the entries still pending (their events
+    only) and does the same.  Entries made under stream capture are not logged: a replay repeats the
+    kernels, not this bookkeeping."""
+
+    def __init__(self):
+        import collections
+        import threading
+
+        self._lock = threading.Lock()
+        self._pending = collections.deque()
+        self._last = {}
+
+    def log(self, kind: str, ws: torch.Tensor, what: str):
+        if torch.cuda.is_current_stream_capturing():
+            return
+        host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+        host.copy_(ws[:4].view(torch.int32), non_blocking=True)
+        ev = torch.cuda.Event()
+        ev.record()
+        entry = (kind, what, host, ev)
+        with self._lock:
+            self._pending.append(entry)
+            self._last[kind] = entry
+
+    def poll(self, wait: bool = False):
+        if torch.cuda.is_current_stream_capturing():
+            return  # (querying an event is not allowed while this thread captures)
+        failed = []
+        with self._lock:
+            keep = []
+            while self._pending:
+                entry = self._pending.popleft()
+                kind, what, host, ev = entry
+                if wait:
+                    ev.synchronize()
+                if ev.query():
+                    if int(host[0]) != 0:
+                        failed.append(f"{kind} of {what}")
+                else:
+                    keep.append(entry)
+            self._pending.extend(keep)
+        if failed:
+            raise RuntimeError(
+                "flashrnn_amd: a bounded wait between the workgroups of a head ran out in an earlier fused call ("
+                + "; ".join(failed) + "): its outputs are NaN.  The workgroups of a head must all be resident; "
+                "another process's kernels on the same device can prevent that")
+
+    def last(self, kind: str) -> int:
+        with self._lock:
+            entry = self._last.get(kind)
+        if entry is None:
+            return 0
+        entry[3].synchronize()
+        return int(entry[2][0])
+
+
+_status = _StatusLog()
+
+
+def check_status() -> None:
+    """Waits for the fused calls made so far (their events, not the device) and raises RuntimeError if one of
+    them reported that a bounded wait between workgroups ran out."""
+    _status.poll(wait=True)
 
 
 def last_status(kind: str = "forward") -> int:
-    """Status word of the most recent fused call of this kind (synchronises): 0 ok, 1 = a bounded
-    wait between workgroups ran out and the outputs were filled with NaN."""
-    ws = _last_workspace.get(kind)
-    return 0 if ws is None else int(ws[:4].view(torch.int32).item())
+    """Status word of the most recent fused call of this kind (waits for that call): 0 ok, 1 = a bounded
+    wait between workgroups ran out and the outputs were filled with NaN.  Does not raise."""
+    return _status.last(kind)
 
 
 def fused_plan(function: str, dtype: str, B: int, N: int, D: int, backward: bool = False):
@@ -150,6 +245,12 @@ class _FlashRNNFunction(torch.autograd.Function):
         f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
         B, T, Gw, N, D = Wx.shape
         S = cfg.num_states
+        _status.poll()
+        if not cfg.enable_automatic_mixed_precision:
+            for name, x in (("Wx", Wx), ("R", R), ("b", b), ("states", s0)):
+                if x.dtype != kdt:
+                    raise TypeError(f"{name} is {x.dtype}, the kernel type is {kdt} and "
+                                    "enable_automatic_mixed_precision is off")
         # cast to the kernel type as the reference's custom_fwd(cast_inputs=...) does (:690-695)
         Wx_k = Wx.detach().to(kdt).contiguous()
         R_k = R.detach().to(kdt).contiguous()
@@ -160,7 +261,7 @@ class _FlashRNNFunction(torch.autograd.Function):
             if rc != 0:
                 _raise(rc, f"{cfg.backend} backend")
             states = torch.empty((S, B, T, N, D), dtype=kdt, device=Wx.device)
-            cache_bytes = _entry(cfg.backend, "cache_bytes")(f_id, d_id, B, T, N, D) if training else 0
+            cache_bytes = _entry(cfg.backend, "cache_bytes_opt")(f_id, d_id, B, T, N, D, _options(cfg)) if training else 0
             cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx.device)
             ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 0)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx.device)
@@ -171,8 +272,8 @@ class _FlashRNNFunction(torch.autograd.Function):
                 ws.data_ptr(), ws.numel(), stream, _options(cfg))
             if rc != 0:
                 _raise(rc, f"{cfg.backend} forward")
-        if cfg.backend == "hip_fused":
-            _last_workspace["forward"] = ws
+            if cfg.backend == "hip_fused":
+                _status.log("forward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
         ctx.cfg, ctx.training = cfg, training
         ctx.dims = (B, T, N, D)
         ctx.save_for_backward(R_k, b_k, s0_k, states, cache)
@@ -190,6 +291,7 @@ class _FlashRNNFunction(torch.autograd.Function):
         B, T, N, D = ctx.dims
         S, Gw, Gr, Gt = cfg.num_states, cfg.num_gates_w, cfg.num_gates_r, cfg.num_gates_t
         dev = states.device
+        _status.poll()
         ds = dstates.to(kdt).contiguous()
         with torch.cuda.device(dev):
             dWx = torch.empty((B, T, Gw, N, D), dtype=kdt, device=dev)
@@ -205,8 +307,8 @@ class _FlashRNNFunction(torch.autograd.Function):
                 ws.data_ptr(), ws.numel(), stream, _options(cfg))
             if rc != 0:
                 _raise(rc, f"{cfg.backend} backward")
-        if cfg.backend == "hip_fused":
-            _last_workspace["backward"] = ws
+            if cfg.backend == "hip_fused":
+                _status.log("backward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
         # dR / db stay fp32: autograd casts them to the dtype of the leaf they belong to, so fp32
         # master weights receive unrounded gradients
         return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None
@@ -286,8 +388,83 @@ def flashrnn(
     if D == 16:
         out = _paired_heads(Wx, R, b, states, config, training)
     else:
-        out = _FlashRNNFunction.apply(Wx, R, b, states, config, training)
+        out = _apply_in_batch_ranges(Wx, R, b, states, config, training)
     return _permuted(out, "SBTHD", config.output_shape), _permuted(out[:, :, -1:], "SBTHD", config.output_shape)
+
+
+_FUSED_TENSOR_LIMIT = 1 << 31  # the fused kernels address each tensor with 32-bit byte offsets
+
+
+def _apply_in_batch_ranges(Wx, R, b, states, config, training):
+    """Batch rows are independent, so a fused problem one of whose tensors (Wx, the states or the gate cache)
+    would reach 2 GiB runs as several calls over ranges of the batch; autograd sums dR and db over the ranges.
+    Wx[b0:b1] is a view (the batch is its leading axis); the outputs of the ranges are concatenated."""
+    B, T, Gw, N, D = Wx.shape
+    if config.backend != "hip_fused":
+        return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
+    es = 4 if config.dtype == "float32" else 2
+    per_row = T * N * D * es * max(Gw, config.num_states, 6 if training else 0)  # at most 6 cached values per element
+    rows = max(1, (_FUSED_TENSOR_LIMIT - 1) // per_row)
+    if rows >= B:
+        return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
+    rows = max(16, rows // 16 * 16) if rows >= 16 else rows  # whole batch tiles
+    outs = [_FlashRNNFunction.apply(Wx[b0:b0 + rows], R, b, states[:, b0:b0 + rows], config, training)
+            for b0 in range(0, B, rows)]
+    return torch.cat(outs, dim=1)
+
+
+def flashrnn_step(
+    Wx: torch.Tensor,  # [B, 1, G_w, N, D]
+    R: torch.Tensor,  # [G_r, N, D, D]
+    b: torch.Tensor,  # [G_t, N, D]
+    states: torch.Tensor,  # [S, B, 1, N, D]
+    function: str = "lstm",
+    config: Optional[FlashRNNConfig] = None,
+    backend: str = "hip_fused",
+    dtype: str = "bfloat16",
+    carry: Optional[torch.Tensor] = None,  # [S, B, N, D] float32, updated in place
+) -> torch.Tensor:
+    """One time step with carried state, for inference / decoding (the reference's step kernels,
+    flashrnn.py:957-985): returns the new states [S,B,1,N,D].  One kernel launch, no workspace, nothing cleared;
+    not differentiable.  Tensors must already be in the kernel dtype and the default layouts (nothing is cast
+    or copied on this path).
+
+    ``carry`` (``make_carry(states)`` before the first step, then the same tensor every step) holds the unrounded
+    state: with it a chain of steps yields bit for bit what one ``flashrnn()`` call over the sequence does, which
+    keeps the state in fp32 registers between time steps; without it every step starts from the rounded
+    ``states``."""
+    if config is None:
+        config = _get_config(Wx, R, b, function, backend, dtype)
+    kdt = DTYPE_DICT[config.dtype]
+    Gr, Gw, _, Gt, S = rnn_function_registry[config.function]["gates_states"]
+    if Wx.dim() != 5 or Wx.shape[1] != 1 or Wx.shape[2] != Gw:
+        raise ValueError(f"Wx must be [B,1,{Gw},N,D], got {tuple(Wx.shape)}")
+    B, _, _, N, D = Wx.shape
+    if tuple(R.shape) != (Gr, N, D, D) or tuple(b.shape) != (Gt, N, D) or tuple(states.shape) != (S, B, 1, N, D):
+        raise ValueError(f"R, b, states must be [{Gr},{N},{D},{D}], [{Gt},{N},{D}], [{S},{B},1,{N},{D}]; got "
+                         f"{tuple(R.shape)}, {tuple(b.shape)}, {tuple(states.shape)}")
+    for name, x in (("Wx", Wx), ("R", R), ("b", b), ("states", states)):
+        if not x.is_cuda:
+            raise RuntimeError("flashrnn_amd runs on a GPU only (got a CPU tensor); there is no CPU fallback")
+        if x.dtype != kdt or not x.is_contiguous():
+            raise TypeError(f"{name} must be a contiguous {kdt} tensor (the step path casts and copies nothing)")
+    if carry is not None and (carry.dtype != torch.float32 or tuple(carry.shape) != (S, B, N, D)
+                              or not carry.is_contiguous() or carry.device != Wx.device):
+        raise TypeError(f"carry must be a contiguous float32 tensor [{S},{B},{N},{D}] on the device of Wx")
+    f_id, d_id = _lib.FUNCTION_IDS[config.function], _lib.DTYPE_IDS[config.dtype]
+    with torch.cuda.device(Wx.device):
+        out = torch.empty((S, B, 1, N, D), dtype=kdt, device=Wx.device)
+        rc = _entry(config.backend, "step")(
+            f_id, d_id, B, N, D, Wx.data_ptr(), R.data_ptr(), b.data_ptr(), states.data_ptr(), out.data_ptr(),
+            carry.data_ptr() if carry is not None else None, torch.cuda.current_stream().cuda_stream, _options(config))
+        if rc != 0:
+            _raise(rc, f"{config.backend} step")
+    return out
+
+
+def make_carry(states: torch.Tensor) -> torch.Tensor:
+    """The fp32 carry of ``flashrnn_step`` for a chain that starts at ``states`` [S,B,1,N,D]."""
+    return states[:, :, 0].to(torch.float32).contiguous()
 
 
 def _paired_heads(Wx, R, b, states, config, training):

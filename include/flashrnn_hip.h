@@ -149,8 +149,9 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
  * alternating/flashrnn.cc:220-302); here they are run-time arguments of *_opt twins of the four
  * entry points above (opt == NULL or all fields zero: identical to the plain entry point).
  *   forward_clipval > 0:  every new h is clamped to [-v, v] before it is stored and fed back
- *     (lstm_fused_pointwise.cuh:75-80); the backward pass does not see the clamp.  Not available
- *     for FRNN_ELMAN (its backward rebuilds tanh' from the stored h): FRNN_E_UNSUPPORTED.
+ *     (lstm_fused_pointwise.cuh:75-80); the backward pass does not see the clamp.  For FRNN_ELMAN the
+ *     training forward then fills a gate cache with the unclamped h (sizes: *_cache_bytes_opt), which the
+ *     backward call, given the same options, reads for tanh'.
  *   gradient_recurrent_clipval > 0:  in every reverse step the cotangent carried into h_t from
  *     step t+1 is clamped to [-v, v] before the upstream cotangent is added
  *     (lstm_fused_pointwise.cuh:115-121); ds0 itself is not clamped.
@@ -163,6 +164,11 @@ typedef struct frnn_options {
   float gradient_recurrent_clipval;
   int gradient_recurrent_cut;
 } frnn_options;
+
+/* Gate-cache size under options: an Elman cell under forward_clipval caches the unclamped h (one value per
+ * element, as elman_fused_pointwise.cuh:44-47), without it nothing.  opt == NULL: as the plain queries. */
+size_t frnn_fused_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt);
+size_t frnn_alt_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt);
 
 int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,
                            const void* Wx, const void* R, const void* b, const void* s0,
@@ -184,6 +190,23 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
                           void* dWx, void* ds0, float* dR, float* db,
                           void* workspace, size_t workspace_bytes, void* stream,
                           const frnn_options* opt);
+
+/* ---- one time step with carried state (inference / decoding) --------------------------------------------
+ * Replaces the reference's step kernels (_get_kernel_step, flashrnn.py:957-985, which run the whole-sequence
+ * function on a sequence of one; ForwardPass::Iterate, alternating/flashrnn.h:97-101).  One kernel launch,
+ * no workspace, nothing cleared, nothing allocated; can be captured into a HIP graph.
+ *   Wx_t [B,G_w,N,D], s_in / s_out [S,B,N,D] in the storage type; s_out must not be s_in (ping-pong).
+ *   carry: null, or [S,B,N,D] fp32, updated in place: the unrounded state.  The whole-sequence kernels keep
+ *     c, n, m (and the h that enters the gate math) in fp32 across time steps and round only what they store;
+ *     with a carry a chain of steps does the same and yields the bits of one call over the sequence, without
+ *     it every step restarts from the rounded s_in (which is what the reference's step kernel does).  Before
+ *     the first step fill it with the initial state converted to fp32. */
+int frnn_fused_step(int function, int dtype, int B, int N, int D,
+                    const void* Wx_t, const void* R, const void* b, const void* s_in, void* s_out,
+                    float* carry, void* stream, const frnn_options* opt);
+int frnn_alt_step(int function, int dtype, int B, int N, int D,
+                  const void* Wx_t, const void* R, const void* b, const void* s_in, void* s_out,
+                  float* carry, void* stream, const frnn_options* opt);
 
 /* Forward for callers that cannot allocate device memory (code under HIP graph capture, tight serving
  * loops, harnesses that forbid hipMalloc).  No counterpart in the reference, whose forward allocates its

@@ -37,9 +37,11 @@ Pinning (tests/test_oracle_*.py, none of them re-types these formulas):
   the three options by hand-derived closed forms on a scalar Elman cell, by the agreement of
   the autograd formulation (identity-forward / clamp-backward node, detach) with the explicit
   reverse scan, and by their no-op limits (huge clip value, R = 0).
-  PARITY UNPINNED: the sLSTM backward under ``forward_clipval`` -- the native adjoint reads the
-  stored (clamped) h (slstm_fused_pointwise.cuh:117-186); only ``flashrnn_oracle_fwbw_manual``
-  restates that and nothing independent checks it.
+  the sLSTM backward under ``forward_clipval`` (the native adjoint reads the stored, clamped h,
+  slstm_fused_pointwise.cuh:117-186, which only ``flashrnn_oracle_fwbw_manual`` restates) by a closed
+  form derived by hand on a scalar cell over two steps with the clamp active;
+  the sLSTM adjoint for cotangents on c and n (stabiliser held constant) by float64 autograd with the
+  stabiliser detached.
   The reference holds no golden vectors for this path (its only known-answer test is
   flashrnn/tests/test_lstm.py:70-115, LSTM vs torch.nn.LSTM, which is reproduced).
 """
@@ -93,10 +95,16 @@ def _pw_elman(Wx_t, Ry, b, s):
     return (torch.tanh(Wx_t[:, 0] + Ry[:, 0] + b[0]),)
 
 
-def _pw_slstm(Wx_t, Ry, b, s, per_element_first_step=False):
+def _pw_slstm(Wx_t, Ry, b, s, per_element_first_step=False, detach_m=False):
     raw = Wx_t + Ry + b[None]
     i, f, z, o = raw.unbind(1)
     _, c, n, m = s
+    if detach_m:
+        # the native adjoint holds the stabiliser constant: no cotangent enters m_t or leaves through
+        # m_{t-1} (slstm_fused_pointwise.cuh:117-186 differentiates exp(i - m') and exp(logsig(f) + m - m')
+        # with m, m' fixed and returns ds[3] = 0).  For a loss on h this is the full gradient (h does not
+        # depend on m); for a loss on c or n, which scale with exp(-m), it is not.
+        m = m.detach()
     lfm = F.logsigmoid(f) + m
     if per_element_first_step:
         # what the native kernels test (slstm_fused_pointwise.cuh:54-62)
@@ -105,10 +113,19 @@ def _pw_slstm(Wx_t, Ry, b, s, per_element_first_step=False):
         m_new = i
     else:
         m_new = torch.maximum(i, lfm)
+    if detach_m:
+        m_new = m_new.detach()
     ig = torch.exp(i - m_new)
     fg = torch.exp(lfm - m_new)
     c_new = fg * c + ig * torch.tanh(z)
-    n_new = torch.maximum(fg * n + ig, torch.ones_like(n))
+    n_raw = fg * n + ig
+    n_new = torch.maximum(n_raw, torch.ones_like(n))
+    if detach_m:
+        # the native adjoint differentiates n' = fg n + ig and ignores the guard max(., 1), which is never
+        # strictly active on reachable states ("n cannot get smaller than one by construction",
+        # slstm_fused_pointwise.cuh:90-92) but ties at the very first step (n' = 0 + 1), where autograd
+        # would halve the slope
+        n_new = n_raw + (n_new - n_raw).detach()
     h_new = torch.sigmoid(o) * c_new / n_new
     return (h_new, c_new, n_new, m_new)
 
@@ -137,6 +154,7 @@ def flashrnn_oracle(
     states: Optional[torch.Tensor] = None,
     function: str = "lstm",
     slstm_per_element_first_step: bool = False,
+    slstm_detach_m: bool = False,
     forward_clipval: Optional[float] = None,
     gradient_recurrent_clipval: Optional[float] = None,
     gradient_recurrent_cut: bool = False,
@@ -145,6 +163,8 @@ def flashrnn_oracle(
 
     ``forward_clipval``: the new h of every step is clamped to [-v, v]; the backward pass does not
     see the clamp (straight-through), as the native backward pointwise functions do not.
+    ``slstm_detach_m``: differentiation as the native adjoint does it (values unchanged): the stabiliser
+    state is held constant and the guard max(., 1) on n is transparent.
     ``gradient_recurrent_clipval``: the cotangent that step t+1 sends to h_t (through R and through
     the pointwise carry) is clamped before the upstream cotangent of h_t is added; the cotangent
     of the initial state is not clamped.  ``gradient_recurrent_cut``: no gradient through R h.
@@ -173,7 +193,7 @@ def flashrnn_oracle(
         Ry = torch.matmul(h_rec.transpose(0, 1), Rm)  # [N,B,G_r*D]
         Ry = Ry.reshape(N, B, Gr, D).permute(1, 2, 0, 3)  # [B,G_r,N,D]
         if function == "slstm":
-            s = pw(Wx_t[t], Ry, b, s_in, slstm_per_element_first_step)
+            s = pw(Wx_t[t], Ry, b, s_in, slstm_per_element_first_step, slstm_detach_m)
         else:
             s = pw(Wx_t[t], Ry, b, s_in)
         if forward_clipval is not None:

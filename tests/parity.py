@@ -19,6 +19,18 @@ of the oracle fed the same bf16-rounded inputs):
                             returns them in fp32.
   fp16   as bf16 with every bound divided by 4 (3 more mantissa bits; the reference states no
          fp16 tolerance).
+On top of the element-wise bounds, for the 16-bit types:
+  * a norm-wise bound per tensor, ||err||_F / ||ref||_F <= 3e-3 for states and 8e-3 for gradients (bf16;
+    measured at the full-size benchmark configurations: 1.7e-3 for every state, 2.1e-3 .. 4.6e-3 for the
+    gradients), which a missing or mis-indexed small term cannot hide behind one large element;
+  * where asked (``vs_bf16_vanilla``: the full-size configurations), a second reference: the oracle run
+    in torch.bfloat16 on the CPU, which is what the reference's own ``vanilla`` backend computes in bf16
+    (vanilla/__init__.py:46-50).  Per tensor the HIP path must be at least as close to the fp32 oracle as
+    that run is, in max-abs and in Frobenius norm.  This is the demonstration that the bounds above are
+    what bf16 storage costs: the all-bf16 run misses plain 2e-2 max-abs by far more (dR: 4.6 against the
+    kernel's 0.17 at the metric configuration).
+sLSTM gradients are compared with autograd in which the stabiliser m is held constant, as the native
+adjoint holds it (cotangents on c and n included; equal to plain autograd for a cotangent on h alone).
 """
 import torch
 
@@ -29,7 +41,7 @@ from oracle.flashrnn_oracle import flashrnn_oracle_fwbw_manual
 def oracle_run(function, inp, dtype, backward=True, options=None):
     odt = torch.float64 if dtype == "float32" else torch.float32
     options = dict(options or {})
-    kw = {"slstm_per_element_first_step": True} if function == "slstm" else {}
+    kw = {"slstm_per_element_first_step": True, "slstm_detach_m": True} if function == "slstm" else {}
     args = [inp[k].to(odt) for k in ("Wx", "R", "b", "states")]
     if backward and function == "slstm" and options.get("forward_clipval") is not None:
         # the native sLSTM adjoint reads the stored (clamped) h: only the explicit scan states that
@@ -43,7 +55,7 @@ def oracle_run(function, inp, dtype, backward=True, options=None):
 
 
 def hip_run(function, inp, dtype, backend, device, backward=True, options=None):
-    from flashrnn_amd import FlashRNNConfig, flashrnn, last_status
+    from flashrnn_amd import FlashRNNConfig, check_status, flashrnn
 
     leaves = [inp[k].to(device).requires_grad_(backward) for k in ("Wx", "R", "b", "states")]
     B, _, _, N, D = inp["Wx"].shape
@@ -55,12 +67,34 @@ def hip_run(function, inp, dtype, backend, device, backward=True, options=None):
         grads = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(device).to(out.dtype))
         grads = [g.float().cpu() for g in grads]
     torch.cuda.synchronize()
-    if backend == "hip_fused":
-        assert last_status("forward") == 0, "a bounded wait between workgroups ran out (forward)"
-        if backward:
-            assert last_status("backward") == 0, "a bounded wait between workgroups ran out (backward)"
+    check_status()  # raises if a bounded wait between workgroups ran out in any fused call so far
     assert torch.equal(last, out[:, :, -1:])
     return out.detach().float().cpu(), grads
+
+
+def bf16_vanilla_run(function, inp, backward=True):
+    """The oracle in torch.bfloat16 on the CPU: every matmul, gate and state in bf16, as the reference's
+    ``vanilla`` backend run with dtype=bfloat16."""
+    kw = {"slstm_per_element_first_step": True, "slstm_detach_m": True} if function == "slstm" else {}
+    args = [inp[k].to(torch.bfloat16) for k in ("Wx", "R", "b", "states")]
+    if backward:
+        out, grads = flashrnn_oracle_backward(*args, function, inp["dstates"].to(torch.bfloat16), **kw)
+        return out.float(), [g.float() for g in grads]
+    with torch.no_grad():
+        return flashrnn_oracle(*args, function, **kw)[0].float(), None
+
+
+def assert_not_worse_than(name, got, other, ref):
+    """err(got vs ref) <= err(other vs ref) in max-abs and in Frobenius norm."""
+    ref = ref.double()
+    e, eo = (got.double() - ref), (other.double() - ref)
+    assert float(e.abs().max()) <= float(eo.abs().max()), \
+        f"{name}: max-abs error {float(e.abs().max()):.3e} exceeds that of the bf16 vanilla run, {float(eo.abs().max()):.3e}"
+    assert float(e.norm()) <= float(eo.norm()), \
+        f"{name}: Frobenius error {float(e.norm()):.3e} exceeds that of the bf16 vanilla run, {float(eo.norm()):.3e}"
+
+
+REL_F = {"h": 3e-3, "state": 3e-3, "token": 8e-3, "sum": 8e-3}   # bf16; fp16: / 4
 
 
 def assert_close(name, got, ref, dtype, kind):
@@ -69,6 +103,9 @@ def assert_close(name, got, ref, dtype, kind):
     assert torch.isfinite(got).all(), f"{name}: non-finite values"
     # float16 carries 3 more mantissa bits than bfloat16: its tolerances are the bf16 ones / 4
     q = 0.25 if dtype == "float16" else 1.0
+    if dtype != "float32" and float(ref.norm()) > 0:
+        rel = float(err.norm() / ref.norm())
+        assert rel <= REL_F[kind] * q, f"{name}: ||err||_F / ||ref||_F = {rel:.3e} > {REL_F[kind] * q:.1e}"
     if dtype == "float32":
         tol = 1e-5 * max(1.0, float(ref.abs().max()))
         assert float(err.max()) <= tol, f"{name}: max err {float(err.max()):.3e} > {tol:.3e}"
@@ -87,11 +124,14 @@ def assert_close(name, got, ref, dtype, kind):
 
 
 def check_case(device, function, B, T, N, D, dtype, backend, seed=1, init="randn", backward=True,
-               forget_bias_linspace=False, options=None):
-    grad_on = "h" if function == "slstm" else "all"
+               forget_bias_linspace=False, options=None, grad_on="all", vs_bf16_vanilla=False):
     inp = make_inputs(function, B, T, N, D, seed, init=init,
                       round_to={"bfloat16": torch.bfloat16, "float16": torch.float16}.get(dtype), grad_on=grad_on,
                       forget_bias_linspace=forget_bias_linspace)
+    if function == "slstm":
+        inp["dstates"][3] = 0  # the stabiliser gets no cotangent anywhere in the native path
+        if options and options.get("forward_clipval") is not None:
+            inp["dstates"][1:] = 0  # (the closed form that pins this corner has a cotangent on h only)
     ref_out, ref_g = oracle_run(function, inp, dtype, backward, options)
     out, grads = hip_run(function, inp, dtype, backend, device, backward, options)
     S = FUNCTIONS[function][4]
@@ -103,8 +143,19 @@ def check_case(device, function, B, T, N, D, dtype, backend, seed=1, init="randn
         assert_close("db", grads[2], ref_g[2], dtype, "sum")
         for k in range(S):
             if function == "slstm" and k == 3:
-                continue  # the stabiliser m is held constant by design: its cotangent is reported as 0
-            if function == "slstm" and k == 2 and init == "zeros":
-                continue  # n0 = 0 sits on the kink of max(., 1) and of the first-step branch
+                assert float(grads[3][k].abs().max()) == 0.0  # the stabiliser is held constant: d/dm0 = 0
+                continue
             assert_close(f"dstates0[{k}]", grads[3][k], ref_g[3][k], dtype, "token")
+    if vs_bf16_vanilla:
+        assert dtype == "bfloat16" and not options
+        v_out, v_g = bf16_vanilla_run(function, inp, backward)
+        for k in range(S):
+            assert_not_worse_than(f"state {k}", out[k], v_out[k], ref_out[k])
+        if backward:
+            for name, i in (("dWx", 0), ("dR", 1), ("db", 2)):
+                assert_not_worse_than(name, grads[i], v_g[i], ref_g[i])
+            for k in range(S):
+                if function == "slstm" and k == 3:
+                    continue
+                assert_not_worse_than(f"dstates0[{k}]", grads[3][k], v_g[3][k], ref_g[3][k])
     return out, grads

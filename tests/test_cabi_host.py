@@ -165,7 +165,8 @@ def test_missing_library_is_an_error(monkeypatch, tmp_path):
 
 
 def test_options_are_validated_before_launch(lib):
-    """frnn_options: negative or NaN clip values are argument errors; forward_clipval has no elman kernel."""
+    """frnn_options: negative or NaN clip values are argument errors; forward_clipval is accepted for every cell
+    (elman then needs a gate cache for the unclamped h, which the size query reports)."""
     import math
 
     def fwd(entry, function=0, **opt):
@@ -176,9 +177,14 @@ def test_options_are_validated_before_launch(lib):
     for entry in ("frnn_fused_forward_opt", "frnn_alt_forward_opt"):
         assert fwd(entry, f=-1.0) == _lib.E_ARG
         assert fwd(entry, g=math.nan) == _lib.E_ARG
-        assert fwd(entry, function=_lib.FUNCTION_IDS["elman"], f=0.5) == _lib.E_UNSUPPORTED
-        assert b"elman" in lib.frnn_last_error()
+        assert fwd(entry, function=_lib.FUNCTION_IDS["elman"], f=0.5) == _lib.E_WORKSPACE
         assert fwd(entry, f=0.5) == _lib.E_WORKSPACE  # options accepted: the next check is the workspace size
+    el, clip = _lib.FUNCTION_IDS["elman"], _lib.Options(0.5, 0.0, 0)
+    for pre, per_elem in (("frnn_fused_", 2 * 2), ("frnn_alt_", 2)):  # fused: values padded to whole dwords
+        assert getattr(lib, pre + "cache_bytes_opt")(el, 0, 8, 4, 1, 64, None) == 0
+        assert getattr(lib, pre + "cache_bytes_opt")(el, 0, 8, 4, 1, 64, ctypes.byref(clip)) == 8 * 4 * 64 * per_elem
+        assert getattr(lib, pre + "cache_bytes_opt")(0, 0, 8, 4, 1, 64, ctypes.byref(clip)) == \
+            getattr(lib, pre + "cache_bytes")(0, 0, 8, 4, 1, 64)
     for entry in ("frnn_fused_backward_opt", "frnn_alt_backward_opt"):
         o = _lib.Options(0.0, -2.0, 0)
         assert getattr(lib, entry)(0, 0, 8, 4, 1, 64, *([FAKE] * 11), 0, None, ctypes.byref(o)) == _lib.E_ARG

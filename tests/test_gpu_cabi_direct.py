@@ -42,8 +42,9 @@ def test_entry_points_with_raw_pointers(gpu, function, B, T, N, D, dtype, pre):
     lib = _open()
     Gr, Gw, _, Gt, S = FUNCTIONS[function]
     kdt = {"bfloat16": torch.bfloat16, "float32": torch.float32}[dtype]
-    inp = make_inputs(function, B, T, N, D, 5, init="randn", round_to=kdt if kdt != torch.float32 else None,
-                      grad_on="h" if function == "slstm" else "all")
+    inp = make_inputs(function, B, T, N, D, 5, init="randn", round_to=kdt if kdt != torch.float32 else None)
+    if function == "slstm":
+        inp["dstates"][3] = 0  # the stabiliser gets no cotangent in the native path
     dev = lambda x: x.to(gpu, kdt).contiguous()
     Wx, R, b = dev(inp["Wx"]), dev(inp["R"]), dev(inp["b"])
     s0 = dev(inp["states"].reshape(S, B, N, D))

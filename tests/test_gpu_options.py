@@ -22,7 +22,8 @@ CASES = [
     ("gru", 6, 8, 2, 128, "bfloat16", "hip_fused"),
     ("gru", 4, 7, 1, 256, "float32", "hip_fused"),
     ("slstm", 7, 10, 2, 192, "bfloat16", "hip_fused"),
-    ("elman", 9, 8, 1, 512, "bfloat16", "hip_fused"),
+    ("elman", 9, 8, 1, 512, "bfloat16", "hip_fused"),   # under forward_clipval: gate cache with the unclamped h
+    ("elman", 5, 7, 2, 64, "float32", "hip_fused"),
     ("lstm", 5, 6, 2, 64, "bfloat16", "hip"),
     ("gru", 3, 7, 2, 96, "float32", "hip"),
     ("slstm", 4, 6, 1, 64, "float32", "hip"),
@@ -33,20 +34,8 @@ CASES = [
 @pytest.mark.parametrize("function,B,T,N,D,dtype,backend", CASES)
 @pytest.mark.parametrize("options", OPTIONS, ids=lambda o: "+".join(sorted(o)))
 def test_options_match_oracle(gpu, options, function, B, T, N, D, dtype, backend):
-    if function == "elman" and "forward_clipval" in options:
-        pytest.skip("forward_clipval is refused for elman (see test_forward_clip_refused_for_elman)")
     print(f"case options {options} {backend} {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
     check_case(gpu, function, B, T, N, D, dtype, backend, seed=17, init="randn", options=options)
-
-
-def test_forward_clip_refused_for_elman(gpu):
-    from flashrnn_amd import FlashRNNConfig, flashrnn
-
-    cfg = FlashRNNConfig(backend="hip_fused", function="elman", dtype="bfloat16", head_dim=64, num_heads=1,
-                         forward_clipval=0.5)
-    Wx = torch.zeros(2, 3, 1, 1, 64, device=gpu)
-    with pytest.raises(ValueError, match="elman"):
-        flashrnn(Wx, torch.zeros(1, 1, 64, 64, device=gpu), torch.zeros(1, 1, 64, device=gpu), config=cfg)
 
 
 def test_options_off_are_bit_identical_to_plain_entry_points(gpu):

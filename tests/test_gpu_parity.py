@@ -166,35 +166,63 @@ def test_config1_lstm_fp32_forward(gpu):
     check_case(gpu, "lstm", 4, 256, 1, 64, "float32", "hip", seed=1001, init="zeros", backward=False)
 
 
-def test_config2_lstm_bf16_full_size(gpu):
-    print("case C2 full", flush=True)
-    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", "hip_fused", seed=1002, init="randn")
-
-
-def test_config2_alternating_full_size(gpu):
-    print("case C2 alt full", flush=True)
-    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", "hip", seed=1002, init="randn")
+# Full size, both backends; besides the fp32 oracle every bf16 configuration is also held against the
+# oracle run in torch.bfloat16 (the reference's vanilla backend in bf16): the HIP path must be closer.
+@pytest.mark.parametrize("backend", ["hip_fused", "hip"])
+def test_config2_lstm_bf16_full_size(gpu, backend):
+    print(f"case C2 full {backend}", flush=True)
+    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", backend, seed=1002, init="randn", vs_bf16_vanilla=True)
 
 
 @pytest.mark.parametrize("backend", ["hip_fused", "hip"])
 def test_config3_gru_bf16_full_size(gpu, backend):
     print(f"case C3 full {backend}", flush=True)
-    check_case(gpu, "gru", 16, 2048, 4, 128, "bfloat16", backend, seed=1003, init="zeros")
+    check_case(gpu, "gru", 16, 2048, 4, 128, "bfloat16", backend, seed=1003, init="zeros", vs_bf16_vanilla=True)
 
 
-def test_config4_slstm_bf16_full_size(gpu):
-    print("case C4 full", flush=True)
-    check_case(gpu, "slstm", 16, 4096, 4, 192, "bfloat16", "hip_fused", seed=1004, init="zeros",
-               forget_bias_linspace=True)
+@pytest.mark.parametrize("backend", ["hip_fused", "hip"])
+def test_config4_slstm_bf16_full_size(gpu, backend):
+    print(f"case C4 full {backend}", flush=True)
+    check_case(gpu, "slstm", 16, 4096, 4, 192, "bfloat16", backend, seed=1004, init="zeros",
+               forget_bias_linspace=True, grad_on="h", vs_bf16_vanilla=True)
 
 
 @pytest.mark.parametrize("backend", ["hip", "hip_fused"])
 def test_config5_elman_full_size(gpu, backend):
     print(f"case C5 full {backend}", flush=True)
-    check_case(gpu, "elman", 32, 1024, 1, 1024, "bfloat16", backend, seed=1005, init="zeros")
+    check_case(gpu, "elman", 32, 1024, 1, 1024, "bfloat16", backend, seed=1005, init="zeros", vs_bf16_vanilla=True)
 
 
 @pytest.mark.parametrize("N,D", [(24, 32), (12, 64), (6, 128), (3, 256), (1, 512)])
-def test_head_dim_sweep_points(gpu, N, D):
+def test_head_dim_sweep_points_full_length(gpu, N, D):
+    """The fused-path head-dim sweep of the fifth configuration (B = 16, T = 1024) at its real length."""
     print(f"case sweep N{N} D{D}", flush=True)
-    check_case(gpu, "lstm", 16, 64, N, D, "bfloat16", "hip_fused", seed=1006, init="zeros")
+    check_case(gpu, "lstm", 16, 1024, N, D, "bfloat16", "hip_fused", seed=1006, init="zeros", vs_bf16_vanilla=True)
+
+
+def test_slstm_mixed_fresh_and_running_elements(gpu):
+    """Initial n zero for some elements and not for others: the kernels take the first-step branch m' = i per
+    element, like the reference's native kernels (slstm_fused_pointwise.cuh:54-62); vanilla/slstm.py:21 would
+    take it for none of them.  The HIP path must match the per-element oracle and differ from the whole-tensor
+    one at the fresh elements."""
+    import torch
+    from flashrnn_amd import flashrnn
+    from oracle import flashrnn_oracle, make_inputs
+    from parity import assert_close
+
+    print("case slstm mixed n0", flush=True)
+    B, T, N, D = 6, 5, 2, 64
+    for backend in ("hip_fused", "hip"):
+        inp = make_inputs("slstm", B, T, N, D, 71, init="randn")
+        s0 = inp["states"]
+        s0[:, ::2, :, :, ::3] = 0.0              # every third unit of every other batch row starts fresh
+        inp["Wx"][::2, 0, 0, :, ::3] = -4.0      # and has an input gate well below log sigmoid(f) + m
+        dev = [inp[k].to(gpu) for k in ("Wx", "R", "b")]
+        out, _ = flashrnn(*dev, s0.to(gpu), function="slstm", backend=backend, dtype="float32")
+        per, _ = flashrnn_oracle(inp["Wx"].double(), inp["R"].double(), inp["b"].double(), s0.double(), "slstm",
+                                 slstm_per_element_first_step=True)
+        whole, _ = flashrnn_oracle(inp["Wx"].double(), inp["R"].double(), inp["b"].double(), s0.double(), "slstm")
+        got = out.float().cpu()
+        for k in range(4):
+            assert_close(f"{backend} state {k}", got[k], per[k], "float32", "state")
+        assert float((got[0].double() - whole[0]).abs().max()) > 1e-2

@@ -238,3 +238,67 @@ def test_cooperative_launch_gives_the_same_result(gpu, function, B, T, N, D, mon
     coop = run()
     for a, b in zip(plain, coop):
         assert torch.equal(a, b)
+
+
+@pytest.mark.parametrize("function,B,N,D,note", [
+    ("lstm", 80, 1, 768, "12 workgroups per head: an XCD of 32 compute units holds 2 groups, a launch 16; 20 groups"),
+    ("slstm", 100, 4, 192, "3 workgroups per head forward: 10 groups per XCD, 80 per launch; 100 groups"),
+    ("lstm", 70, 1, 320, "5 workgroups per head: 6 groups per XCD, 48 per launch; 18 groups at 4 rows"),
+])
+def test_launches_sized_by_the_room_of_an_xcd(gpu, monkeypatch, function, B, N, D, note):
+    """The workgroups of a group share one XCD, so a launch holds 8 * floor(32 / workgroups per head) groups;
+    calls with more groups run as several launches.  4-row tiles are forced to get many groups from a small
+    batch."""
+    from parity import check_case
+
+    print(f"case xcd room {function} B{B} N{N} D{D}: {note}", flush=True)
+    monkeypatch.setenv("FRNN_TILE_ROWS", "4")
+    check_case(gpu, function, B, 3, N, D, "bfloat16", "hip_fused", seed=27, init="randn")
+
+
+def test_batch_ranges_for_tensors_beyond_32_bit_offsets(gpu, monkeypatch):
+    """flashrnn() splits a fused problem whose tensors would reach 2 GiB into calls over batch ranges (the
+    kernels use 32-bit byte offsets); dR and db are summed over the ranges by autograd.  The limit is lowered
+    here so that a small problem splits into ranges of 16, 16 and 8 rows."""
+    import importlib
+
+    from parity import check_case
+
+    mod = importlib.import_module("flashrnn_amd.flashrnn")  # (the package attribute of that name is the function)
+    print("case batch ranges", flush=True)
+    B, T, N, D = 40, 6, 2, 64
+    monkeypatch.setattr(mod, "_FUSED_TENSOR_LIMIT", T * N * D * 2 * 6 * 17)
+    calls = []
+    real = mod._FlashRNNFunction.apply
+    monkeypatch.setattr(mod._FlashRNNFunction, "apply", lambda *a: (calls.append(a[0].shape[0]), real(*a))[1])
+    check_case(gpu, "lstm", B, T, N, D, "bfloat16", "hip_fused", seed=28, init="randn")
+    assert calls == [16, 16, 8], calls
+
+
+@pytest.mark.parametrize("backend", ["hip_fused", "hip"])
+def test_slstm_backward_through_the_carried_state_of_two_calls(gpu, backend):
+    """Truncated sequences: the second call starts from the last states of the first and autograd carries its
+    ds0 (cotangents on h, c and n; 0 on the stabiliser m) back into the first call.  In fp32 the result must
+    equal the oracle over the whole sequence (stabiliser held constant, as the native adjoint holds it)."""
+    from flashrnn_amd import flashrnn
+    from oracle import flashrnn_oracle_backward
+    from parity import assert_close
+
+    print(f"case slstm two chunks {backend}", flush=True)
+    B, T, N, D, T1 = 5, 12, 2, 64, 7
+    inp = make_inputs("slstm", B, T, N, D, 29, init="randn", grad_on="all")
+    inp["dstates"][3] = 0
+    leaves = [inp[k].to(gpu).requires_grad_(True) for k in ("Wx", "R", "b", "states")]
+    Wx, R, b, s0 = leaves
+    o1, last1 = flashrnn(Wx[:, :T1], R, b, s0, function="slstm", backend=backend, dtype="float32")
+    o2, _ = flashrnn(Wx[:, T1:], R, b, last1, function="slstm", backend=backend, dtype="float32")
+    out = torch.cat([o1, o2], dim=2)
+    grads = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(gpu))
+    torch.cuda.synchronize()
+    ref_out, ref_g = flashrnn_oracle_backward(*[inp[k].double() for k in ("Wx", "R", "b", "states")], "slstm",
+                                              inp["dstates"].double(), slstm_per_element_first_step=True,
+                                              slstm_detach_m=True)
+    for k in range(4):
+        assert_close(f"state {k}", out[k].detach().cpu(), ref_out[k], "float32", "state")
+    for name, g, r in zip(("dWx", "dR", "db", "ds0"), grads, ref_g):
+        assert_close(name, g.cpu(), r, "float32", "token")

@@ -362,3 +362,146 @@ def test_options_noop_limits(function):
     # forward clamp: every stored h lies inside the interval and the untouched steps are unchanged
     o4, _ = flashrnn_oracle_backward(*a, function, ds, **base, forward_clipval=0.25)
     assert float(o4[0].abs().max()) <= 0.25 + 1e-15
+
+
+# ---- sLSTM: what the native adjoint does beyond plain autograd -------------------------------------
+def test_slstm_adjoint_for_cotangents_on_c_and_n_is_autograd_with_the_stabiliser_held_constant():
+    """The explicit reverse scan (the native adjoint, slstm_fused_pointwise.cuh:117-186) with cotangents on
+    every state equals float64 autograd of the forward with the stabiliser m detached, and differs from
+    plain autograd, which also differentiates exp(-m) in c and n.  For a cotangent on h alone the two
+    autograd variants agree (h does not depend on m).  Initial n > 1 keeps max(., 1) away from its kink."""
+    B, T, N, D = 3, 6, 2, 5
+    inp = make_inputs("slstm", B, T, N, D, seed=31, init="randn", grad_on="all")
+    Wx, R, b, s0, ds = (inp[k].to(DT) for k in ("Wx", "R", "b", "states", "dstates"))
+    ds[3] = 0  # m itself gets no cotangent anywhere in the native path
+    kw = dict(slstm_per_element_first_step=True)
+    out_d, g_det = flashrnn_oracle_backward(Wx, R, b, s0, "slstm", ds, slstm_detach_m=True, **kw)
+    out_p, g_plain = flashrnn_oracle_backward(Wx, R, b, s0, "slstm", ds, **kw)
+    out_m, g_man = flashrnn_oracle_fwbw_manual(Wx, R, b, s0, "slstm", ds)
+    assert torch.equal(out_d, out_p) and torch.allclose(out_m, out_d, atol=1e-12)
+    for k, (x, y) in enumerate(zip(g_man, g_det)):
+        assert torch.allclose(x, y, atol=1e-10), (k, float((x - y).abs().max()))
+    assert float(g_det[3][3].abs().max()) == 0.0 and float(g_man[3][3].abs().max()) == 0.0   # d/dm0 = 0
+    assert float((g_plain[0] - g_det[0]).abs().max()) > 1e-2   # plain autograd is a different function here
+    # zero initial state: n' = max(0 + 1, 1) ties at the first step; the native adjoint (and the detached
+    # autograd, whose guard is transparent) takes slope 1 there, so even d/dn0 agrees
+    z0 = torch.zeros_like(s0)
+    _, gz_det = flashrnn_oracle_backward(Wx, R, b, z0, "slstm", ds, slstm_detach_m=True, **kw)
+    _, gz_man = flashrnn_oracle_fwbw_manual(Wx, R, b, z0, "slstm", ds)
+    for k, (x, y) in enumerate(zip(gz_man, gz_det)):
+        assert torch.allclose(x, y, atol=1e-10), ("zero init", k, float((x - y).abs().max()))
+    ds_h = ds.clone()
+    ds_h[1:] = 0
+    _, a = flashrnn_oracle_backward(Wx, R, b, s0, "slstm", ds_h, slstm_detach_m=True, **kw)
+    _, c = flashrnn_oracle_backward(Wx, R, b, s0, "slstm", ds_h, **kw)
+    for k in range(3):
+        assert torch.allclose(a[k], c[k], atol=1e-10), k
+
+
+def test_slstm_backward_through_carried_state_of_two_chunks():
+    """Truncated sequences carry (h, c, n, m) from chunk to chunk; the gradient of the whole equals the
+    chunk-wise reverse scan in which the second chunk's ds0 is the first chunk's extra cotangent on its
+    last states (c and n included: the path that only a cotangent on c, n exercises)."""
+    B, T, N, D = 2, 8, 1, 4
+    inp = make_inputs("slstm", B, T, N, D, seed=32, init="randn", grad_on="h")
+    Wx, R, b, s0, ds = (inp[k].to(DT) for k in ("Wx", "R", "b", "states", "dstates"))
+    _, (dWx, dR, db, ds0) = flashrnn_oracle_fwbw_manual(Wx, R, b, s0, "slstm", ds)
+    T1 = 5
+    out1, _ = flashrnn_oracle_fwbw_manual(Wx[:, :T1], R, b, s0, "slstm", ds[:, :, :T1])
+    mid = out1[:, :, -1:]
+    _, (dWx2, dR2, db2, dmid) = flashrnn_oracle_fwbw_manual(Wx[:, T1:], R, b, mid, "slstm", ds[:, :, T1:])
+    ds1 = ds[:, :, :T1].clone()
+    ds1[:, :, -1] += dmid[:, :, 0]
+    _, (dWx1, dR1, db1, ds0c) = flashrnn_oracle_fwbw_manual(Wx[:, :T1], R, b, s0, "slstm", ds1)
+    assert float(dmid[1].abs().max()) > 0 and float(dmid[2].abs().max()) > 0
+    assert torch.allclose(torch.cat([dWx1, dWx2], 1), dWx, atol=1e-11)
+    assert torch.allclose(dR1 + dR2, dR, atol=1e-11) and torch.allclose(db1 + db2, db, atol=1e-11)
+    assert torch.allclose(ds0c, ds0, atol=1e-11)
+
+
+def test_slstm_backward_under_forward_clip_closed_form_scalar_cell():
+    """A scalar sLSTM cell, zero initial state, two steps, forward_clipval active at step 1.  Every quantity
+    is written out by hand from the native definitions: the forward pass clamps h after the cache is taken
+    (slstm_fused_pointwise.cuh:96-109) and the adjoint reads the stored, clamped h where the unclamped
+    derivative has o c / n (:154-166: dn -= dy/n * h, do = (1 - o) h dy), while dc keeps o/n."""
+    sig = lambda x: 1.0 / (1.0 + math.exp(-x))
+    lsig = lambda x: -math.log1p(math.exp(-x))
+    clamp = lambda x, v: max(-v, min(v, x))
+    v = 0.3
+    w1, w2 = [0.4, 1.1, 1.7, 2.0], [-0.3, 0.6, -0.9, 0.5]      # Wx of the gates i, f, z, o at steps 1 and 2
+    r, bb = [0.7, -0.5, 1.3, 0.9], [0.1, 0.2, -0.1, 0.05]     # recurrent weight and bias per gate
+    g1, g2 = 0.8, -1.2                                         # cotangents of h_1, h_2
+    # step 1: h_0 = 0, n_0 = 0 -> m_1 = i_1, ig = 1, c_1 = z_1, n_1 = 1
+    i1, f1 = w1[0] + bb[0], w1[1] + bb[1]
+    z1, o1 = math.tanh(w1[2] + bb[2]), sig(w1[3] + bb[3])
+    m1, ig1, fg1 = i1, 1.0, math.exp(lsig(f1) - i1)
+    c1, n1 = z1, 1.0
+    y1 = o1 * c1 / n1
+    h1 = clamp(y1, v)
+    assert h1 == v and y1 > v                                  # the clamp is active
+    # step 2
+    i2, f2 = w2[0] + r[0] * h1 + bb[0], w2[1] + r[1] * h1 + bb[1]
+    z2, o2 = math.tanh(w2[2] + r[2] * h1 + bb[2]), sig(w2[3] + r[3] * h1 + bb[3])
+    lfm = lsig(f2) + m1
+    m2 = max(i2, lfm)
+    ig2, fg2 = math.exp(i2 - m2), math.exp(lfm - m2)
+    c2 = fg2 * c1 + ig2 * z2
+    n2 = max(fg2 * n1 + ig2, 1.0)
+    y2 = o2 * c2 / n2
+    h2 = clamp(y2, v)
+    # reverse step 2
+    dy = g2
+    dc, dn = dy / n2 * o2, -dy / n2 * h2
+    dg2 = [ig2 * (z2 * dc + dn), fg2 * (dc * c1 + dn * n1) * (1 - sig(f2)), dc * ig2 * (1 - z2 * z2), (1 - o2) * h2 * dy]
+    dc1, dn1 = fg2 * dc, fg2 * dn
+    dh1 = sum(rg * d for rg, d in zip(r, dg2))
+    # reverse step 1 (c_0 = n_0 = 0, n_1 = 1)
+    dy = g1 + dh1
+    dc, dn = dc1 + dy * o1, dn1 - dy * h1
+    dg1 = [ig1 * (z1 * dc + dn), 0.0, dc * ig1 * (1 - z1 * z1), (1 - o1) * h1 * dy]
+    want_dR = [d * h1 for d in dg2]                            # h_0 = 0: only step 2 contributes
+    want_db = [a + c for a, c in zip(dg1, dg2)]
+    want_ds0 = [sum(rg * d for rg, d in zip(r, dg1)), fg1 * dc, fg1 * dn, 0.0]
+
+    t = lambda x: torch.tensor(x, dtype=torch.float64)
+    Wx = t([w1, w2]).reshape(1, 2, 4, 1, 1)
+    R = t(r).reshape(4, 1, 1, 1)
+    b = t(bb).reshape(4, 1, 1)
+    s0 = torch.zeros(4, 1, 1, 1, 1, dtype=torch.float64)
+    ds = torch.zeros(4, 1, 2, 1, 1, dtype=torch.float64)
+    ds[0, 0, 0], ds[0, 0, 1] = g1, g2
+    out, (dWx, dR, db, ds0) = flashrnn_oracle_fwbw_manual(Wx, R, b, s0, "slstm", ds, forward_clipval=v)
+    assert torch.allclose(out[:, 0, 0].flatten(), t([h1, c1, n1, m1]), atol=1e-14)
+    assert torch.allclose(out[:, 0, 1].flatten(), t([h2, c2, n2, m2]), atol=1e-14)
+    assert torch.allclose(dWx.flatten(), t(dg1 + dg2), atol=1e-13)
+    assert torch.allclose(dR.flatten(), t(want_dR), atol=1e-13)
+    assert torch.allclose(db.flatten(), t(want_db), atol=1e-13)
+    assert torch.allclose(ds0.flatten(), t(want_ds0), atol=1e-13)
+    # and the clamp does matter for the gradient: with the unclamped h in the adjoint dWx differs
+    _, (dWx_plain, _, _, _) = flashrnn_oracle_fwbw_manual(Wx, R, b, s0, "slstm", ds)
+    assert float((dWx_plain - dWx).abs().max()) > 1e-3
+
+
+def test_slstm_first_step_branch_mixed_initial_n_differs_between_native_and_vanilla():
+    """vanilla/slstm.py:21 takes m' = i only when EVERY n is zero; the native kernels (and the HIP kernels)
+    decide per element (slstm_fused_pointwise.cuh:54-62).  With some initial n zero and some not the two
+    differ, exactly at the elements whose n is zero: there vanilla uses max(i, logsig(f) + m)."""
+    inp = make_inputs("slstm", 2, 2, 1, 4, seed=33, init="randn")
+    s0 = inp["states"].clone()
+    s0[:, 0, 0, 0, :2] = 0.0            # two elements of batch row 0 start fresh: h = c = n = m = 0
+    inp["Wx"][0, 0, 0, 0, :2] = -4.0    # their input gate is far below log sigmoid(f) + m
+    whole, _ = flashrnn_oracle(inp["Wx"], inp["R"], inp["b"], s0, "slstm")
+    per, _ = flashrnn_oracle(inp["Wx"], inp["R"], inp["b"], s0, "slstm", slstm_per_element_first_step=True)
+    diff = (whole - per).abs()[:, :, 0]                       # first step, [S,B,N,D]
+    raw = inp["Wx"][:, 0] + torch.einsum("bnp,gndp->bgnd", s0[0, :, 0], inp["R"]) + inp["b"][None]
+    fresh_and_lfm_wins = (s0[2, :, 0] == 0) & (torch.nn.functional.logsigmoid(raw[:, 1]) + s0[3, :, 0] > raw[:, 0])
+    assert bool(fresh_and_lfm_wins.any())
+    assert bool((diff[3] > 0)[fresh_and_lfm_wins].all())       # m' differs where the fresh element's i loses
+    assert float(diff[3][~fresh_and_lfm_wins].max()) == 0.0    # and nowhere else
+    # h differs there too: n' = max(ig, 1) = 1 hides the scale exp(i - m') < 1 that c' = ig tanh(z) carries
+    i, f, z, o = raw.unbind(1)
+    fresh = fresh_and_lfm_wins
+    h_native = torch.sigmoid(o) * torch.tanh(z)                # the closed form of a first step: m' = i, ig = 1
+    h_vanilla = h_native * torch.exp(i - torch.nn.functional.logsigmoid(f))   # m' = logsig(f) + 0, ig = exp(i - m')
+    assert torch.allclose(per[0, :, 0][fresh], h_native[fresh], atol=1e-6)
+    assert torch.allclose(whole[0, :, 0][fresh], h_vanilla[fresh], atol=1e-6)
