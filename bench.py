@@ -156,6 +156,9 @@ def main():
     ap.add_argument("--backend", default=None, choices=["hip_fused", "hip"])
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-alt", action="store_true", help="skip the other-backend comparison leg")
+    ap.add_argument("--copy-calibration", action="store_true",
+                    help="also run one plain device-to-device copy of 256 MiB (a kernel of known traffic: 256 MiB read, "
+                         "256 MiB written) so that a counter profile of this command holds its own calibration")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py measures one GPU: the recurrent path has no multi-GPU leg in this build "
@@ -177,6 +180,12 @@ def main():
     backend = args.backend or ("hip" if args.workload == "C5" else "hip_fused")
     tokens = w["B"] * w["T"]
 
+    if args.copy_calibration:
+        src = torch.arange(64 << 20, dtype=torch.float32, device=device)  # 256 MiB
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     ms, kern = run_gpu(w, backend, args.steps, args.warmup, device)
 
     # dominant kernel and its roofline: 2*N*G_r*D^2 flops per token in the forward scan and the

@@ -403,7 +403,9 @@ def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     if config.backend != "hip_fused":
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
     es = 4 if config.dtype == "float32" else 2
-    per_row = T * N * D * es * max(Gw, config.num_states, 6 if training else 0)  # at most 6 cached values per element
+    f_id, d_id = _lib.FUNCTION_IDS[config.function], _lib.DTYPE_IDS[config.dtype]
+    cache_row = _lib.load_library().frnn_fused_cache_bytes_opt(f_id, d_id, 1, T, N, D, _options(config)) if training else 0
+    per_row = max(T * N * D * es * max(Gw, config.num_states), cache_row)  # bytes per batch row of the largest tensor
     rows = max(1, (_FUSED_TENSOR_LIMIT - 1) // per_row)
     if rows >= B:
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
