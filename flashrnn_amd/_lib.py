@@ -21,7 +21,7 @@ class Options(ctypes.Structure):
     """frnn_options of include/flashrnn_hip.h (0 / False = option off)."""
 
     _fields_ = [("forward_clipval", ctypes.c_float), ("gradient_recurrent_clipval", ctypes.c_float),
-                ("gradient_recurrent_cut", c_int)]
+                ("gradient_recurrent_cut", c_int), ("recompute", c_int)]
 
 
 _P6 = [c_int] * 6
@@ -53,6 +53,9 @@ _SIGNATURES = {
     "frnn_alt_backward_opt": (c_int, _BWD + [POINTER(Options)]),
     "frnn_fused_cache_bytes_opt": (c_size_t, _P6 + [POINTER(Options)]),
     "frnn_alt_cache_bytes_opt": (c_size_t, _P6 + [POINTER(Options)]),
+    "frnn_fused_recompute_supported": (c_int, [c_int] * 5),
+    "frnn_fused_workspace_bytes_opt": (c_size_t, _P6 + [c_int, POINTER(Options)]),
+    "frnn_fused_backward_recompute": (c_int, _P6 + [c_void_p] * 11 + [c_size_t, c_void_p, POINTER(Options)]),
     "frnn_fused_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),
     "frnn_alt_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),
     "frnn_fused_forward_static_max_bytes": (c_size_t, []),

@@ -75,6 +75,10 @@ static const Plan kBwd3B[] = {FRNN_BWD_PLANS_GR3_BF16(FRNN_ROW)};
 static const Plan kBwd3F[] = {FRNN_BWD_PLANS_GR3_F32(FRNN_ROW)};
 static const Plan kBwd1B[] = {FRNN_BWD_PLANS_GR1_BF16(FRNN_ROW)};
 static const Plan kBwd1F[] = {FRNN_BWD_PLANS_GR1_F32(FRNN_ROW)};
+static const Plan kRc4B[] = {FRNN_BWD_RC_PLANS_GR4_BF16(FRNN_ROW)};
+static const Plan kRc4F[] = {FRNN_BWD_RC_PLANS_GR4_F32(FRNN_ROW)};
+static const Plan kRc3B[] = {FRNN_BWD_RC_PLANS_GR3_BF16(FRNN_ROW)};
+static const Plan kRc3F[] = {FRNN_BWD_RC_PLANS_GR3_F32(FRNN_ROW)};
 #undef FRNN_ROW
 
 bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* out) {
@@ -86,19 +90,23 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
     if (GR == 4) { if (dtype == FRNN_F32) PICK(kFwd4F) else if (function == FRNN_SLSTM) PICK(kFwdSB) else PICK(kFwd4B) }
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kFwd3B) else PICK(kFwd3F) }
     else { if (dtype != FRNN_F32) PICK(kFwd1B) else PICK(kFwd1F) }
-  } else {
+  } else if (backward == 1) {
     if (GR == 4) { if (dtype != FRNN_F32) PICK(kBwd4B) else PICK(kBwd4F) }
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kBwd3B) else PICK(kBwd3F) }
     else { if (dtype != FRNN_F32) PICK(kBwd1B) else PICK(kBwd1F) }
+  } else {  // reverse scan in recompute mode
+    if (GR == 4) { if (dtype != FRNN_F32) PICK(kRc4B) else PICK(kRc4F) }
+    else if (GR == 3) { if (dtype != FRNN_F32) PICK(kRc3B) else PICK(kRc3F) }
+    else return false;
   }
 #undef PICK
   const Plan* dflt = nullptr;
   for (size_t i = 0; i < n; ++i) {
     if (tab[i].D != D) continue;
-    if (tab[i].variant == variant) { *out = tab[i]; return true; }
+    if (tab[i].variant == variant) { *out = tab[i]; out->recompute = backward == 2; return true; }
     if (tab[i].variant == 0) dflt = &tab[i];
   }
-  if (dflt) { *out = *dflt; return true; }
+  if (dflt) { *out = *dflt; out->recompute = backward == 2; return true; }
   return false;
 }
 
@@ -205,9 +213,10 @@ static void gate_leave(LaunchGate* g, hipStream_t st) {
 
 // fx is the cell the kernels are instantiated for: the function itself, except that an Elman cell under
 // forward_clipval runs as FRNN_ELMAN_CLIP (one cached value per element: the unclamped h).
-struct Opts { float h_clip, g_clip; int cut; int fx; };
+// rc: the gate cache is left out (forward) / rebuilt (backward): only for cells that have one.
+struct Opts { float h_clip, g_clip; int cut; int fx; int rc; };
 static int parse_opts(const frnn_options* o, int function, Opts* out) {
-  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0; out->fx = function;
+  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0; out->fx = function; out->rc = 0;
   if (!o) return 0;
   if (o->forward_clipval != o->forward_clipval || o->gradient_recurrent_clipval != o->gradient_recurrent_clipval ||
       o->forward_clipval < 0.f || o->gradient_recurrent_clipval < 0.f)
@@ -215,6 +224,7 @@ static int parse_opts(const frnn_options* o, int function, Opts* out) {
                 (double)o->gradient_recurrent_clipval);
   out->h_clip = o->forward_clipval; out->g_clip = o->gradient_recurrent_clipval; out->cut = o->gradient_recurrent_cut != 0;
   if (function == FRNN_ELMAN && out->h_clip > 0.f) out->fx = FRNN_ELMAN_CLIP;
+  out->rc = o->recompute != 0 && function != FRNN_ELMAN;  // (elman caches nothing, or one value under forward_clipval)
   return 0;
 }
 
@@ -423,7 +433,7 @@ size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int 
 size_t frnn_fused_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt) {
   Opts o;
   if (check_problem(function, dtype, B, T, N, D) || parse_opts(opt, function, &o)) return 0;
-  return fused_cache_bytes_of(o.fx, dtype, B, T, N, D);
+  return o.rc ? 0 : fused_cache_bytes_of(o.fx, dtype, B, T, N, D);
 }
 
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
@@ -431,6 +441,16 @@ size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, 
   Plan p;
   if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p)) return 0;
   return backward ? carve_fused_bwd(nullptr, function, dtype, B, T, N, D, p).total
+                  : carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
+}
+
+size_t frnn_fused_workspace_bytes_opt(int function, int dtype, int B, int T, int N, int D, int backward,
+                                      const frnn_options* opt) {
+  Opts o;
+  if (check_problem(function, dtype, B, T, N, D) || parse_opts(opt, function, &o)) return 0;
+  Plan p;
+  if (!find_plan(o.fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward ? (o.rc ? 2 : 1) : 0, &p)) return 0;
+  return backward ? carve_fused_bwd(nullptr, o.fx, dtype, B, T, N, D, p).total
                   : carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
 }
 
@@ -462,7 +482,12 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   e = check_fused_sizes(fx, dtype, B, T, N, D);
   if (e) return e;
   CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
-  const bool need_cache = training && cell_dims(fx).NC > 0;
+  if (o.rc) {
+    Plan prc;
+    if (!find_plan(fx, dtype, D, 0, 2, &prc))
+      return fail(FRNN_E_UNSUPPORTED, "no recompute-mode kernel for function %d dtype %d head dim %d", function, dtype, D);
+  }
+  const bool need_cache = training && cell_dims(fx).NC > 0 && !o.rc;
   if (need_cache) CHECK_PTR(cache)
   hipStream_t st = (hipStream_t)stream;
   FusedFwdWs w = carve_fused_fwd(workspace, dtype, B, N, D, p);
@@ -555,13 +580,14 @@ int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
                                  workspace, workspace_bytes, stream, nullptr);
 }
 
-int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
-                            const void* R, const void* b, const void* s0, const void* states,
-                            const void* cache, const void* dstates,
-                            void* dWx, void* ds0, float* dR, float* db,
-                            void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
+// The backward call proper.  Recompute mode (opt->recompute, a cell that has a gate cache): `Wx` and `b` are
+// read instead of `cache`, which is ignored.
+static int fused_backward_impl(int function, int dtype, int B, int T, int N, int D,
+                               const void* Wx, const void* R, const void* b, const void* s0, const void* states,
+                               const void* cache, const void* dstates,
+                               void* dWx, void* ds0, float* dR, float* db,
+                               void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
   g_err[0] = 0;
-  (void)b;
   int e = check_problem(function, dtype, B, T, N, D);
   if (e) return e;
   Opts o;
@@ -570,13 +596,15 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   const int fx = o.fx;
   const CellDims c = cell_dims(fx);
   Plan p;
-  if (!find_plan(fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 1, &p))
-    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  if (!find_plan(fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), o.rc ? 2 : 1, &p))
+    return fail(FRNN_E_UNSUPPORTED, "no fused%s kernel for function %d dtype %d head dim %d", o.rc ? " recompute-mode" : "",
+                function, dtype, D);
   e = check_fused_sizes(fx, dtype, B, T, N, D);
   if (e) return e;
   CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
   CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
-  if (c.NC > 0) CHECK_PTR(cache)
+  if (o.rc) { CHECK_PTR(Wx) CHECK_PTR(b) }
+  else if (c.NC > 0) CHECK_PTR(cache)
   const FusedBwdWs w = carve_fused_bwd(workspace, fx, dtype, B, T, N, D, p);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
@@ -596,7 +624,8 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
     if (per_launch < 1) return fail(FRNN_E_DEVICE, "an eighth of the device has fewer compute units than the %d workgroups of one head", p.kw);
   }
   BwdArgs a;
-  a.Rt = w.Rt; a.s0 = s0; a.states = states; a.cache = cache; a.dstates = dstates;
+  a.Rt = w.Rt; a.s0 = s0; a.states = states; a.cache = o.rc ? nullptr : cache; a.dstates = dstates;
+  a.Wx = Wx; a.R = R; a.b = b;
   a.dWx = dWx; a.dgx = w.dgx; a.ds0 = ds0; a.dbp = w.dbp;
   a.ll = w.ll; a.status = w.status;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
@@ -628,6 +657,41 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
   gate_leave(gate, st);
   if (e) return hip_fail(e, "fused backward launch");
   return weight_grads(fx, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, bt, dR, db, st);
+}
+
+int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
+                            const void* R, const void* b, const void* s0, const void* states,
+                            const void* cache, const void* dstates,
+                            void* dWx, void* ds0, float* dR, float* db,
+                            void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
+  if (opt && opt->recompute && function != FRNN_ELMAN) {
+    g_err[0] = 0;
+    return fail(FRNN_E_ARG, "recompute mode has no gate cache: call frnn_fused_backward_recompute, which takes Wx");
+  }
+  return fused_backward_impl(function, dtype, B, T, N, D, nullptr, R, b, s0, states, cache, dstates, dWx, ds0, dR, db,
+                             workspace, workspace_bytes, stream, opt);
+}
+
+int frnn_fused_backward_recompute(int function, int dtype, int B, int T, int N, int D,
+                                  const void* Wx, const void* R, const void* b, const void* s0, const void* states,
+                                  const void* dstates, void* dWx, void* ds0, float* dR, float* db,
+                                  void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
+  frnn_options o2;
+  memset(&o2, 0, sizeof(o2));
+  if (opt) o2 = *opt;
+  o2.recompute = 1;
+  if (Wx && Wx == dWx) { g_err[0] = 0; return fail(FRNN_E_ARG, "dWx must not be Wx: the scan reads Wx two steps ahead of its dWx stores"); }
+  return fused_backward_impl(function, dtype, B, T, N, D, Wx, R, b, s0, states, nullptr, dstates, dWx, ds0, dR, db,
+                             workspace, workspace_bytes, stream, &o2);
+}
+
+int frnn_fused_recompute_supported(int function, int dtype, int B, int N, int D) {
+  int e = frnn_fused_supported(function, dtype, B, N, D);
+  if (e) return e;
+  Plan p;
+  if (function != FRNN_ELMAN && !find_plan(function, dtype, D, 0, 2, &p))
+    return fail(FRNN_E_UNSUPPORTED, "no recompute-mode kernel for function %d dtype %d head dim %d", function, dtype, D);
+  return 0;
 }
 
 // ---- alternating --------------------------------------------------------------------------------------

@@ -50,6 +50,9 @@ struct BwdArgs {
   float g_clip;  // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip] (gradient_recurrent_clipval)
   int cut;       // != 0: no gradient through R h (gradient_recurrent_cut)
   long long* trace;  // phase cycle sums per wave; only written by -DFRNN_TRACE builds
+  // recompute mode (kernels instantiated with RC = true): no gate cache; the gates of step t are rebuilt from
+  // Wx_t, b and R h_(t-1), with h_(t-1) read back from the stored states
+  const void* Wx; const void* R; const void* b;
 };
 
 // words (64-bit for fp32 storage, 32-bit otherwise) of one inbox area of one group:
@@ -73,10 +76,11 @@ constexpr int bwd_lds_tiles(int GR, int D, int WAVES, int UTW, int KW, int esize
   if (KW - 1 > 8) return (want + 3) / 4 * 4 < room / 4 * 4 ? (want + 3) / 4 * 4 : room / 4 * 4;
   return want < room ? want : room;
 }
-constexpr size_t bwd_lds_bytes(int GR, int D, int WAVES, int UTW, int KW, int esize) {
+constexpr size_t bwd_lds_bytes(int GR, int D, int WAVES, int UTW, int KW, int esize, bool rc = false) {
   const int KM = esize == 4 ? 4 : 32, FRB = esize == 4 ? 4 : 16;
   const int KS = GR * (D / KW) / KM;
-  return (size_t)2 * 16 * GR * (D / KW) * esize + (size_t)WAVES * bwd_lds_tiles(GR, D, WAVES, UTW, KW, esize) * UTW * KS * 64 * FRB;
+  return (size_t)2 * 16 * GR * (D / KW) * esize + (size_t)WAVES * bwd_lds_tiles(GR, D, WAVES, UTW, KW, esize) * UTW * KS * 64 * FRB +
+         (rc ? (size_t)2 * 16 * D * esize : 0);  // recompute mode: two buffers for h_(t-1) of the whole head
 }
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag_at(const T* p);
@@ -84,7 +88,15 @@ template <> __device__ __forceinline__ bf16x8 load_frag_at<bf16_t>(const bf16_t*
 template <> __device__ __forceinline__ f16x8 load_frag_at<half_t>(const half_t* p) { return *reinterpret_cast<const f16x8*>(p); }
 template <> __device__ __forceinline__ float load_frag_at<float>(const float* p) { return *p; }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR>
+// RC = true: recompute mode.  Nothing is cached by the forward pass; the reverse scan rebuilds the gates of
+// step t-1 while the partial sums of step t travel between the workgroups (the rebuild does not depend on
+// the running cotangent, so it is off the chain of dependent steps): h_(t-2) of the whole head comes back
+// from the stored states (a few bytes per thread, fetched two steps ahead) into LDS, the forward product
+// R h_(t-2) of the own units runs on MFMA with R resident beside R^T, and the forward gate math yields what
+// the cache would have held.  For the sLSTM the stabilised gates exp(i - m') and exp(logsig(f) + m - m')
+// are rebuilt from the stored (rounded) m_(t-2); the larger of the two is still exactly 1, the other carries
+// the rounding error of m_(t-2) as a relative error (2^-9 |m| for bf16).
+template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool RC = false>
 __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
@@ -104,7 +116,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   // so as few rounds as 16 words per lane and probe allow, of equal size (no dummy loads)
   constexpr int RC_MAX = 16 / (UTW * (TR / 4)) > 0 ? 16 / (UTW * (TR / 4)) : 1;
   constexpr int ROUNDS = KW == 1 ? 1 : (KW - 1 + RC_MAX - 1) / RC_MAX;
-  constexpr int RC = KW == 1 ? 1 : (KW - 1 + ROUNDS - 1) / ROUNDS;
+  constexpr int PSRC = KW == 1 ? 1 : (KW - 1 + ROUNDS - 1) / ROUNDS;  // sources polled per round
   constexpr size_t INW = bwd_inbox_words(D, KW);
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
   constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
@@ -117,6 +129,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   // this lane's fragments of the last RLD destination tiles: [wave][tile][u][ks][lane]
   Frag* const rl = reinterpret_cast<Frag*>(smem_raw + (size_t)2 * 16 * KDL * sizeof(T)) +
                    (size_t)(threadIdx.x >> 6) * RLD * UTW * KS * 64 + (threadIdx.x & 63);
+  // recompute mode: h_(t-1) of the whole head, 16 x D in fragment order, two buffers (behind the R^T tiles)
+  constexpr int KSF = D / X::KM;   // k-steps of the forward product
+  T* const hb0 = reinterpret_cast<T*>(smem_raw + bwd_lds_bytes(GR, D, WAVES, UTW, KW, (int)sizeof(T)));
+  T* const hb1 = hb0 + 16 * D;
   // a static LDS word, not a slice of the dynamic array: through a pointer computed from the
   // dynamic array the compiler reads the flag with a flat load, which has to wait for every global
   // load in flight (measured: the operand prefetch's full HBM latency, once per step)
@@ -144,6 +160,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * (NC ? NCP : 0) * ES);
   const rsrc_t rDw = make_rsrc(a.dWx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rDx = make_rsrc(a.dgx, (size_t)B * Tn * ND * ES);
+  const rsrc_t rWx = make_rsrc(a.Wx, RC ? (size_t)B * Tn * GW * ND * ES : 0);
 
   int ub[UTW];
   unsigned wx_v[UTW], st_v[UTW], s0_v[UTW], ca_v[UTW];
@@ -176,8 +193,45 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     }
   }
 
-  // zero both LDS buffers once (rows beyond the tile are never written) and the flag
+  // recompute mode: rows of R of the own unit tiles (the forward kernel's resident operand) and the biases
+  constexpr int GX = GT - GR > 0 ? GT - GR : 1;
+  constexpr bool BIAS_C = O::E == 4;
+  Frag rfw[RC ? UTW : 1][RC ? GR : 1][RC ? KSF : 1];
+  f32x4 biasc[RC && BIAS_C ? UTW : 1][GR];
+  float bown[RC ? UTW : 1][GR][BIAS_C ? 1 : O::E];
+  float bxr[RC ? UTW : 1][O::E][GX];
+  if constexpr (RC) {
+    const T* __restrict__ Rm = static_cast<const T*>(a.R);
+    const T* __restrict__ bias_g = static_cast<const T*>(a.b);
+    typedef typename X::Vec4 Vec4;
+#pragma unroll
+    for (int u = 0; u < UTW; ++u) {
+#pragma unroll
+      for (int g = 0; g < GR; ++g) {
+        const T* row = Rm + ((size_t)(g * N + n) * D + ub[u] + r16) * D;
+#pragma unroll
+        for (int ks = 0; ks < KSF; ++ks) rfw[u][g][ks] = load_frag<T>(row, ks, q4);
+        if constexpr (BIAS_C) {
+          float v[4];
+          unpack4<T>(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
+          biasc[u][g] = f32x4{v[0], v[1], v[2], v[3]};
+        } else {
+#pragma unroll
+          for (int e = 0; e < O::E; ++e) bown[u][g][e] = (float)bias_g[(size_t)(g * N + n) * D + ub[u] + esub + e];
+        }
+      }
+#pragma unroll
+      for (int e = 0; e < O::E; ++e)
+#pragma unroll
+        for (int g = GR; g < GT; ++g) bxr[u][e][g - GR] = (float)bias_g[(size_t)(g * N + n) * D + ub[u] + esub + e];
+    }
+  }
+
+  // zero the LDS buffers once (rows beyond the tile are never written) and the flag
   for (int idx = tid; idx < (2 * 16 * KDL * (int)sizeof(T)) / 4; idx += NT) reinterpret_cast<unsigned*>(smem_raw)[idx] = 0u;
+  if constexpr (RC) {
+    for (int idx = tid; idx < (2 * 16 * D * (int)sizeof(T)) / 4; idx += NT) reinterpret_cast<unsigned*>(hb0)[idx] = 0u;
+  }
   if (tid == 0) dead_flag_word = 0;
 
   float ds[UTW][E][S];
@@ -200,21 +254,56 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 
   // operands of one step.  s_t is not among them: it is the s_(t-1) of the step before (kept in
   // registers, `sn` below), so only the first step loads it
-  struct Pre { Dw<NWC> cache[UTW]; Dw<ND_> sp[UTW][S], dso[UTW][S]; };
+  // recompute mode: h_(t-1) of the whole head (TR rows x D) goes from the stored states to LDS in pieces of HC
+  // consecutive elements of one row (a power of two, at most 8: a piece never straddles an 8-element group of
+  // the fragment order), NCHK pieces per thread (the last may fall beyond the end: loads return 0, no write)
+  constexpr int HPT = D * TR / NT;  // elements per thread, rounded down
+  constexpr int HC = HPT >= 8 ? 8 : HPT >= 4 ? 4 : HPT >= 2 ? 2 : 1;
+  constexpr int HPIECES = D * TR / HC, NCHK = (HPIECES + NT - 1) / NT;
+  constexpr int HCW = NDW<T, HC>::value;
+  constexpr bool HSB = NDW<T, HC>::SUB;
+  int h_row[NCHK], h_k0[NCHK];
+  unsigned hs_v[NCHK], h0_v[NCHK];
+  bool h_in[NCHK];
+#pragma unroll
+  for (int j = 0; j < NCHK; ++j) {
+    const int piece = tid + j * NT;
+    h_in[j] = piece < HPIECES;
+    h_row[j] = piece / (D / HC); h_k0[j] = (piece % (D / HC)) * HC;
+    const bool ok = h_in[j] && bt * TR + h_row[j] < B;
+    hs_v[j] = ok ? ((unsigned)(bt * TR + h_row[j]) * Tn * ND + n * D + h_k0[j]) * ES : kInvalidOff;
+    h0_v[j] = ok ? ((unsigned)(bt * TR + h_row[j]) * ND + n * D + h_k0[j]) * ES : kInvalidOff;
+  }
+  struct Pre {
+    Dw<NWC> cache[UTW]; Dw<ND_> sp[UTW][S], dso[UTW][S];
+    Dw<ND_> wx[RC ? UTW : 1][RC ? GW : 1]; Dw<HCW> hrow[NCHK];  // recompute mode: Wx_t, pieces of h_(t-1)
+  };
   // operands are fetched PD steps ahead into a ring of PD + 1 register sets: a head that
-  // exchanges nothing (KW = 1) has steps shorter than a fetch from HBM takes
+  // exchanges nothing (KW = 1) has steps shorter than a fetch from HBM takes.  Recompute mode: two steps
+  // ahead, because the rebuild of the gates of step t-1 uses the operands of step t-1 during step t
 #ifdef FRNN_PD
-  constexpr int PD = KW == 1 ? FRNN_PD : 1;
+  constexpr int PD = RC ? 2 : KW == 1 ? FRNN_PD : 1;
 #else
-  constexpr int PD = KW > 1 || WAVES >= 8 ? 1 : 3;  // measured: with 8 waves and more, other waves hide the fetch
+  constexpr int PD = RC ? 2 : KW > 1 || WAVES >= 8 ? 1 : 3;  // measured: with 8 waves and more, other waves hide the fetch
 #endif
   Pre pre[PD + 1];
   auto load_pre = [&](Pre& p, int t) __attribute__((always_inline)) {
     const bool first = t == 0;
     const rsrc_t rPrev = first ? rS0 : rSt;
+    if constexpr (RC) {
+#pragma unroll
+      for (int j = 0; j < NCHK; ++j) {
+        if constexpr (HSB) p.hrow[j] = buf_load<1, true>(rPrev, first ? h0_v[j] : hs_v[j], first ? 0u : (unsigned)(t - 1) * ND * ES);
+        else p.hrow[j] = buf_load_wide<HCW>(rPrev, first ? h0_v[j] : hs_v[j], first ? 0u : (unsigned)(t - 1) * ND * ES);
+      }
+    }
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-      if constexpr (NC > 0)
+      if constexpr (RC) {
+#pragma unroll
+        for (int g = 0; g < GW; ++g) p.wx[u][g] = buf_load<ND_, SB>(rWx, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
+      }
+      if constexpr (NC > 0 && !RC)
         p.cache[u] = buf_load_wide<NWC>(rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
@@ -237,12 +326,82 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   long long tr[4] = {0, 0, 0, 0};
   const long long tr_begin = clock64();
 #endif
+  // recompute mode: the rebuilt gates of the step whose adjoint comes next
+  float gc[RC ? UTW : 1][NCA][E];
+  // h_(tau-1), this thread's piece (from the operands of step tau), to the LDS buffer of step tau
+  auto stage_h = [&](const Pre& p, int tau) __attribute__((always_inline)) {
+    T* const hb = (tau & 1) ? hb1 : hb0;
+#pragma unroll
+    for (int j = 0; j < NCHK; ++j) {
+      float v[HC];
+      unpack<HC>(p.hrow[j], v, (T*)0);
+      if (NCHK * NT == HPIECES || h_in[j]) {
+        if constexpr (HC >= 4) {
+#pragma unroll
+          for (int i = 0; i < HC; i += 4) lds_write<4>(hb, h_row[j], h_k0[j] + i, v + i);
+        } else {
+          lds_write<HC>(hb, h_row[j], h_k0[j], v);
+        }
+      }
+    }
+  };
+  // the gates of step tau from its operands and h_(tau-1) in LDS (staged before the last barrier)
+  auto rebuild_gates = [&](const Pre& p, int tau) __attribute__((always_inline)) {
+    const Frag* hf = reinterpret_cast<const Frag*>((tau & 1) ? hb1 : hb0) + lane;
+    Frag hq[KSF];
+#pragma unroll
+    for (int ks = 0; ks < KSF; ++ks) hq[ks] = hf[ks * 64];
+    f32x4 acc[UTW][GR];
+#pragma unroll
+    for (int ks = 0; ks < KSF; ++ks)
+#pragma unroll
+      for (int u = 0; u < UTW; ++u)
+#pragma unroll
+        for (int g = 0; g < GR; ++g)
+          acc[u][g] = X::mfma(rfw[u][g][ks], hq[ks], ks == 0 ? (BIAS_C ? biasc[u][g] : f32x4{0.f, 0.f, 0.f, 0.f}) : acc[u][g]);
+#pragma unroll
+    for (int u = 0; u < UTW; ++u) {
+      float ryv[GR][E], wxv[GW][E], spv[S][E];
+#pragma unroll
+      for (int g = 0; g < GR; ++g) {
+        own_elems<TR>(acc[u][g], ryv[g]);
+        if constexpr (!BIAS_C) {
+#pragma unroll
+          for (int e = 0; e < E; ++e) ryv[g][e] += bown[u][g][e];
+        }
+      }
+#pragma unroll
+      for (int g = 0; g < GW; ++g) unpack<E>(p.wx[u][g], wxv[g], (T*)0);
+#pragma unroll
+      for (int k = 0; k < S; ++k) unpack<E>(p.sp[u][k], spv[k], (T*)0);
+#pragma unroll
+      for (int e = 0; e < E; ++e) {
+        float ry[GR], wx[GW], sv[S], cc[NCA];
+#pragma unroll
+        for (int g = 0; g < GR; ++g) ry[g] = ryv[g][e];
+#pragma unroll
+        for (int g = 0; g < GW; ++g) wx[g] = wxv[g][e];
+#pragma unroll
+        for (int k = 0; k < S; ++k) sv[k] = spv[k][e];
+        CM::fwd(ry, wx, bxr[u][e], sv, cc);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) gc[u][c][e] = cc[c];
+      }
+    }
+  };
+  if constexpr (RC) {  // the gates of the first reverse step
+    stage_h(pre[0], Tn - 1);
+    __syncthreads();
+    rebuild_gates(pre[0], Tn - 1);
+  }
+
   bool dead = false, fail = false;
   // one reverse step: consumes `pc` (operands of step t), prefetches those of step t-1 into `pn`.
   // CUT (a std::bool_constant): truncated backpropagation, the step ends with the pointwise carry;
   // it is a compile-time variant of the step so that the full step carries no trace of it
   // (a run-time early exit cost 8 % at D = 128)
-  auto step = [&](auto CUT, const int t, Pre& pc, Pre& pn) __attribute__((always_inline)) {
+  // Recompute mode: `pm` holds the operands of step t-1, whose gates are rebuilt during this step.
+  auto step = [&](auto CUT, const int t, Pre& pc, Pre& pm, Pre& pn) __attribute__((always_inline)) {
     constexpr bool cut = decltype(CUT)::value;
     T* const gb = (t & 1) ? gbuf1 : gbuf0;
     FRNN_STAMP(c0);
@@ -262,7 +421,13 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
-      if constexpr (NC > 0) cache_unpack<T, NCA, E>(pc.cache[u], cv);
+      if constexpr (NC > 0 && !RC) cache_unpack<T, NCA, E>(pc.cache[u], cv);
+      if constexpr (NC > 0 && RC) {
+#pragma unroll
+        for (int c = 0; c < NC; ++c)
+#pragma unroll
+          for (int e = 0; e < E; ++e) cv[c][e] = gc[u][c][e];
+      }
 #pragma unroll
       for (int k = 0; k < S; ++k) {
         unpack<E>(pc.sp[u][k], spv[k], (T*)0); unpack<E>(sn[u][k], snv[k], (T*)0); unpack<E>(pc.dso[u][k], dsov[k], (T*)0);
@@ -303,7 +468,15 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
       }
     }
-    if constexpr (cut) return;
+    if constexpr (RC) {
+      if (t > 0) stage_h(pm, t - 1);  // uniform
+    }
+    if constexpr (cut) {
+      if constexpr (RC) {
+        if (t > 0) { lds_barrier(); rebuild_gates(pm, t - 1); }
+      }
+      return;
+    }
     FRNN_STAMP(c1);
     // the barrier also spreads a failed wait of the previous step to the whole workgroup
     if (barrier_or(fail, dead_flag)) { dead = true; return; }
@@ -496,14 +669,18 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
           for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
         }
       }
-      // receive: KW-1 partial sums of the own tiles, RC sources at a time
+      // recompute mode: the gates of step t-1, while the partial sums of step t travel
+      if constexpr (RC) {
+        if (t > 0) rebuild_gates(pm, t - 1);
+      }
+      // receive: KW-1 partial sums of the own tiles, PSRC sources at a time
       const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
 #pragma unroll
-      for (int r0 = 1; r0 < KW; r0 += RC) {
-        constexpr int NWR = RC * UTW * E;
+      for (int r0 = 1; r0 < KW; r0 += PSRC) {
+        constexpr int NWR = PSRC * UTW * E;
         int off[NWR]; bool need[NWR]; IW v[NWR];
 #pragma unroll
-        for (int rr = 0; rr < RC; ++rr) {
+        for (int rr = 0; rr < PSRC; ++rr) {
           const int src = (slice + (r0 + rr < KW ? r0 + rr : 1)) % KW;
 #pragma unroll
           for (int u = 0; u < UTW; ++u)
@@ -515,7 +692,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         }
         if (!fail) fail = poll_words_staggered<PT, NWR>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
 #pragma unroll
-        for (int rr = 0; rr < RC; ++rr)
+        for (int rr = 0; rr < PSRC; ++rr)
           if (r0 + rr < KW) {
 #pragma unroll
             for (int u = 0; u < UTW; ++u)
@@ -523,6 +700,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
               for (int e = 0; e < E; ++e) ds[u][e][0] += part_value((PT*)0, v[(rr * UTW + u) * E + e]);
           }
       }
+    }
+    if constexpr (RC && KW == 1) {
+      if (t > 0) rebuild_gates(pm, t - 1);
     }
 #ifdef FRNN_TRACE
     FRNN_STAMP(c4);
@@ -533,34 +713,51 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   // the time loop, unrolled over the ring: step t - j consumes set j and refills the set that the
   // step before it consumed
   int t = Tn - 1;
-  if (a.cut) {
+  if constexpr (RC) {
+    // ring of 3 sets: step t consumes set j (its own operands) and set j+1 (those of step t-1, for the
+    // rebuild) and refills set j+2 with the operands of step t-2
+    auto run = [&](auto CUT) __attribute__((always_inline)) {
+      for (; t >= 2 && !dead; t -= 3) {
+        step(CUT, t, pre[0], pre[1], pre[2]);
+        if (dead) break;
+        step(CUT, t - 1, pre[1], pre[2], pre[0]);
+        if (dead) break;
+        step(CUT, t - 2, pre[2], pre[0], pre[1]);
+      }
+      if (!dead && t >= 0) {
+        step(CUT, t, pre[0], pre[1], pre[2]);
+        if (!dead && t >= 1) step(CUT, t - 1, pre[1], pre[2], pre[0]);
+      }
+    };
+    if (a.cut) run(std::true_type{}); else run(std::false_type{});
+  } else if (a.cut) {
     for (; t >= PD; t -= PD + 1) {
 #pragma unroll
-      for (int j = 0; j <= PD; ++j) step(std::true_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
+      for (int j = 0; j <= PD; ++j) step(std::true_type{}, t - j, pre[j], pre[j], pre[(j + PD) % (PD + 1)]);
     }
 #pragma unroll
     for (int j = 0; j < PD; ++j)
-      if (t - j >= 0) step(std::true_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
+      if (t - j >= 0) step(std::true_type{}, t - j, pre[j], pre[j], pre[(j + PD) % (PD + 1)]);
   } else if constexpr (PD == 1) {
     // (written out: in the general form below the register allocation of the largest kernels,
     // which sit at the 256-register limit, comes out with spills)
     for (; t >= 1 && !dead; t -= 2) {
-      step(std::false_type{}, t, pre[0], pre[1]);
+      step(std::false_type{}, t, pre[0], pre[0], pre[1]);
       if (dead) break;
-      step(std::false_type{}, t - 1, pre[1], pre[0]);
+      step(std::false_type{}, t - 1, pre[1], pre[1], pre[0]);
     }
-    if (!dead && t == 0) step(std::false_type{}, 0, pre[0], pre[1]);
+    if (!dead && t == 0) step(std::false_type{}, 0, pre[0], pre[0], pre[1]);
   } else {
     for (; t >= PD && !dead; t -= PD + 1) {
 #pragma unroll
       for (int j = 0; j <= PD; ++j) {
-        step(std::false_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
+        step(std::false_type{}, t - j, pre[j], pre[j], pre[(j + PD) % (PD + 1)]);
         if (dead) break;
       }
     }
 #pragma unroll
     for (int j = 0; j < PD; ++j)
-      if (!dead && t - j >= 0) step(std::false_type{}, t - j, pre[j], pre[(j + PD) % (PD + 1)]);
+      if (!dead && t - j >= 0) step(std::false_type{}, t - j, pre[j], pre[j], pre[(j + PD) % (PD + 1)]);
   }
   if (!dead && barrier_or(fail, dead_flag)) dead = true;
 #ifdef FRNN_TRACE

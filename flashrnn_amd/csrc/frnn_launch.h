@@ -14,7 +14,8 @@ struct BwdArgs;
 template <int F, int DT> int fused_fwd_launch(const Plan& p, const FwdArgs& a, hipStream_t st);
 template <int F, int DT> int fused_bwd_launch(const Plan& p, const BwdArgs& a, hipStream_t st);
 
-// plan table lookup: function, dtype, D, variant -> plan; false if none
+// plan table lookup: function, dtype, D, variant -> plan; false if none.
+// backward: 0 forward, 1 reverse scan with gate cache, 2 reverse scan in recompute mode
 bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* out);
 
 }  // namespace frnn
@@ -26,6 +27,21 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
 #define FRNN_TU_T frnn::half_t
 #else
 #define FRNN_TU_T float
+#endif
+#if FRNN_F == 0 || FRNN_F == 1
+#if FRNN_DT != 1
+#define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_GR4_BF16
+#else
+#define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_GR4_F32
+#endif
+#elif FRNN_F == 2
+#if FRNN_DT != 1
+#define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_GR3_BF16
+#else
+#define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_GR3_F32
+#endif
+#else
+#define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_NONE
 #endif
 #if FRNN_F == 0 || FRNN_F == 1
 #if FRNN_DT != 1 && FRNN_F == 1

@@ -15,6 +15,7 @@ namespace frnn {
 struct Plan {
   int D, variant, waves, utw, kw;
   int cooperative = 0;  // host side only: launch the kernel as a cooperative one (see fused_*_tu.hip)
+  int recompute = 0;    // host side only: the reverse kernel of recompute mode
 };
 }
 
@@ -61,3 +62,14 @@ struct Plan {
   X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) X(256, 0, 4, 4, 1) \
   X(512, 0, 4, 2, 4) X(1024, 0, 4, 1, 16)
 #define FRNN_BWD_PLANS_GR1_F32 FRNN_PLANS_GR1_F32
+
+// ---- reverse scan in recompute mode (no gate cache): R and R^T are both resident, so only the head
+// dims whose two operands fit the registers beside the working set; same tilings as above where those
+// fit (gru D = 192 runs as 3 workgroups of 4 waves here: 12 waves have 168 registers each)
+#define FRNN_BWD_RC_PLANS_GR4_BF16(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+#define FRNN_BWD_RC_PLANS_GR3_BF16(X) \
+  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+#define FRNN_BWD_RC_PLANS_GR4_F32(X) X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1)
+#define FRNN_BWD_RC_PLANS_GR3_F32(X) X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1)
+#define FRNN_BWD_RC_PLANS_NONE(X)

@@ -67,6 +67,11 @@ class FlashRNNConfig:
     bias_shape: str = "GHD"
     # value of the default initial state, one number or one per state (flashrnn.py:204, :946-953)
     initial_val: Union[float, Sequence[float]] = 0.0
+    # hip_fused only, no counterpart in the reference (which always stores the activated gates of every step,
+    # fused/flashrnn.cc:97-112): the training forward writes no gate cache and the backward pass rebuilds the
+    # gates from Wx, b and R h_(t-1).  Halves what a training forward writes and the activation memory it
+    # leaves behind; ValueError where no such kernel exists (see frnn_fused_recompute_supported)
+    recompute_gates: bool = False
     # per-tensor types of the reference (flashrnn.py:190-197: biases, recurrent matrix, inputs, gates,
     # states, internal accumulation).  The kernels take every tensor in the one storage type `dtype`,
     # accumulate in fp32 and compute the gates in fp32, so each may only be None or `dtype`
@@ -134,7 +139,14 @@ def _options(cfg: "FlashRNNConfig"):
     import ctypes
 
     return ctypes.byref(_lib.Options(float(cfg.forward_clipval or 0.0), float(cfg.gradient_recurrent_clipval or 0.0),
-                                     int(bool(cfg.gradient_recurrent_cut))))
+                                     int(bool(cfg.gradient_recurrent_cut)),
+                                     int(bool(cfg.recompute_gates) and cfg.backend == "hip_fused")))
+
+
+def _workspace_bytes(cfg: "FlashRNNConfig", f_id, d_id, B, T, N, D, backward: int) -> int:
+    if cfg.backend == "hip_fused":
+        return _lib.load_library().frnn_fused_workspace_bytes_opt(f_id, d_id, B, T, N, D, backward, _options(cfg))
+    return _lib.load_library().frnn_alt_workspace_bytes(f_id, d_id, B, T, N, D, backward)
 
 
 def _raise(code: int, what: str):
@@ -258,12 +270,16 @@ class _FlashRNNFunction(torch.autograd.Function):
         s0_k = s0.detach().to(kdt).reshape(S, B, N, D).contiguous()
         with torch.cuda.device(Wx.device):
             rc = _entry(cfg.backend, "supported")(f_id, d_id, B, N, D)
+            if rc == 0 and cfg.recompute_gates:
+                if cfg.backend != "hip_fused":
+                    raise ValueError("recompute_gates is an option of the hip_fused backend")
+                rc = _lib.load_library().frnn_fused_recompute_supported(f_id, d_id, B, N, D)
             if rc != 0:
                 _raise(rc, f"{cfg.backend} backend")
             states = torch.empty((S, B, T, N, D), dtype=kdt, device=Wx.device)
             cache_bytes = _entry(cfg.backend, "cache_bytes_opt")(f_id, d_id, B, T, N, D, _options(cfg)) if training else 0
             cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx.device)
-            ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 0)
+            ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 0)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx.device)
             stream = torch.cuda.current_stream().cuda_stream
             rc = _entry(cfg.backend, "forward_opt")(
@@ -276,7 +292,8 @@ class _FlashRNNFunction(torch.autograd.Function):
                 _status.log("forward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
         ctx.cfg, ctx.training = cfg, training
         ctx.dims = (B, T, N, D)
-        ctx.save_for_backward(R_k, b_k, s0_k, states, cache)
+        # (recompute mode reads Wx again in the backward pass; it is the caller's tensor unless it was cast)
+        ctx.save_for_backward(R_k, b_k, s0_k, states, cache, Wx_k if cfg.recompute_gates else cache)
         return states
 
     @staticmethod
@@ -285,7 +302,7 @@ class _FlashRNNFunction(torch.autograd.Function):
         if not ctx.training:
             raise RuntimeError("FlashRNN backward can only be called in training mode")
         cfg = ctx.cfg
-        R_k, b_k, s0_k, states, cache = ctx.saved_tensors
+        R_k, b_k, s0_k, states, cache, Wx_k = ctx.saved_tensors
         kdt = DTYPE_DICT[cfg.dtype]
         f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
         B, T, N, D = ctx.dims
@@ -298,13 +315,19 @@ class _FlashRNNFunction(torch.autograd.Function):
             ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
             dR = torch.empty((Gr, N, D, D), dtype=torch.float32, device=dev)
             db = torch.empty((Gt, N, D), dtype=torch.float32, device=dev)
-            ws_bytes = _entry(cfg.backend, "workspace_bytes")(f_id, d_id, B, T, N, D, 1)
+            ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 1)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
             stream = torch.cuda.current_stream().cuda_stream
-            rc = _entry(cfg.backend, "backward_opt")(
-                f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
-                cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
-                ws.data_ptr(), ws.numel(), stream, _options(cfg))
+            if cfg.recompute_gates:
+                rc = _lib.load_library().frnn_fused_backward_recompute(
+                    f_id, d_id, B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(),
+                    states.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
+                    ws.data_ptr(), ws.numel(), stream, _options(cfg))
+            else:
+                rc = _entry(cfg.backend, "backward_opt")(
+                    f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
+                    cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
+                    ws.data_ptr(), ws.numel(), stream, _options(cfg))
             if rc != 0:
                 _raise(rc, f"{cfg.backend} backward")
             if cfg.backend == "hip_fused":
@@ -485,7 +508,7 @@ def _paired_heads(Wx, R, b, states, config, training):
     R2 = torch.cat([torch.cat([Rp[:, :, 0], torch.zeros_like(Rp[:, :, 0])], -1),
                     torch.cat([torch.zeros_like(Rp[:, :, 1]), Rp[:, :, 1]], -1)], -2)
     cfg2 = FlashRNNConfig(**{**{k: getattr(config, k) for k in ("function", "backend", "dtype", "forward_clipval",
-                                                                "gradient_recurrent_clipval", "gradient_recurrent_cut")},
+                                                                "gradient_recurrent_clipval", "gradient_recurrent_cut", "recompute_gates")},
                              "head_dim": 32, "num_heads": M, "batch_size": B})
     out = _FlashRNNFunction.apply(Wx.reshape(B, T, Gw, M, 32), R2, b.reshape(b.shape[0], M, 32),
                                   states.reshape(states.shape[0], B, 1, M, 32), cfg2, training)

@@ -163,6 +163,7 @@ typedef struct frnn_options {
   float forward_clipval;
   float gradient_recurrent_clipval;
   int gradient_recurrent_cut;
+  int recompute;  /* fused backend: no gate cache, see frnn_fused_backward_recompute */
 } frnn_options;
 
 /* Gate-cache size under options: an Elman cell under forward_clipval caches the unclamped h (one value per
@@ -190,6 +191,25 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
                           void* dWx, void* ds0, float* dR, float* db,
                           void* workspace, size_t workspace_bytes, void* stream,
                           const frnn_options* opt);
+
+/* ---- recompute mode of the fused backend: training without the gate cache -------------------------------
+ * The reference stores the activated gates of every step for the backward pass, unconditionally
+ * (fused/flashrnn.cc:97-112, flashrnn_fused_forward.cu:573-644): G_i values per element and step, more than
+ * the states themselves.  With opt->recompute != 0 the training forward writes the states only (cache may be
+ * null, frnn_fused_cache_bytes_opt is 0), and frnn_fused_backward_recompute, which takes Wx and b in place
+ * of the cache, rebuilds the gates of every step from Wx_t, b and R h_(t-1), with h_(t-1) read back from the
+ * stored states.  Results equal those of the cached path up to the rounding of the stored states (lstm, gru:
+ * the same bits in fp32 storage; slstm: its stabilised gates are rebuilt from the stored, rounded m).
+ * Available where R and R^T fit the registers together (frnn_fused_recompute_supported; bf16 / fp16: D = 32, 64,
+ * 96, 128, 192, 256; fp32: 32, 64), else FRNN_E_UNSUPPORTED.  For FRNN_ELMAN, which caches nothing, the flag
+ * changes nothing.  The workspace size depends on the mode: frnn_fused_workspace_bytes_opt. */
+int frnn_fused_recompute_supported(int function, int dtype, int B, int N, int D);
+size_t frnn_fused_workspace_bytes_opt(int function, int dtype, int B, int T, int N, int D, int backward,
+                                      const frnn_options* opt);
+int frnn_fused_backward_recompute(int function, int dtype, int B, int T, int N, int D,
+                                  const void* Wx, const void* R, const void* b, const void* s0, const void* states,
+                                  const void* dstates, void* dWx, void* ds0, float* dR, float* db,
+                                  void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt);
 
 /* ---- one time step with carried state (inference / decoding) --------------------------------------------
  * Replaces the reference's step kernels (_get_kernel_step, flashrnn.py:957-985, which run the whole-sequence
