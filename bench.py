@@ -62,18 +62,21 @@ def _launches_per_step(w, backend):
     return 1 + (5 if w["bwd"] else 0)
 
 
-def run_gpu(w, backend, steps, warmup, device):
+def run_gpu(w, backend, steps, warmup, device, recompute=False):
     """Returns (ms_per_step, {kernel name: (avg ms, launches per step)})."""
     import torch
-    from flashrnn_amd import flashrnn, load_library
+    from flashrnn_amd import FlashRNNConfig, flashrnn, load_library
 
     lib = load_library()
     _, dev = make_gpu_inputs(w, device)
     leaves = [dev[k].requires_grad_(w["bwd"]) for k in ("Wx", "R", "b", "states")]
     dst = dev["dstates"]
 
+    cfg = FlashRNNConfig(backend=backend, function=w["function"], dtype=w["dtype"], head_dim=w["D"], num_heads=w["N"],
+                         batch_size=w["B"], recompute_gates=bool(recompute and backend == "hip_fused"))
+
     def step():
-        out, _ = flashrnn(*leaves, function=w["function"], backend=backend, dtype=w["dtype"])
+        out, _ = flashrnn(*leaves, config=cfg)
         if w["bwd"]:
             torch.autograd.grad(out, leaves, grad_outputs=dst)
 
@@ -154,6 +157,8 @@ def main():
     ap.add_argument("--shape", default=None, help="function:dtype:B:T:N:D, e.g. lstm:bfloat16:16:1024:1:768 (fwd+bwd, "
                     "zero initial state, cotangent on every state); replaces --workload")
     ap.add_argument("--backend", default=None, choices=["hip_fused", "hip"])
+    ap.add_argument("--recompute", action="store_true",
+                    help="hip_fused in recompute mode: no gate cache, the backward pass rebuilds the gates")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-alt", action="store_true", help="skip the other-backend comparison leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -186,7 +191,7 @@ def main():
         dst.copy_(src)
         torch.cuda.synchronize()
         del src, dst
-    ms, kern = run_gpu(w, backend, args.steps, args.warmup, device)
+    ms, kern = run_gpu(w, backend, args.steps, args.warmup, device, recompute=args.recompute)
 
     # dominant kernel and its roofline: 2*N*G_r*D^2 flops per token in the forward scan and the
     # same in the reverse scan (dh = R^T dg) and in the dR GEMM
@@ -221,6 +226,7 @@ def main():
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16" if w["dtype"] == "bfloat16" else "f32", "data": "synthetic",
         "config": {"workload": f"{args.workload}: {describe(w)}", "backend": backend, "seed": w["seed"],
+                   "gate_cache": "recomputed in the backward pass" if args.recompute and backend == "hip_fused" else "stored",
                    "timed": "flashrnn() + torch.autograd.grad through the C ABI, inputs resident in HBM"},
         "roofline": roofline,
         "kernels_ms": {k: {"avg_ms": v[0], "per_step": v[1]} for k, v in kern.items()},

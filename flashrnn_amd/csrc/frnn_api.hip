@@ -61,7 +61,7 @@ static int prof_slot(int i) {  // i-th oldest entry still held -> ring slot, or 
 }
 
 // ---- plan table -------------------------------------------------------------------------------
-#define FRNN_ROW(Dv, VAR, W, U, K) {Dv, VAR, W, U, K},
+#define FRNN_ROW(Dv, VAR, W, U, K, MTR) {Dv, VAR, W, U, K, MTR},
 static const Plan kFwd4B[] = {FRNN_PLANS_GR4_BF16(FRNN_ROW)};
 static const Plan kFwd4F[] = {FRNN_PLANS_GR4_F32(FRNN_ROW)};
 static const Plan kFwdSB[] = {FRNN_PLANS_SLSTM_BF16(FRNN_ROW)};
@@ -70,6 +70,7 @@ static const Plan kFwd3F[] = {FRNN_PLANS_GR3_F32(FRNN_ROW)};
 static const Plan kFwd1B[] = {FRNN_PLANS_GR1_BF16(FRNN_ROW)};
 static const Plan kFwd1F[] = {FRNN_PLANS_GR1_F32(FRNN_ROW)};
 static const Plan kBwd4B[] = {FRNN_BWD_PLANS_GR4_BF16(FRNN_ROW)};
+static const Plan kBwdSB[] = {FRNN_BWD_PLANS_SLSTM_BF16(FRNN_ROW)};
 static const Plan kBwd4F[] = {FRNN_BWD_PLANS_GR4_F32(FRNN_ROW)};
 static const Plan kBwd3B[] = {FRNN_BWD_PLANS_GR3_BF16(FRNN_ROW)};
 static const Plan kBwd3F[] = {FRNN_BWD_PLANS_GR3_F32(FRNN_ROW)};
@@ -91,7 +92,7 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kFwd3B) else PICK(kFwd3F) }
     else { if (dtype != FRNN_F32) PICK(kFwd1B) else PICK(kFwd1F) }
   } else if (backward == 1) {
-    if (GR == 4) { if (dtype != FRNN_F32) PICK(kBwd4B) else PICK(kBwd4F) }
+    if (GR == 4) { if (dtype == FRNN_F32) PICK(kBwd4F) else if (function == FRNN_SLSTM) PICK(kBwdSB) else PICK(kBwd4B) }
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kBwd3B) else PICK(kBwd3F) }
     else { if (dtype != FRNN_F32) PICK(kBwd1B) else PICK(kBwd1F) }
   } else {  // reverse scan in recompute mode
@@ -158,13 +159,11 @@ static int groups_per_launch(int kw) { return 8 * ((device_cus() / 8) / kw); }
 // unit of its own.  Heads that run as one small workgroup (up to 4 waves, no exchange) may share a
 // compute unit three at a time: one workgroup's gate math then runs while another waits for memory
 // (measured at B = 128..256: LSTM D = 32 2.74 -> 2.17 ms, D = 64 3.72 -> 3.35; not so with 8 waves).
-static int tile_rows_for(int B, int N, int kw, int waves) {
+// `largest` is the tallest tile the tiling is compiled for (Plan::max_tr: taller ones would spill registers).
+static int tile_rows_for(int B, int N, int kw, int waves, int largest) {
   const int forced = env_int("FRNN_TILE_ROWS", 0);
-  if (forced == 4 || forced == 8 || forced == 16) return forced;
+  if (forced == 4 || forced == 8 || forced == 16) return forced < largest ? forced : largest;
   const long room = kw > 1 ? groups_per_launch(kw) : (long)device_cus() * (waves <= 4 ? 3 : 1);
-  // one workgroup of 10 or 12 waves per head: 168 registers per wave, the 16-row variants spill
-  // (LSTM D = 192 B = 1024: 3.6 ms with 16-row tiles, 3.1 with 8-row tiles in two rounds)
-  const int largest = kw == 1 && waves > 8 ? 8 : 16;
   for (int tr = 4; tr < largest; tr *= 2)
     if ((long)N * ((B + tr - 1) / tr) <= room) return tr;
   return largest;
@@ -268,7 +267,7 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   Bump bp{(unsigned char*)ws, 0};
   FusedFwdWs w;
   w.status = (int*)bp.take(256);
-  const int tr = tile_rows_for(B, N, p.kw, p.waves);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
   const size_t groups = (size_t)N * ((B + tr - 1) / tr);
   const size_t llw = (size_t)16 * D / (dtype == FRNN_F32 ? 1 : 2);
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
@@ -286,7 +285,7 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   Bump bp{(unsigned char*)ws, 0};
   FusedBwdWs w;
   w.status = (int*)bp.take(256);
-  const int tr = tile_rows_for(B, N, p.kw, p.waves);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
   const size_t bt = (B + tr - 1) / tr, groups = (size_t)N * bt;
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * bwd_inbox_words(D, p.kw) * 8 : 0);
   w.zero_bytes = bp.off;
@@ -420,7 +419,7 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
   if (waves) *waves = p.waves;
   if (tiles_per_wave) *tiles_per_wave = p.utw;
   if (wgs_per_head) *wgs_per_head = p.kw;
-  const int tr = tile_rows_for(B, N, p.kw, p.waves);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
   if (active_wgs) *active_wgs = N * ((B + tr - 1) / tr) * p.kw;
   return 0;
 }
@@ -501,7 +500,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
     const size_t one_group = 256 + (p.kw > 1 ? (size_t)3 * 16 * D / (dtype == FRNN_F32 ? 1 : 2) * 8 : 0);
     if (workspace_bytes < one_group) return fail(FRNN_E_WORKSPACE, "step scratch %zu < %zu bytes", workspace_bytes, one_group);
   }
-  const int tr = tile_rows_for(B, N, p.kw, p.waves);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
   const int groups = N * ((B + tr - 1) / tr);
   int per_launch = groups;
   if (p.kw > 1) {  // workgroups that wait for each other must all be resident
@@ -616,7 +615,7 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   prof_end(st);
   if (e) return hip_fail(e, "R transpose");
-  const int tr = tile_rows_for(B, N, p.kw, p.waves);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
   const int bt = (B + tr - 1) / tr, groups = N * bt;
   int per_launch = groups;
   if (p.kw > 1) {
@@ -633,8 +632,11 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
   // measured best, as in the forward call; the cells with several dWx stores issue them between
   // the send and the first probe, which is part of their delay
-  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", c.GR == 1 ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
-                                                                   : (p.kw >= 10 ? 8 : 4));
+  // (recompute mode sends its first probe behind the LDS reads of the rebuild: measured best without a delay,
+  // 2 units for the slstm)
+  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", o.rc ? (fx == FRNN_SLSTM ? 2 : 0)
+                                                : c.GR == 1 ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
+                                                            : (p.kw >= 10 ? 8 : 4));
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

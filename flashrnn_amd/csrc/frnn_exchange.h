@@ -162,6 +162,34 @@ __device__ __forceinline__ bool poll_words_staggered(const W* base, const int* o
         __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
   }
 }
+// The same wait in two halves: the first probe is sent by poll_issue, the caller does work that needs no
+// memory result, poll_finish examines the probe and carries on probing as above.  A probe takes ~900 cycles to
+// come back whether or not the words have arrived; work placed between the halves hides behind that trip.
+template <int NW, typename W>
+__device__ __forceinline__ void poll_issue(const W* base, const int* off, W* v) {
+#pragma unroll
+  for (int i = 0; i < NW; ++i) v[i] = ll_load(base + off[i]);
+}
+template <typename TAG, int NW, typename W>
+__device__ __forceinline__ bool poll_finish(const W* base, const int* off, const bool* need, int t, W* v, W* out,
+                                            int* status, int spin_limit) {
+  if (spin_limit < -1) return true;  // host-side test hook: every wait gives up at once
+  for (int spins = 0;; ++spins) {
+    bool ok = true;
+#pragma unroll
+    for (int i = 0; i < NW; ++i) ok = ok && (!need[i] || ll_ok((TAG*)0, v[i], t));
+    if (__all(ok)) {
+#pragma unroll
+      for (int i = 0; i < NW; ++i) out[i] = v[i];
+      return false;
+    }
+#pragma unroll
+    for (int i = 0; i < NW; ++i) v[i] = ll_load(base + off[i]);
+    if (spins > spin_limit) return true;
+    if ((spins & 63) == 63 &&
+        __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
+  }
+}
 constexpr int probe_depth(int) { return 1; }
 
 // The same wait for pairs of adjacent words, each pair fetched with one 16-byte agent-scope load

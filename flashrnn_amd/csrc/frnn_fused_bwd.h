@@ -176,6 +176,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 
   // rtf[r][u][ks]: rows p of the tiles at this wave's position in workgroup (slice + r) % KW,
   // columns = the own gate rows, local index kk = g*DL + (d - slice*DL)
+  constexpr int FRAG_REGS = (int)sizeof(Frag) / 4, RTF_REGS = KWR * UTW * KS * FRAG_REGS;
+  constexpr int PIN_REGS = RC ? 0 : RTF_REGS > 160 ? (RTF_REGS < 232 ? RTF_REGS : 232) : 0;
   Frag rtf[KWR][UTW][KS];
 #pragma unroll
   for (int r = 0; r < KW; ++r) {
@@ -187,7 +189,17 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       for (int ks = 0; ks < KS; ++ks) {
         const int kk0 = ks * X::KM + q4 * KE;
         const Frag f = load_frag_at<T>(row + (kk0 / DL) * D + (kk0 % DL));
-        if (r < KWR) rtf[r < KWR ? r : 0][u][ks] = f;
+        if (r < KWR) {
+          rtf[r < KWR ? r : 0][u][ks] = f;
+#ifndef FRNN_NO_AGPR_PIN
+          // (see the forward kernel: resident fragments beyond what the architectural VGPRs hold are pinned to
+          // the accumulation registers, where the MFMA reads them in place; in recompute mode the other operand
+          // lives there instead)
+          if constexpr (PIN_REGS > 0) {
+            if (((r * UTW + u) * KS + (KS - 1 - ks)) * FRAG_REGS + FRAG_REGS <= PIN_REGS) asm volatile("" : "+a"(rtf[r][u][ks]));
+          }
+#endif
+        }
         else rl[(((r - KWR) * UTW + u) * KS + ks) * 64] = f;
       }
     }
@@ -210,7 +222,16 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       for (int g = 0; g < GR; ++g) {
         const T* row = Rm + ((size_t)(g * N + n) * D + ub[u] + r16) * D;
 #pragma unroll
-        for (int ks = 0; ks < KSF; ++ks) rfw[u][g][ks] = load_frag<T>(row, ks, q4);
+        for (int ks = 0; ks < KSF; ++ks) {
+          rfw[u][g][ks] = load_frag<T>(row, ks, q4);
+#ifndef FRNN_NO_AGPR_PIN
+          // R and R^T together exceed the 256 architectural VGPRs of a wave; this operand, which is used off
+          // the chain of dependent steps, is the one to live in the accumulation registers, where the MFMA
+          // reads it directly.  Left to the register allocator, fragments of both operands end up there as
+          // spills, each copied back before its MFMA (measured: +400 cycles on the R^T product of a step)
+          asm volatile("" : "+a"(rfw[u][g][ks]));
+#endif
+        }
         if constexpr (BIAS_C) {
           float v[4];
           unpack4<T>(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
@@ -323,7 +344,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   __syncthreads();
 
 #ifdef FRNN_TRACE
-  long long tr[4] = {0, 0, 0, 0};
+  long long tr[5] = {0, 0, 0, 0, 0};
   const long long tr_begin = clock64();
 #endif
   // recompute mode: the rebuilt gates of the step whose adjoint comes next
@@ -345,13 +366,14 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
     }
   };
-  // the gates of step tau from its operands and h_(tau-1) in LDS (staged before the last barrier)
-  auto rebuild_gates = [&](const Pre& p, int tau) __attribute__((always_inline)) {
+  // the gates of step tau from its operands and h_(tau-1) in LDS (staged before the last barrier), in two
+  // halves: the forward product R h_(tau-1) of the own units, then the gate math
+  auto rebuild_fetch = [&](int tau, Frag (&hq)[KSF]) __attribute__((always_inline)) {
     const Frag* hf = reinterpret_cast<const Frag*>((tau & 1) ? hb1 : hb0) + lane;
-    Frag hq[KSF];
 #pragma unroll
     for (int ks = 0; ks < KSF; ++ks) hq[ks] = hf[ks * 64];
-    f32x4 acc[UTW][GR];
+  };
+  auto rebuild_product = [&](const Frag (&hq)[KSF], f32x4 (&acc)[UTW][GR]) __attribute__((always_inline)) {
 #pragma unroll
     for (int ks = 0; ks < KSF; ++ks)
 #pragma unroll
@@ -359,6 +381,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
         for (int g = 0; g < GR; ++g)
           acc[u][g] = X::mfma(rfw[u][g][ks], hq[ks], ks == 0 ? (BIAS_C ? biasc[u][g] : f32x4{0.f, 0.f, 0.f, 0.f}) : acc[u][g]);
+  };
+  auto rebuild_math = [&](const Pre& p, const f32x4 (&acc)[UTW][GR]) __attribute__((always_inline)) {
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float ryv[GR][E], wxv[GW][E], spv[S][E];
@@ -388,6 +412,21 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         for (int c = 0; c < NC; ++c) gc[u][c][e] = cc[c];
       }
     }
+    // the rebuilt gates are used in the next step only; left alone, the compiler sinks their gate math behind
+    // the wait that follows, onto the chain of dependent steps
+#pragma unroll
+    for (int u = 0; u < UTW; ++u)
+#pragma unroll
+      for (int c = 0; c < NC; ++c)
+#pragma unroll
+        for (int e = 0; e < E; ++e) asm volatile("" : "+v"(gc[u][c][e]) : : "memory");
+  };
+  auto rebuild_gates = [&](const Pre& p, int tau) __attribute__((always_inline)) {
+    f32x4 acc[UTW][GR];
+    Frag hq[KSF];
+    rebuild_fetch(tau, hq);
+    rebuild_product(hq, acc);
+    rebuild_math(p, acc);
   };
   if constexpr (RC) {  // the gates of the first reverse step
     stage_h(pre[0], Tn - 1);
@@ -669,10 +708,6 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
           for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
         }
       }
-      // recompute mode: the gates of step t-1, while the partial sums of step t travel
-      if constexpr (RC) {
-        if (t > 0) rebuild_gates(pm, t - 1);
-      }
       // receive: KW-1 partial sums of the own tiles, PSRC sources at a time
       const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
 #pragma unroll
@@ -690,7 +725,25 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
               need[(rr * UTW + u) * E + e] = bvalid && (r0 + rr < KW);
             }
         }
-        if (!fail) fail = poll_words_staggered<PT, NWR>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
+        if constexpr (RC) {
+          // recompute mode: the gates of step t-1 are rebuilt while the partial sums of step t travel.  The
+          // first probe is sent early (behind the LDS reads of the rebuild, which stand in for the delay of the
+          // cached path: a probe that reaches memory before the words costs a second round trip of ~1200
+          // cycles) and the forward product and the gate math run behind its round trip
+          static_assert(ROUNDS == 1, "recompute mode: one round of polling");
+          f32x4 racc[UTW][GR];
+          Frag rhq[KSF];
+          if (t > 0) rebuild_fetch(t - 1, rhq);
+          __builtin_amdgcn_sched_barrier(0);
+          for (int i = 0; i < a.poll_delay; ++i) __builtin_amdgcn_s_sleep(1);
+          IW pv[NWR];
+          poll_issue<NWR>(mine, off, pv);
+          __builtin_amdgcn_sched_barrier(0);
+          if (t > 0) { rebuild_product(rhq, racc); rebuild_math(pm, racc); }
+          if (!fail) fail = poll_finish<PT, NWR>(mine, off, need, t, pv, v, a.status, a.spin_limit);
+        } else {
+          if (!fail) fail = poll_words_staggered<PT, NWR>(mine, off, need, t, v, a.status, a.spin_limit, r0 == 1 ? a.poll_delay : 0);
+        }
 #pragma unroll
         for (int rr = 0; rr < PSRC; ++rr)
           if (r0 + rr < KW) {
@@ -763,7 +816,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #ifdef FRNN_TRACE
   if (lane == 0 && a.trace) {
     long long* o = a.trace + ((size_t)blockIdx.x * WAVES + w) * 8;
-    o[0] = tr[0]; o[1] = tr[1]; o[2] = tr[2]; o[3] = tr[3]; o[4] = clock64() - tr_begin;
+    o[0] = tr[0]; o[1] = tr[1]; o[2] = tr[2]; o[3] = tr[3]; o[4] = clock64() - tr_begin; o[5] = tr[4];
   }
 #endif
 

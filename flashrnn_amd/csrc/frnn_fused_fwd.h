@@ -54,8 +54,8 @@ struct FwdArgs {
 constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
   const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4, FRB = esize == 4 ? 4 : 16;
   const int KS = D / KM, per = UTW * GR * FR, regs = per * KS;
-  if (!(WAVES <= 4 && regs > 400)) return 0;
-  const int want = (regs - 352 + per - 1) / per;
+  if (!(WAVES <= 4 && regs > 336)) return 0;
+  const int want = (regs - 320 + per - 1) / per;
   const int room = (160 * 1024 - 2 * 16 * D * esize - 1024) / (WAVES * UTW * GR * 64 * FRB);
   return want < room ? want : room;
 }
@@ -136,6 +136,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   }
 
   // ---- resident operands ----------------------------------------------------------------
+  constexpr int FRAG_REGS = (int)sizeof(Frag) / 4, RF_REGS = UTW * GR * KSR * FRAG_REGS;
+  constexpr int PIN_REGS = RF_REGS > 160 ? (RF_REGS < 232 ? RF_REGS : 232) : 0;  // (160 registers, D = 320: measured no gain)
   Frag rf[UTW][GR][KSR];
   Frag* const rl = rlds + (size_t)w * RLK * UTW * GR * 64 + lane;
 #pragma unroll
@@ -146,7 +148,18 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const Frag f = load_frag<T>(row, ks, q4);
-        if (ks < KSR) rf[u][g][ks < KSR ? ks : 0] = f;
+        if (ks < KSR) {
+          rf[u][g][ks < KSR ? ks : 0] = f;
+#ifndef FRNN_NO_AGPR_PIN
+          // A resident operand of more than 128 registers does not fit the 256 architectural VGPRs beside the
+          // working set.  Left to the register allocator, some fragments are spilled to accumulation registers
+          // and copied back (4 moves) in front of every MFMA that uses them; pinned there from the start, the
+          // MFMA reads them in place.  As many as the 256 accumulation registers hold, last k-steps first.
+          if constexpr (PIN_REGS > 0) {
+            if (((u * GR + g) * KSR + (KSR - 1 - ks)) * FRAG_REGS + FRAG_REGS <= PIN_REGS) asm volatile("" : "+a"(rf[u][g][ks]));
+          }
+#endif
+        }
         else rl[(((ks - KSR) * UTW + u) * GR + g) * 64] = f;
       }
     }

@@ -46,7 +46,7 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
 #if FRNN_F == 0 || FRNN_F == 1
 #if FRNN_DT != 1 && FRNN_F == 1
 #define FRNN_TU_PLANS FRNN_PLANS_SLSTM_BF16
-#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_SLSTM_BF16
 #elif FRNN_DT != 1
 #define FRNN_TU_PLANS FRNN_PLANS_GR4_BF16
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16

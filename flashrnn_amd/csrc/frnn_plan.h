@@ -2,7 +2,11 @@
 // (gate-row count, storage type), forward and backward.  Replaces the reference's constraint
 // solver + JIT bisection (flashrnn/flashrnn/flashrnn.py:429-589, cuda_init_parametric.py:92-358).
 //
-// X(D, VARIANT, WAVES, UTW, KW):  D = 16 * UTW * WAVES * KW.
+// X(D, VARIANT, WAVES, UTW, KW, MTR):  D = 16 * UTW * WAVES * KW;  MTR = the largest batch tile (4, 8 or 16 rows)
+// this tiling is compiled for: taller tiles keep more state per lane, and where that would spill registers to
+// scratch memory the tile height stops below (a large batch then runs as more groups, in several launches if
+// the workgroups of a head wait for each other).  No compiled kernel uses scratch memory; a test checks the
+// compiler's resource report of every instantiation.
 //   R registers per lane = UTW * G_r * D / 8 (bf16) or UTW * G_r * D / 4 (f32); a workgroup of
 //   4 waves (one per SIMD) may use up to 512 VGPRs per lane, one of 8 waves 256, of 16 waves 128.
 // VARIANT 0 is the default; to try another tiling add an X(D, 1, ...) entry and run with
@@ -13,7 +17,7 @@
 
 namespace frnn {
 struct Plan {
-  int D, variant, waves, utw, kw;
+  int D, variant, waves, utw, kw, max_tr;
   int cooperative = 0;  // host side only: launch the kernel as a cooperative one (see fused_*_tu.hip)
   int recompute = 0;    // host side only: the reverse kernel of recompute mode
 };
@@ -25,51 +29,57 @@ struct Plan {
 // beat fewer, fuller workgroups (the step is a dependency chain, not a throughput problem).
 // ---- 4 recurrent gate rows per unit (lstm, slstm) --------------------------------------------
 #define FRNN_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 2, 1, 32)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 12, 1, 1, 4) \
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 #define FRNN_BWD_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 4, 1, 3) \
-  X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 2, 1, 32)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 4) X(192, 0, 4, 1, 3, 16) \
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
+// slstm backward: as above, but D = 160 as 5 workgroups of 2 waves (10 waves of 168 registers each spill at every tile height)
+#define FRNN_BWD_PLANS_SLSTM_BF16(X) \
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) \
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 // slstm: its heavier gate math tips D = 192 forward to 3 workgroups of 4 waves (1.19 against 1.26 ms)
 #define FRNN_PLANS_SLSTM_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 4, 1, 3) \
-  X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 2, 1, 32)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 4, 1, 3, 16) \
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 #define FRNN_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 4, 1, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 16) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_BWD_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 4, 1, 4) X(320, 0, 4, 1, 5) X(384, 0, 4, 1, 6) X(448, 0, 4, 1, 7) X(512, 0, 4, 1, 8) X(640, 0, 4, 1, 10) X(768, 0, 4, 1, 12) X(1024, 0, 4, 1, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 12, 1, 1, 4) \
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
 #define FRNN_BWD_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 16, 1, 1) X(320, 0, 4, 1, 5) X(384, 0, 8, 3, 1) X(448, 0, 4, 1, 7) X(512, 0, 4, 2, 4) X(640, 0, 4, 1, 10) \
-  X(768, 0, 8, 1, 6) X(1024, 0, 8, 1, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
+  X(256, 0, 16, 1, 1, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 8, 3, 1, 4) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 2, 4, 16) X(640, 0, 4, 1, 10, 16) \
+  X(768, 0, 8, 1, 6, 16) X(1024, 0, 8, 1, 8, 8)
 #define FRNN_BWD_PLANS_GR1_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 8, 1, 1) X(160, 0, 10, 1, 1) X(192, 0, 12, 1, 1) \
-  X(256, 0, 16, 1, 1) X(320, 0, 4, 1, 5) X(384, 0, 8, 1, 3) X(448, 0, 4, 1, 7) X(512, 0, 16, 1, 2) X(640, 0, 4, 1, 10) \
-  X(768, 0, 8, 1, 6) X(1024, 0, 8, 1, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
+  X(256, 0, 16, 1, 1, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 8, 1, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 8, 1, 4, 16) X(640, 0, 4, 1, 10, 16) \
+  X(768, 0, 8, 1, 6, 16) X(1024, 0, 8, 1, 8, 4)
 #define FRNN_PLANS_GR1_F32(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 2, 1) X(192, 0, 4, 3, 1) X(256, 0, 4, 4, 1) \
-  X(512, 0, 4, 2, 4) X(1024, 0, 4, 1, 16)
-#define FRNN_BWD_PLANS_GR1_F32 FRNN_PLANS_GR1_F32
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 16) \
+  X(512, 0, 4, 2, 4, 16)
+#define FRNN_BWD_PLANS_GR1_F32(X) \
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 8) \
+  X(512, 0, 4, 2, 4, 8)
 
 // ---- reverse scan in recompute mode (no gate cache): R and R^T are both resident, so only the head
 // dims whose two operands fit the registers beside the working set; same tilings as above where those
 // fit (gru D = 192 runs as 3 workgroups of 4 waves here: 12 waves have 168 registers each)
 #define FRNN_BWD_RC_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8)
 #define FRNN_BWD_RC_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1) X(96, 0, 6, 1, 1) X(128, 0, 4, 1, 2) X(192, 0, 4, 1, 3) X(256, 0, 4, 1, 4)
-#define FRNN_BWD_RC_PLANS_GR4_F32(X) X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1)
-#define FRNN_BWD_RC_PLANS_GR3_F32(X) X(32, 0, 2, 1, 1) X(64, 0, 4, 1, 1)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
+#define FRNN_BWD_RC_PLANS_GR4_F32(X) X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16)
+#define FRNN_BWD_RC_PLANS_GR3_F32(X) X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16)
 #define FRNN_BWD_RC_PLANS_NONE(X)

@@ -5,16 +5,24 @@
 
 namespace frnn {
 
+// the kernel for a tile height, or null if the tiling is not compiled that tall (a template, so that the
+// taller kernels of such a tiling are never instantiated)
+template <int Dv, int W, int U, int K, int MTR, bool RCV> static void (*bwd_kernel_for(int tile_rows))(const BwdArgs) {
+  if (tile_rows == 4) return fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4, RCV>;
+  if constexpr (MTR >= 8) { if (tile_rows == 8) return fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 8, RCV>; }
+  if constexpr (MTR >= 16) { if (tile_rows == 16) return fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 16, RCV>; }
+  return nullptr;
+}
+
 template <>
 int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
   const bool rc = p.recompute != 0;
   const size_t lds = bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T), rc) + 16;
-#define FRNN_CASE_(RCV, Dv, VAR, W, U, K)                                                               \
+#define FRNN_CASE_(RCV, Dv, VAR, W, U, K, MTR)                                                          \
   if (rc == RCV && p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                               \
-    auto kern = a.tile_rows == 4 ? fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4, RCV>              \
-              : a.tile_rows == 8 ? fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 8, RCV>              \
-                                 : fused_bwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 16, RCV>;            \
+    auto kern = bwd_kernel_for<Dv, W, U, K, MTR, RCV>(a.tile_rows);                                      \
+    if (!kern) return FRNN_E_UNSUPPORTED;                                                                \
     if (lds > 65536) {                                                                                   \
       hipError_t e = hipFuncSetAttribute((const void*)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds); \
       if (e != hipSuccess) return (int)e;                                                                \
@@ -27,8 +35,8 @@ int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream
     hipLaunchKernelGGL(kern, grid, dim3(W * 64), lds, st, a);                                            \
     return (int)hipGetLastError();                                                                       \
   }
-#define FRNN_CASE(Dv, VAR, W, U, K) FRNN_CASE_(false, Dv, VAR, W, U, K)
-#define FRNN_CASE_RC(Dv, VAR, W, U, K) FRNN_CASE_(true, Dv, VAR, W, U, K)
+#define FRNN_CASE(Dv, VAR, W, U, K, MTR) FRNN_CASE_(false, Dv, VAR, W, U, K, MTR)
+#define FRNN_CASE_RC(Dv, VAR, W, U, K, MTR) FRNN_CASE_(true, Dv, VAR, W, U, K, MTR)
   FRNN_TU_BWD_PLANS(FRNN_CASE)
   FRNN_TU_BWD_RC_PLANS(FRNN_CASE_RC)
 #undef FRNN_CASE

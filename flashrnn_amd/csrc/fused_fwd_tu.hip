@@ -8,14 +8,22 @@
 
 namespace frnn {
 
+// the kernel for a tile height, or null if the tiling is not compiled that tall (a template, so that the
+// taller kernels of such a tiling are never instantiated)
+template <int Dv, int W, int U, int K, int MTR> static void (*fwd_kernel_for(int tile_rows))(const FwdArgs) {
+  if (tile_rows == 4) return fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4>;
+  if constexpr (MTR >= 8) { if (tile_rows == 8) return fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 8>; }
+  if constexpr (MTR >= 16) { if (tile_rows == 16) return fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 16>; }
+  return nullptr;
+}
+
 template <>
 int fused_fwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const FwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
-#define FRNN_CASE(Dv, VAR, W, U, K)                                                          \
+#define FRNN_CASE(Dv, VAR, W, U, K, MTR)                                                     \
   if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                 \
-    auto kern = a.tile_rows == 4 ? fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 4>                       \
-              : a.tile_rows == 8 ? fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 8>                       \
-                                 : fused_fwd_kernel<FRNN_F, FRNN_TU_T, Dv, W, U, K, 16>;                     \
+    auto kern = fwd_kernel_for<Dv, W, U, K, MTR>(a.tile_rows);                                \
+    if (!kern) return FRNN_E_UNSUPPORTED;                                                     \
     if (K > 1 && p.cooperative) {                                                             \
       FwdArgs aa = a;                                                                         \
       void* args[] = {(void*)&aa};                                                            \
