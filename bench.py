@@ -29,13 +29,45 @@ WORKLOADS = {
 }
 GATES_R = {"lstm": 4, "slstm": 4, "gru": 3, "elman": 1}
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, published
-# HBM bytes per launch (FETCH_SIZE + WRITE_SIZE, KiB -> bytes, copy-kernel factor 1.00) measured with
-# two `rocprofv3 --pmc` runs of this script; summary and commands in
-# profiles/fused_kernels_lstm_bf16_B8_T1024_N3_D256_hbm_traffic.txt.  Workloads not profiled: null.
-TRAFFIC_BYTES = {
-    ("C2", "fused_fwd_kernel"): (38977.1 + 98304.0) * 1024,
-    ("C2", "fused_bwd_kernel"): (81939.2 + 122928.0) * 1024,
-}
+# roofline.traffic comes from the committed counter profile of the same command, never from a constant in this file:
+# the profile holds one "traffic:" line per kernel template it measured (FETCH_SIZE and WRITE_SIZE in KiB per
+# dispatch and the factors a plain 256 MiB copy gave in the same run).  If the kernel that ran here is not the
+# template that was profiled (another tiling, tile height or mode), traffic is null and the reason is given.
+TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "fused_kernels_lstm_bf16_B8_T1024_N3_D256_hbm_traffic.txt")
+CELL_NAMES = {"lstm": "LSTM", "slstm": "sLSTM", "gru": "GRU", "elman": "Elman"}
+
+
+def kernel_template(w, kernel, recompute):
+    """Name of the fused kernel instantiation this workload runs, as the profiles spell it."""
+    from flashrnn_amd import fused_plan
+
+    backward = kernel == "fused_bwd_kernel"
+    waves, utw, kw, active = fused_plan(w["function"], w["dtype"], w["B"], w["N"], w["D"], backward)
+    tiles = active // kw // w["N"]
+    tr = next(t for t in (4, 8, 16) if (w["B"] + t - 1) // t == tiles)
+    rc = ",RECOMPUTE" if (recompute and backward and w["function"] != "elman") else ""
+    dt = {"bfloat16": "bf16", "float32": "f32", "float16": "f16"}[w["dtype"]]
+    return f"{kernel}<{CELL_NAMES[w['function']]},{dt},D={w['D']},WAVES={waves},UTW={utw},KW={kw},TILE_ROWS={tr}{rc}>"
+
+
+def profiled_traffic(w, kernel, recompute):
+    """(bytes per launch or None, note)."""
+    try:
+        name = kernel_template(w, kernel, recompute)
+    except Exception as e:  # no fused plan (alternating backend)
+        return None, f"no fused kernel template for this run ({e})"
+    mode = "recomputed" if recompute else "stored"
+    try:
+        lines = [l for l in open(TRAFFIC_PROFILE) if l.startswith("traffic:")]
+    except OSError:
+        return None, f"{os.path.relpath(TRAFFIC_PROFILE, ROOT)} is missing"
+    for l in lines:
+        f = dict(x.split("=", 1) for x in l.split()[1:])
+        if f["kernel"] == name and f["mode"] == mode:
+            b = float(f["fetch_kib"]) * 1024 / float(f["fetch_factor"]) + float(f["write_kib"]) * 1024 / float(f["write_factor"])
+            return b, (f"{os.path.relpath(TRAFFIC_PROFILE, ROOT)}: FETCH_SIZE {f['fetch_kib']} KiB / {f['fetch_factor']} + "
+                       f"WRITE_SIZE {f['write_kib']} KiB / {f['write_factor']} (factors of a plain 256 MiB copy in the same run)")
+    return None, f"the committed profile has no entry for {name} (gate cache {mode}): not measured"
 
 
 def describe(w):
@@ -148,12 +180,93 @@ def run_cpu_baseline(w, budget_s=20.0):
                 ms=med * 1e3)
 
 
+def run_sweep(device, steps, warmup):
+    """The fused-path head-dim sweep of the fifth configuration (LSTM bf16 B16 T1024, N*D = 768; D = 512 has N = 1)
+    on both backends, and the fifth configuration itself (Elman D = 1024 B32) on both."""
+    rows = []
+    for N, D in ((24, 32), (12, 64), (6, 128), (3, 256), (1, 512)):
+        w = dict(function="lstm", dtype="bfloat16", B=16, T=1024, N=N, D=D, init="zeros", grad_on="all", bwd=True, seed=1006)
+        r = {"workload": describe(w)}
+        for backend in ("hip_fused", "hip"):
+            ms, _ = run_gpu(w, backend, steps if backend == "hip_fused" else max(3, steps // 4), warmup, device)
+            r[backend + "_ms"] = ms
+        r["tokens_per_s_hip_fused"] = 16 * 1024 / (r["hip_fused_ms"] * 1e-3)
+        r["speedup_of_hip_fused"] = r["hip_ms"] / r["hip_fused_ms"]
+        rows.append(r)
+    w5 = WORKLOADS["C5"]
+    r = {"workload": describe(w5)}
+    for backend in ("hip", "hip_fused"):
+        ms, _ = run_gpu(w5, backend, max(3, steps // 2), warmup, device)
+        r[backend + "_ms"] = ms
+    r["note"] = "the configuration names the alternating backend (hip); the fused kernels also cover this head dim and are faster"
+    rows.append(r)
+    return rows
+
+
+def run_steps(device, n_steps=256):
+    """Single-step decoding (flashrnn_step with the fp32 carry): microseconds per step, eager and replayed from a
+    HIP graph of 64 chained steps (the device-side cost of a dependent step), and the step kernel between two HIP
+    events (which resolve ~6 us at best)."""
+    import torch
+    from flashrnn_amd import flashrnn_step, load_library, make_carry
+    from oracle import make_inputs
+
+    lib = load_library()
+    out = []
+    for function, N, D in (("lstm", 3, 256), ("lstm", 4, 192), ("lstm", 12, 64), ("gru", 4, 128), ("slstm", 4, 192)):
+        for B in (1, 8):
+            for backend in ("hip_fused", "hip"):
+                inp = make_inputs(function, B, 1, N, D, 7, init="randn", round_to=torch.bfloat16)
+                x = {k: v.to(device, torch.bfloat16).contiguous() for k, v in inp.items()}
+                carry = make_carry(x["states"])
+                kw = dict(function=function, backend=backend, dtype="bfloat16", carry=carry)
+                s = x["states"]
+                for _ in range(20):
+                    s = flashrnn_step(x["Wx"], x["R"], x["b"], s, **kw)
+                torch.cuda.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n_steps):
+                    s = flashrnn_step(x["Wx"], x["R"], x["b"], s, **kw)
+                torch.cuda.synchronize()
+                eager = (time.perf_counter() - t0) / n_steps * 1e6
+                lib.frnn_profile_enable(1)
+                for _ in range(32):
+                    s = flashrnn_step(x["Wx"], x["R"], x["b"], s, **kw)
+                torch.cuda.synchronize()
+                ks = [lib.frnn_profile_ms(i) * 1e3 for i in range(lib.frnn_profile_count())]
+                lib.frnn_profile_enable(0)
+                # one graph of 64 chained steps (each reads the states the one before wrote): its replay time / 64 is
+                # the device-side cost of a dependent step, free of host time and of the event resolution
+                CH = 64
+                s_in = x["states"].clone()
+                g = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(g):
+                    s_c = s_in
+                    for _ in range(CH):
+                        s_c = flashrnn_step(x["Wx"], x["R"], x["b"], s_c, **kw)
+                    s_in.copy_(s_c)
+                for _ in range(5):
+                    g.replay()
+                torch.cuda.synchronize()
+                reps = max(1, n_steps // CH)
+                t0 = time.perf_counter()
+                for _ in range(reps):
+                    g.replay()
+                torch.cuda.synchronize()
+                graph = (time.perf_counter() - t0) / (reps * CH) * 1e6
+                out.append({"cell": f"{function} bf16 B{B} N{N} D{D}", "backend": backend, "eager_us_per_step": eager,
+                            "graph_replay_us_per_step": graph, "kernel_event_us": sorted(ks)[len(ks) // 2]})
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=20)
     ap.add_argument("--warmup", type=int, default=5)
-    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS))
+    ap.add_argument("--workload", default="C2", choices=sorted(WORKLOADS) + ["C5s", "step"],
+                    help="C1..C5: the benchmark configurations; C5s: the head-dim sweep of the fifth one on both backends; "
+                         "step: single-step decoding latency")
     ap.add_argument("--shape", default=None, help="function:dtype:B:T:N:D, e.g. lstm:bfloat16:16:1024:1:768 (fwd+bwd, "
                     "zero initial state, cotangent on every state); replaces --workload")
     ap.add_argument("--backend", default=None, choices=["hip_fused", "hip"])
@@ -181,6 +294,24 @@ def main():
         args.workload = "shape " + args.shape
         WORKLOADS[args.workload] = dict(function=f, dtype=dt, B=int(B), T=int(T), N=int(N), D=int(D), init="zeros",
                                         grad_on="all", bwd=True, seed=2000)
+    if args.workload == "C5s":
+        rows = run_sweep(device, args.steps, args.warmup)
+        ref = rows[3]
+        print(json.dumps({"metric": "tokens/s fwd+bwd, LSTM bf16 B16 T1024 head-dim sweep at N*D = 768 (fused vs alternating)",
+                          "value": ref["tokens_per_s_hip_fused"], "unit": "tokens/s", "n_gpus": 1, "steps": args.steps,
+                          "warmup": args.warmup, "ms_per_step": ref["hip_fused_ms"], "higher_is_better": True, "scaling": "weak",
+                          "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": "C5s: value and ms_per_step are the D = 256 point on hip_fused"}, "sweep": rows}))
+        return
+    if args.workload == "step":
+        rows = run_steps(device)
+        ref = rows[0]
+        print(json.dumps({"metric": "microseconds per single decoding step (flashrnn_step, fp32 carry)", "value": ref["graph_replay_us_per_step"],
+                          "unit": "us/step", "n_gpus": 1, "steps": 256, "warmup": 20, "ms_per_step": ref["graph_replay_us_per_step"] / 1e3,
+                          "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
+                          "config": {"workload": "step: value is " + ref["cell"] + " on " + ref["backend"] + ", graph replay"},
+                          "steps_table": rows}))
+        return
     w = WORKLOADS[args.workload]
     backend = args.backend or ("hip" if args.workload == "C5" else "hip_fused")
     tokens = w["B"] * w["T"]
@@ -203,8 +334,9 @@ def main():
     dom_ms = cand[dom][0]
     peak = PEAK_TFLOPS[w["dtype"]]
     achieved = algo[dom] / cand[dom][1] / (dom_ms * 1e-3) / 1e12
+    traffic, traffic_note = profiled_traffic(w, dom, args.recompute)
     roofline = dict(kernel=dom, bound="mfma", achieved=achieved, peak=peak, unit="TFLOP/s", frac=achieved / peak,
-                    traffic=TRAFFIC_BYTES.get((args.workload, dom)), avg_launch_ms=dom_ms, launches_per_step=cand[dom][1],
+                    traffic=traffic, traffic_source=traffic_note, avg_launch_ms=dom_ms, launches_per_step=cand[dom][1],
                     us_per_time_step=dom_ms * 1e3 / w["T"])
     # the whole step against the same peak: 3 contractions of flops_scan each when there is a backward pass
     step_flops = flops_scan * (3.0 if w["bwd"] else 1.0)
