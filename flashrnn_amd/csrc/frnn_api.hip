@@ -77,6 +77,7 @@ static const Plan kBwd3F[] = {FRNN_BWD_PLANS_GR3_F32(FRNN_ROW)};
 static const Plan kBwd1B[] = {FRNN_BWD_PLANS_GR1_BF16(FRNN_ROW)};
 static const Plan kBwd1F[] = {FRNN_BWD_PLANS_GR1_F32(FRNN_ROW)};
 static const Plan kRc4B[] = {FRNN_BWD_RC_PLANS_GR4_BF16(FRNN_ROW)};
+static const Plan kRcSB[] = {FRNN_BWD_RC_PLANS_SLSTM_BF16(FRNN_ROW)};
 static const Plan kRc4F[] = {FRNN_BWD_RC_PLANS_GR4_F32(FRNN_ROW)};
 static const Plan kRc3B[] = {FRNN_BWD_RC_PLANS_GR3_BF16(FRNN_ROW)};
 static const Plan kRc3F[] = {FRNN_BWD_RC_PLANS_GR3_F32(FRNN_ROW)};
@@ -96,7 +97,7 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kBwd3B) else PICK(kBwd3F) }
     else { if (dtype != FRNN_F32) PICK(kBwd1B) else PICK(kBwd1F) }
   } else {  // reverse scan in recompute mode
-    if (GR == 4) { if (dtype != FRNN_F32) PICK(kRc4B) else PICK(kRc4F) }
+    if (GR == 4) { if (dtype == FRNN_F32) PICK(kRc4F) else if (function == FRNN_SLSTM) PICK(kRcSB) else PICK(kRc4B) }
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kRc3B) else PICK(kRc3F) }
     else return false;
   }
@@ -115,22 +116,26 @@ static int env_int(const char* name, int dflt) {
   const char* v = getenv(name);
   return (v && *v) ? atoi(v) : dflt;
 }
+// Exchange stores of a group whose workgroups share an XCD stay in that XCD's L2 (workgroup scope; the kernels
+// check the placement themselves, see xcd_handshake).  FRNN_AGENT_STORES=1 keeps every store at agent scope.
+static bool near_stores_allowed() { return env_int("FRNN_AGENT_STORES", 0) == 0; }
 
 // s_sleep units before the first probe of a forward step.  A probe that reaches memory before the
 // data costs a whole extra round trip and adds traffic, one that comes late costs its lateness; where
 // the data arrives depends on how long the other workgroups' gate math and stores take, so the best
-// value differs by cell and tiling.  Measured on MI355X (bf16, T = 1024; a unit off costs 1-3 %):
-//   lstm  D=256 (4 workgroups) 3, D=384 (6) 6, D=512 (8) 3;  gru D=256 5;  slstm D=192 (3) 2;
-//   lstm D=320 (5) 3, D=448 (7) 3, D=640 (10) 5, D=768 (12) 6;  gru D=1024 (16 workgroups) 8;
-//   elman D=512 (4 workgroups, 2 tiles per wave) 6, D=1024 (8 workgroups of 8 waves) 12.
+// value differs by cell and tiling.  Measured on MI355X (bf16, T = 1024, exchange stores kept in the XCD's
+// L2; a unit off costs up to 1-3 %, most curves are flat within 2 units):
+//   lstm  D=256 (4 workgroups) 3, D=384 (6) 4, D=512 (8) 0-4, D=768 (12) 6, D=1024 (32 workgroups of 2 waves) 3-6;
+//   gru D=256 4, D=1024 (16) 6;  slstm D=192 (3) 2;
+//   elman D=512 (4 workgroups, 2 tiles per wave) 6, D=1024 (8 workgroups of 8 waves) 2.
 static int fwd_poll_delay_default(int function, const Plan& p) {
   if (p.kw <= 1) return 0;
-  if (function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP) return p.waves > 4 ? 12 : 6;
+  if (function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP) return p.waves > 4 ? 2 : 6;
   if (p.kw == 3) return 2;
-  if (p.kw == 6 || p.kw == 12) return 6;
+  if (p.kw == 6) return 4;
   if (p.kw == 10) return 5;
-  if (p.kw >= 16) return 8;  // (lstm D=1024, 32 workgroups of 2 waves: 8 as well)
-  if (p.kw == 4 && function == FRNN_GRU) return 5;
+  if (p.kw >= 12) return 6;
+  if (p.kw == 4 && function == FRNN_GRU) return 4;
   return 3;
 }
 
@@ -262,7 +267,7 @@ static int check_ptr(const void* p, const char* name) {
 #define CHECK_PTR(p) { int e_ = check_ptr(p, #p); if (e_) return e_; }
 
 // ---- fused workspace layouts --------------------------------------------------------------------
-struct FusedFwdWs { int* status; u64* ll; size_t zero_bytes; size_t total; };
+struct FusedFwdWs { int* status; u64* ll; int* xcd; size_t zero_bytes; size_t total; };
 static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, const Plan& p) {
   Bump bp{(unsigned char*)ws, 0};
   FusedFwdWs w;
@@ -271,14 +276,15 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   const size_t groups = (size_t)N * ((B + tr - 1) / tr);
   const size_t llw = (size_t)16 * D / (dtype == FRNN_F32 ? 1 : 2);
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
-  w.zero_bytes = bp.off;  // status + exchange slots must start at zero for every call
+  w.xcd = (int*)bp.take(p.kw > 1 ? groups * 32 * 4 : 0);  // words of xcd_handshake
+  w.zero_bytes = bp.off;  // status, exchange slots and handshake words must start at zero for every call
 #ifdef FRNN_TRACE
   bp.take(1 << 20);
 #endif
   w.total = bp.off;
   return w;
 }
-struct FusedBwdWs { int* status; u64* ll; size_t zero_bytes; void* Rt; void* dgx; float* dbp; float* part; int splits; size_t total; };
+struct FusedBwdWs { int* status; u64* ll; int* xcd; size_t zero_bytes; void* Rt; void* dgx; float* dbp; float* part; int splits; size_t total; };
 static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int T, int N, int D, const Plan& p) {
   const CellDims c = cell_dims(function);
   const size_t es = dtype_size(dtype);
@@ -288,6 +294,7 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
   const size_t bt = (B + tr - 1) / tr, groups = (size_t)N * bt;
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * bwd_inbox_words(D, p.kw) * 8 : 0);
+  w.xcd = (int*)bp.take(p.kw > 1 ? groups * 32 * 4 : 0);  // words of xcd_handshake
   w.zero_bytes = bp.off;
 #ifdef FRNN_TRACE
   bp.take(1 << 20);
@@ -497,7 +504,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
     prof_end(st);
     if (e) return hip_fail(e, "workspace clear");
   } else {
-    const size_t one_group = 256 + (p.kw > 1 ? (size_t)3 * 16 * D / (dtype == FRNN_F32 ? 1 : 2) * 8 : 0);
+    const size_t one_group = 256 + (p.kw > 1 ? (size_t)3 * 16 * D / (dtype == FRNN_F32 ? 1 : 2) * 8 + 256 : 0);
     if (workspace_bytes < one_group) return fail(FRNN_E_WORKSPACE, "step scratch %zu < %zu bytes", workspace_bytes, one_group);
   }
   const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
@@ -510,6 +517,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   FwdArgs a;
   a.Wx = Wx; a.R = R; a.b = b; a.s0 = s0; a.states = states; a.cache = cache;
   a.ll = w.ll; a.status = w.status;
+  a.xcd = (p.kw > 1 && !step && near_stores_allowed()) ? w.xcd : nullptr;
   a.carry = carry; a.step = step;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
@@ -627,16 +635,16 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   a.Wx = Wx; a.R = R; a.b = b;
   a.dWx = dWx; a.dgx = w.dgx; a.ds0 = ds0; a.dbp = w.dbp;
   a.ll = w.ll; a.status = w.status;
+  a.xcd = (p.kw > 1 && near_stores_allowed()) ? w.xcd : nullptr;
   a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
-  // measured best, as in the forward call; the cells with several dWx stores issue them between
-  // the send and the first probe, which is part of their delay
-  // (recompute mode sends its first probe behind the LDS reads of the rebuild: measured best without a delay,
-  // 2 units for the slstm)
+  // measured best, as in the forward call (exchange stores kept in the XCD's L2): the gated cells 0-2 units at every
+  // head dim from 192 to 1024 (their dWx stores are issued between the send and the first probe, which is part of
+  // their delay), elman D = 512 4, D = 1024 8; recompute mode sends its first probe behind the LDS reads of the
+  // rebuild: best without a delay, 2 units for the slstm
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", o.rc ? (fx == FRNN_SLSTM ? 2 : 0)
-                                                : c.GR == 1 ? (p.kw > 4 ? (p.waves > 4 ? 12 : 8) : 6)
-                                                            : (p.kw >= 10 ? 8 : 4));
+                                                : c.GR == 1 ? (p.kw > 4 ? 8 : 4) : 2);
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE

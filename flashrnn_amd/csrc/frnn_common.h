@@ -321,19 +321,48 @@ __device__ __forceinline__ float part_value(Part32*, unsigned w) { return __uint
 __device__ __forceinline__ unsigned ll_load(const unsigned* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void ll_store(unsigned* p, unsigned v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
-
-__device__ __forceinline__ void ll_store32(unsigned* p, unsigned v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
 __device__ __forceinline__ u64 ll_load(const u64* p) {
   return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
-__device__ __forceinline__ void ll_store(u64* p, u64 v) {
-  __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-}
+// Stores of tagged words, N per lane at `base + voff + i * STRIDE` bytes (base uniform, voff per lane).
+// near == 0: agent scope (sc1), the store is written through to memory, where an agent-scope load of any
+// compute unit finds it.  near == ~0: workgroup scope (sc0), the store is written through the compute unit's L1
+// into the L2 of its XCD and stays there; the agent-scope loads of the other workgroups miss their L1 and meet
+// it in that L2, provided they run on the same XCD (each XCD has an L2 of its own; a store left in another
+// XCD's L2 is never seen).  Measured for an all-to-all exchange of one word per thread between 4 workgroups of
+// one XCD: 1080 cycles per step against 1610-1980 with agent-scope stores (2 workgroups 840 against 1570,
+// 8: 1420 against 2240).  The kernels pass near == ~0 only after xcd_handshake has shown that the workgroups of
+// the group share an XCD.  `near` is a lane mask, all ones or zero: both forms of the store are issued, one of
+// them with no lane enabled, inside one asm block.  A branch that the compiler sees splits the step's schedule and
+// costs the kernels at the register limit spills; a scalar branch inside the block costs 35-60 cycles per store
+// group (measured), which adds up where a wave sends to 31 other workgroups per step.
+#define FRNN_SEL_HEAD "s_mov_b64 %[tmp], exec\n\ts_and_b64 exec, %[tmp], %[nr]\n\t"
+#define FRNN_SEL_MID "s_andn2_b64 exec, %[tmp], %[nr]\n\t"
+#define FRNN_SEL_TAIL "s_mov_b64 exec, %[tmp]"
+#define FRNN_ST0(op, sc) op " %[o], %[v0], %[b] " sc "\n\t"
+#define FRNN_ST1(op, sc) op " %[o], %[v1], %[b] offset:%[k1] " sc "\n\t"
+#define FRNN_ST2(op, sc) op " %[o], %[v2], %[b] offset:%[k2] " sc "\n\t"
+#define FRNN_ST3(op, sc) op " %[o], %[v3], %[b] offset:%[k3] " sc "\n\t"
+#define FRNN_SEL_DEFINE(W, op)                                                                                   \
+  template <int N, int STRIDE> __device__ __forceinline__ void ll_store_sel(const void* base, unsigned voff, const W* v, u64 near) { \
+    static_assert(N == 1 || N == 2 || N == 4, "1, 2 or 4 words per lane");                                       \
+    static_assert(3 * STRIDE < 4096, "immediate offsets");                                                      \
+    u64 tmp;                                                                                                     \
+    if constexpr (N == 1)                                                                                        \
+      asm volatile(FRNN_SEL_HEAD FRNN_ST0(op, "sc0") FRNN_SEL_MID FRNN_ST0(op, "sc1") FRNN_SEL_TAIL                \
+                   : [tmp] "=&s"(tmp) : [o] "v"(voff), [b] "s"(base), [v0] "v"(v[0]), [nr] "s"(near) : "scc");    \
+    else if constexpr (N == 2)                                                                                   \
+      asm volatile(FRNN_SEL_HEAD FRNN_ST0(op, "sc0") FRNN_ST1(op, "sc0") FRNN_SEL_MID FRNN_ST0(op, "sc1") FRNN_ST1(op, "sc1") FRNN_SEL_TAIL \
+                   : [tmp] "=&s"(tmp) : [o] "v"(voff), [b] "s"(base), [v0] "v"(v[0]), [v1] "v"(v[1]), [k1] "n"(STRIDE), [nr] "s"(near) : "scc"); \
+    else                                                                                                         \
+      asm volatile(FRNN_SEL_HEAD FRNN_ST0(op, "sc0") FRNN_ST1(op, "sc0") FRNN_ST2(op, "sc0") FRNN_ST3(op, "sc0") FRNN_SEL_MID \
+                   FRNN_ST0(op, "sc1") FRNN_ST1(op, "sc1") FRNN_ST2(op, "sc1") FRNN_ST3(op, "sc1") FRNN_SEL_TAIL    \
+                   : [tmp] "=&s"(tmp) : [o] "v"(voff), [b] "s"(base), [v0] "v"(v[0]), [v1] "v"(v[1]), [v2] "v"(v[2]), [v3] "v"(v[3]), \
+                      [k1] "n"(STRIDE), [k2] "n"(2 * STRIDE), [k3] "n"(3 * STRIDE), [nr] "s"(near) : "scc");     \
+  }
+FRNN_SEL_DEFINE(unsigned, "global_store_dword")
+FRNN_SEL_DEFINE(u64, "global_store_dwordx2")
+#undef FRNN_SEL_DEFINE
 
 // largest divisor of n that is <= 8: k-steps whose LDS fragments are fetched together
 constexpr int chunk_of(int n) { for (int c = 8; c > 1; --c) if (n % c == 0) return c; return 1; }

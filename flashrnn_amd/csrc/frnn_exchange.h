@@ -64,21 +64,51 @@ template <int E> __device__ __forceinline__ void lds_write(float* buf, int row, 
   for (int i = 0; i < E; ++i) buf[ST<float>::frag_elem(row, k0 + i)] = v[i];
 }
 
-// tagged global stores of E consecutive elements (row, k0..) for step t
-template <int E, typename T> __device__ __forceinline__ void ll_write16(u64* slot, int row, int k0, const float* v, int t) {
+// tagged global stores of E consecutive elements (row, k0..) for step t into the slot that starts `slot_off`
+// bytes behind `base` (base uniform; near: see ll_store_sel)
+template <int E, typename T> __device__ __forceinline__ void ll_write16(const void* base, unsigned slot_off, int row, int k0, const float* v, int t, u64 near) {
   if constexpr (E == 1) {  // one 32-bit tagged half of a word; the other half belongs to another lane
-    ll_store32(reinterpret_cast<unsigned*>(slot) + ST16::frag_elem(row, k0), (tag16(t) << 16) | (H16<T>::pack2(v[0], 0.f) & 0xffffu));
+    const unsigned wv[1] = {(tag16(t) << 16) | (H16<T>::pack2(v[0], 0.f) & 0xffffu)};
+    ll_store_sel<1, 0>(base, slot_off + (unsigned)ST16::frag_elem(row, k0) * 4u, wv, near);
   } else {
-    const int q = ST16::frag_elem(row, k0) >> 1;
+    u64 wv[E / 2];
 #pragma unroll
-    for (int k = 0; k < E / 2; ++k) ll_store(slot + q + k, ll_pack16<T>(v[2 * k], v[2 * k + 1], t));
+    for (int k = 0; k < E / 2; ++k) wv[k] = ll_pack16<T>(v[2 * k], v[2 * k + 1], t);
+    ll_store_sel<E / 2, 8>(base, slot_off + (unsigned)(ST16::frag_elem(row, k0) >> 1) * 8u, wv, near);
   }
 }
-template <int E> __device__ __forceinline__ void ll_write(bf16_t*, u64* slot, int row, int k0, const float* v, int t) { ll_write16<E, bf16_t>(slot, row, k0, v, t); }
-template <int E> __device__ __forceinline__ void ll_write(half_t*, u64* slot, int row, int k0, const float* v, int t) { ll_write16<E, half_t>(slot, row, k0, v, t); }
-template <int E> __device__ __forceinline__ void ll_write(float*, u64* slot, int row, int k0, const float* v, int t) {
+template <int E> __device__ __forceinline__ void ll_write(bf16_t*, const void* base, unsigned slot_off, int row, int k0, const float* v, int t, u64 near) { ll_write16<E, bf16_t>(base, slot_off, row, k0, v, t, near); }
+template <int E> __device__ __forceinline__ void ll_write(half_t*, const void* base, unsigned slot_off, int row, int k0, const float* v, int t, u64 near) { ll_write16<E, half_t>(base, slot_off, row, k0, v, t, near); }
+template <int E> __device__ __forceinline__ void ll_write(float*, const void* base, unsigned slot_off, int row, int k0, const float* v, int t, u64 near) {
+  // (k0 is a multiple of E <= 4: the E elements sit in one group of 4 k, 16 words apart)
+  u64 wv[E];
 #pragma unroll
-  for (int i = 0; i < E; ++i) ll_store(slot + ST<float>::frag_elem(row, k0 + i), ll_pack((float*)0, v[i], t));
+  for (int i = 0; i < E; ++i) wv[i] = ll_pack((float*)0, v[i], t);
+  ll_store_sel<E, 128>(base, slot_off + (unsigned)ST<float>::frag_elem(row, k0) * 8u, wv, near);
+}
+
+// Do the KW workgroups of one group run on one XCD?  The launch places them on workgroup ids that are congruent
+// mod 8, which the dispatcher hands to one XCD; this handshake checks it where it matters, once per launch: every
+// workgroup publishes the id of its XCD (agent scope, visible anywhere) in the group's `words` (KW of them, zero at
+// launch) and waits, bounded, for the others.  Called by the first wave of the workgroup; returns 1 if all ids
+// agree (workgroup-scope exchange stores are then seen by the whole group), 0 if not, -1 if the wait ran out.
+template <int KW>
+__device__ __forceinline__ int xcd_handshake(int* words, int slice, int lane, int* status, int spin_limit) {
+  static_assert(KW <= 64, "one lane per workgroup of the group");
+  if (spin_limit < -1) return -1;  // host-side test hook: every wait gives up at once
+  unsigned x;
+  asm volatile("s_getreg_b32 %0, hwreg(HW_REG_XCC_ID)" : "=s"(x));
+  const int mine = (int)(x & 15u) + 1;
+  if (lane == 0) __hip_atomic_store(words + slice, mine, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  int v = mine;
+  for (int spins = 0;; ++spins) {
+    if (lane < KW) v = __hip_atomic_load(words + lane, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (__all(v != 0)) break;
+    if (spins > spin_limit) return -1;
+    if ((spins & 63) == 63 &&
+        __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return -1;
+  }
+  return __all(v == mine) ? 1 : 0;
 }
 
 // The words thread `tid` of NT polls, for a [rows_valid x KDIM] vector without the `own` columns

@@ -44,6 +44,7 @@ struct BwdArgs {
   void* ds0;       // [S,B,N,D]
   float* dbp;      // [batch tiles][G_t][N][D] partial bias sums
   u64* ll; int* status;
+  int* xcd;        // 32 words per group for xcd_handshake (zero at launch), or null: exchange stores stay agent scope
   int B, T, N;
   int grp0, groups, groups_total, tile_rows;
   int spin_limit, poll_delay;
@@ -136,7 +137,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   // a static LDS word, not a slice of the dynamic array: through a pointer computed from the
   // dynamic array the compiler reads the flag with a flat load, which has to wait for every global
   // load in flight (measured: the operand prefetch's full HBM latency, once per step)
-  __shared__ int dead_flag_word;
+  __shared__ int dead_flag_word, near_word;
   int* const dead_flag = &dead_flag_word;
 
   int grp_l, slice;
@@ -341,7 +342,16 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   for (int u = 0; u < UTW; ++u)
 #pragma unroll
     for (int k = 0; k < S; ++k) sn[u][k] = buf_load<ND_, SB>(rSt, st_v[u], ((unsigned)k * B * Tn + (Tn - 1)) * ND * ES);
+  // exchange stores may stay in the L2 of the XCD once the group is known to share one
+  if (KW > 1 && w == 0) {
+    const int r = (a.xcd && !a.cut) ? xcd_handshake<KW>(a.xcd + (size_t)grp * 32, slice, lane, a.status, a.spin_limit) : 0;
+    if (lane == 0) near_word = r;
+  }
   __syncthreads();
+  const int near_i = KW > 1 ? __builtin_amdgcn_readfirstlane(near_word) : 0;  // 1: stores stay in the XCD's L2, -1: wait ran out
+  u64 near_m;  // lane mask for ll_store_sel: all ones or zero, in scalar registers
+  asm("s_cmp_gt_i32 %1, 0\n\ts_cselect_b64 %0, -1, 0" : "=s"(near_m) : "s"(near_i) : "scc");
+  const int w_u = __builtin_amdgcn_readfirstlane(w);
 
 #ifdef FRNN_TRACE
   long long tr[5] = {0, 0, 0, 0, 0};
@@ -434,7 +444,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     rebuild_gates(pre[0], Tn - 1);
   }
 
-  bool dead = false, fail = false;
+  bool dead = near_i < 0, fail = false;
   // one reverse step: consumes `pc` (operands of step t), prefetches those of step t-1 into `pn`.
   // CUT (a std::bool_constant): truncated backpropagation, the step ends with the pointwise carry;
   // it is a compile-time variant of the step so that the full step carries no trace of it
@@ -551,7 +561,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (GROUPED) {
-      IW* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
+      const unsigned sslot = ((unsigned)(bvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
       auto send_group = [&](int r0, int nr, f32x4 (&ag)[RI][UTW]) __attribute__((always_inline)) {
 #pragma unroll
         for (int rr = 0; rr < RI; ++rr) {
@@ -561,9 +571,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
           for (int u = 0; u < UTW; ++u) {
             float part[E];
             own_elems<TR>(ag[rr][u], part);
-            IW* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
+            IW wv[E];
 #pragma unroll
-            for (int e = 0; e < E; ++e) ll_store(dst + e * 64, part_pack((PT*)0, part[e], t));
+            for (int e = 0; e < E; ++e) wv[e] = part_pack((PT*)0, part[e], t);
+            // (the destination's place in the area is uniform and goes into the scalar base; the lane's offset is the same for all)
+            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * WAVES + w_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
           }
         }
       };
@@ -676,7 +688,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     FRNN_STAMP(c3);
     if constexpr (KW > 1) {
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
-      IW* const sslot = inbox + (size_t)(bvalid ? (t & 1) : 2) * INW;
+      const unsigned sslot = ((unsigned)(bvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
 #pragma unroll
       for (int r = 1; r < (GROUPED ? 0 : KW); ++r) {
         const int x = (slice + r) % KW;
@@ -684,9 +696,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         for (int u = 0; u < UTW; ++u) {
           float part[E];
           own_elems<TR>(acc[r][u], part);
-          IW* dst = sslot + (((size_t)(x * WAVES + w) * UTW + u) * KW + slice) * 256 + lane;
+          IW wv[E];
 #pragma unroll
-          for (int e = 0; e < E; ++e) ll_store(dst + e * 64, part_pack((PT*)0, part[e], t));
+          for (int e = 0; e < E; ++e) wv[e] = part_pack((PT*)0, part[e], t);
+          // (the destination's place in the area is uniform and goes into the scalar base; the lane's offset is the same for all)
+            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * WAVES + w_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
         }
       }
       if constexpr (DW_LATE) {

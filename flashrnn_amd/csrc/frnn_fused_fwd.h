@@ -27,6 +27,7 @@ struct FwdArgs {
   const void* Wx; const void* R; const void* b; const void* s0;
   void* states; void* cache;
   u64* ll; int* status;
+  int* xcd;          // 32 words per group for xcd_handshake (zero at launch), or null: exchange stores stay agent scope
   int B, T, N;
   int grp0, groups, groups_total;  // this launch handles groups [grp0, grp0 + groups)
   int tile_rows;                   // batch rows per group: 4, 8 or 16
@@ -96,7 +97,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr unsigned ES = sizeof(T);
 
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
-  __shared__ int dead_flag;
+  __shared__ int dead_flag, near_word;
   constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
@@ -233,13 +234,22 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   };
 #pragma unroll
   for (int i = 0; i < PD; ++i) load_wx(wx[i], min(i, Tn - 1));
+  // exchange stores may stay in the L2 of the XCD once the group is known to share one (a single step sends
+  // nothing that is read)
+  if (KW > 1 && w == 0) {
+    const int r = (a.xcd && Tn > 1 && !a.step) ? xcd_handshake<KW>(a.xcd + (size_t)grp * 32, slice, lane, a.status, a.spin_limit) : 0;
+    if (lane == 0) near_word = r;
+  }
   __syncthreads();
+  const int near_i = KW > 1 ? __builtin_amdgcn_readfirstlane(near_word) : 0;  // 1: stores stay in the XCD's L2, -1: wait ran out
+  u64 near_m;  // lane mask for ll_store_sel: all ones or zero, in scalar registers
+  asm("s_cmp_gt_i32 %1, 0\n\ts_cselect_b64 %0, -1, 0" : "=s"(near_m) : "s"(near_i) : "scc");
 
 #ifdef FRNN_TRACE
   long long tr[3] = {0, 0, 0};
   const long long tr_begin = clock64();
 #endif
-  bool dead = false;
+  bool dead = near_i < 0;
   // one time step: consumes `wc` (Wx of step t), prefetches Wx of step t+PD into `wn`
   auto step = [&](const int t, Dw<ND_> (&wc)[UTW][GW], Dw<ND_> (&wn)[UTW][GW]) __attribute__((always_inline)) {
     const int cur = t & 1;
@@ -369,7 +379,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       }
       // the new h first: it is what the next step (of every workgroup of the head) waits for
       // (the own slice goes straight to the LDS buffer of the next step: the workgroup does not poll it)
-      if (KW > 1) ll_write<E>((T*)0, llbase + (size_t)(bvalid ? (t & 1) : 2) * LLW, brow, ub[u] + esub, so[0], t);
+      if (KW > 1) ll_write<E>((T*)0, llbase, (unsigned)(bvalid ? (t & 1) : 2) * (unsigned)(LLW * 8), brow, ub[u] + esub, so[0], t, near_m);
       lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
 #pragma unroll
       for (int k = 0; k < S; ++k)

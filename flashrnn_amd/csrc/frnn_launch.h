@@ -29,7 +29,9 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
 #define FRNN_TU_T float
 #endif
 #if FRNN_F == 0 || FRNN_F == 1
-#if FRNN_DT != 1
+#if FRNN_DT != 1 && FRNN_F == 1
+#define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_SLSTM_BF16
+#elif FRNN_DT != 1
 #define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_GR4_BF16
 #else
 #define FRNN_TU_BWD_RC_PLANS FRNN_BWD_RC_PLANS_GR4_F32

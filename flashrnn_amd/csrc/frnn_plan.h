@@ -78,6 +78,9 @@ struct Plan {
 // fit (gru D = 192 runs as 3 workgroups of 4 waves here: 12 waves have 168 registers each)
 #define FRNN_BWD_RC_PLANS_GR4_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8)
+// slstm: D = 192 stops at 8-row tiles (its 16-row kernel, with both operands resident and four states, spills)
+#define FRNN_BWD_RC_PLANS_SLSTM_BF16(X) \
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 8) X(256, 0, 4, 1, 4, 8)
 #define FRNN_BWD_RC_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
 #define FRNN_BWD_RC_PLANS_GR4_F32(X) X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16)

@@ -240,6 +240,32 @@ def test_cooperative_launch_gives_the_same_result(gpu, function, B, T, N, D, mon
         assert torch.equal(a, b)
 
 
+@pytest.mark.parametrize("function,B,T,N,D,dtype", [
+    ("lstm", 8, 24, 3, 256, torch.bfloat16), ("elman", 9, 20, 1, 1024, torch.bfloat16), ("gru", 5, 9, 1, 256, torch.float32),
+])
+def test_agent_scope_exchange_stores_give_the_same_result(gpu, function, B, T, N, D, dtype, monkeypatch):
+    """The workgroups of a head exchange h (forward) and partial sums (backward) through tagged words.  When a
+    group's workgroups share an XCD (checked by the kernels at launch) the stores stay in that XCD's L2; otherwise,
+    or with FRNN_AGENT_STORES=1, they are written through to memory.  Both paths carry the same words: same bits."""
+    print(f"case agent stores {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
+    inp = make_inputs(function, B, T, N, D, 33, init="randn", round_to=dtype)
+
+    def run():
+        from flashrnn_amd import flashrnn
+
+        leaves = [inp[k].to(gpu, dtype).requires_grad_(True) for k in ("Wx", "R", "b", "states")]
+        out, _ = flashrnn(*leaves, function=function, backend="hip_fused", dtype={torch.bfloat16: "bfloat16", torch.float32: "float32"}[dtype])
+        g = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(gpu, dtype))
+        torch.cuda.synchronize()
+        return (out,) + g
+
+    near = run()
+    monkeypatch.setenv("FRNN_AGENT_STORES", "1")
+    far = run()
+    for a, b in zip(near, far):
+        assert torch.equal(a, b)
+
+
 @pytest.mark.parametrize("function,B,N,D,note", [
     ("lstm", 80, 1, 768, "12 workgroups per head: an XCD of 32 compute units holds 2 groups, a launch 16; 20 groups"),
     ("slstm", 100, 4, 192, "3 workgroups per head forward: 10 groups per XCD, 80 per launch; 100 groups"),
