@@ -82,7 +82,11 @@ template <> struct ST<half_t> : ST16 {
 };
 template <> struct ST<float> {
   static constexpr int KM = 4, EPW = 1, ID = FRNN_F32;
+#ifdef FRNN_F32_PRECISE
   static constexpr bool FAST = false;
+#else
+  static constexpr bool FAST = true;
+#endif
   typedef float Frag;
   typedef float4 Vec4;
   static __device__ __forceinline__ int frag_elem(int row, int k) {
@@ -92,6 +96,17 @@ template <> struct ST<float> {
     return __builtin_amdgcn_mfma_f32_16x16x4f32(a, b, c, 0, 0, 0);
   }
 };
+
+// 16 consecutive k of a product on v_mfma_f32_4x4x1_16B_f32: k-th instruction with the A values (4 rows) of block
+// k of `a` broadcast to all 16 blocks (CBSZ = 4, ABID = k: immediates of the instruction), B = b[k] (per block 4
+// columns), accumulating round robin into the 4 chains acc[0..3] (first: the chains start from zero).
+__device__ __forceinline__ void mfma_4x4x1_bcast16(float a, const float* b, f32x4 (&acc)[4], bool first) {
+  const f32x4 z = {0.f, 0.f, 0.f, 0.f};
+#define FRNN_K(i) acc[i & 3] = __builtin_amdgcn_mfma_f32_4x4x1f32(a, b[i], (first && i < 4) ? z : acc[i & 3], 4, i, 0);
+  FRNN_K(0) FRNN_K(1) FRNN_K(2) FRNN_K(3) FRNN_K(4) FRNN_K(5) FRNN_K(6) FRNN_K(7)
+  FRNN_K(8) FRNN_K(9) FRNN_K(10) FRNN_K(11) FRNN_K(12) FRNN_K(13) FRNN_K(14) FRNN_K(15)
+#undef FRNN_K
+}
 
 __device__ __forceinline__ float bf2f(unsigned short u) { return __uint_as_float(((unsigned)u) << 16); }
 __device__ __forceinline__ unsigned short f2bf(float f) {  // round to nearest even; NaN stays NaN

@@ -49,6 +49,35 @@ template <int TR> __device__ __forceinline__ void own_elems(const f32x4& acc, fl
   else { out[0] = quarter_pick(half_pick(acc[0], acc[2]), half_pick(acc[1], acc[3])); }
 }
 
+// fp32 vector of a 4-row tile as the broadcast operand of v_mfma_f32_4x4x1_16B_f32: element (row, k) at
+// k*4 + row, so that lane l reads the operand of the 16 k-values 16v .. 16v+15 with one access at 64v + l
+__device__ __forceinline__ int lds_index4(int row, int k) { return k * 4 + row; }
+// the same from the element's position in an exchange slot (fp32 fragment order, ST<float>::frag_elem)
+__device__ __forceinline__ int lds_index4_of_word(int word) { return (((word >> 6) << 2) + ((word >> 4) & 3)) * 4 + (word & 15); }
+
+// 4x4 transpose between the lanes of a quad and 4 registers: lane j of a quad passes r[i] = M[j][i] and
+// gets r[i] = M[i][j] (two butterfly steps: partner lane ^ 1 with registers (0,1), (2,3), then lane ^ 2 with
+// (0,2), (1,3))
+__device__ __forceinline__ float quad_xor1(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0xB1 /* quad_perm:[1,0,3,2] */, 0xF, 0xF, false));
+}
+__device__ __forceinline__ float quad_xor2(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), 0x4E /* quad_perm:[2,3,0,1] */, 0xF, 0xF, false));
+}
+__device__ __forceinline__ void quad_transpose(float (&r)[4], int lane) {
+  const bool b0 = lane & 1, b1 = lane & 2;
+  {
+    const float x0 = quad_xor1(b0 ? r[0] : r[1]), x1 = quad_xor1(b0 ? r[2] : r[3]);
+    r[0] = b0 ? x0 : r[0]; r[1] = b0 ? r[1] : x0;
+    r[2] = b0 ? x1 : r[2]; r[3] = b0 ? r[3] : x1;
+  }
+  {
+    const float x0 = quad_xor2(b1 ? r[0] : r[2]), x1 = quad_xor2(b1 ? r[1] : r[3]);
+    r[0] = b1 ? x0 : r[0]; r[2] = b1 ? r[2] : x0;
+    r[1] = b1 ? x1 : r[1]; r[3] = b1 ? r[3] : x1;
+  }
+}
+
 // LDS writes of E consecutive elements (row, k0..k0+E-1) in fragment order; k0 % E == 0
 template <int E, typename T> __device__ __forceinline__ void lds_write16(T* buf, int row, int k0, const float* v) {
   const Dw<(E + 1) / 2> p = pack16<E, T>(v);
@@ -272,7 +301,8 @@ __device__ __forceinline__ bool ll_gather_pairs(rsrc_t slots, unsigned soff, con
 }
 
 // Forward gather: poll the planned words of slot, then copy their payloads to LDS.
-template <typename T, int NP>
+// C4: the LDS vector is kept as [k][4 rows] (the fp32 4-row tiles, see lds_index4) instead of fragment order
+template <typename T, int NP, bool C4 = false>
 __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, T* lds_dst,
                                           int* status, int spin_limit, int first_delay) {
   constexpr int CH = NP < 16 ? NP : 16;  // words polled together
@@ -287,7 +317,7 @@ __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, 
     if (!fail) {
 #pragma unroll
       for (int i = 0; i < CH; ++i)
-        if (need[i]) reinterpret_cast<unsigned*>(lds_dst)[off[i]] = ll_payload((T*)0, v[i]);
+        if (need[i]) reinterpret_cast<unsigned*>(lds_dst)[C4 ? lds_index4_of_word(off[i]) : off[i]] = ll_payload((T*)0, v[i]);
     }
   }
   return fail;

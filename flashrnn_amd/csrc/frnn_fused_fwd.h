@@ -96,6 +96,12 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
   constexpr unsigned ES = sizeof(T);
 
+  // fp32, 4-row batch tiles, cells with 3 or 4 recurrent gates: the product runs on v_mfma_f32_4x4x1_16B_f32 with
+  // the 4 batch rows on the 4-wide side, so that no MFMA work goes into padded batch columns (the 16x16x4
+  // instruction computes 16 columns, 12 of them padding, at the same rate).  Block = unit of the tile, the 4
+  // columns of a block = the gates of that unit, A = h (the values of one block broadcast to all 16), one
+  // instruction per k: D instructions of 8 cycles per tile and step instead of G_r * D / 4 of 32.
+  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && GR >= 3;
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
   __shared__ int dead_flag, near_word;
   constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
@@ -141,8 +147,24 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int PIN_REGS = RF_REGS > 160 ? (RF_REGS < 232 ? RF_REGS : 232) : 0;  // (160 registers, D = 320: measured no gain)
   Frag rf[UTW][GR][KSR];
   Frag* const rl = rlds + (size_t)w * RLK * UTW * GR * 64 + lane;
+  static_assert(!M44 || RLK == 0, "4x4x1 form: the whole operand in registers");
+  // 4x4x1 form: lane 4*blk + j holds row (gate j, unit blk of the tile) of R, one register per k
+  float rb[M44 ? UTW : 1][M44 ? D : 1];
+  if constexpr (M44) {
+    const int blk = lane >> 2, j = lane & 3;
 #pragma unroll
-  for (int u = 0; u < UTW; ++u)
+    for (int u = 0; u < UTW; ++u) {
+      const float* row = reinterpret_cast<const float*>(R) + ((size_t)((j < GR ? j : 0) * N + n) * D + ub[u] + blk) * D;
+#pragma unroll
+      for (int k = 0; k < D; k += 4) {
+        const float4 v = *reinterpret_cast<const float4*>(row + k);
+        rb[u][k] = j < GR ? v.x : 0.f; rb[u][k + 1] = j < GR ? v.y : 0.f;
+        rb[u][k + 2] = j < GR ? v.z : 0.f; rb[u][k + 3] = j < GR ? v.w : 0.f;
+      }
+    }
+  }
+#pragma unroll
+  for (int u = 0; u < (M44 ? 0 : UTW); ++u)
 #pragma unroll
     for (int g = 0; g < GR; ++g) {
       const T* row = R + ((size_t)(g * N + n) * D + ub[u] + r16) * D;
@@ -198,14 +220,22 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 
   // ---- h_0 of the whole head -> LDS (rows beyond B are zero and stay zero or private to their
   //      own MFMA column, so they never reach a valid row) --------------------------------------
-  for (int idx = tid; idx < 16 * D / 4; idx += NT) {
+  for (int idx = tid; idx < (M44 ? 4 : 16) * D / 4; idx += NT) {
     const int row = idx / (D / 4), k0 = (idx % (D / 4)) * 4;
     float v[4] = {0.f, 0.f, 0.f, 0.f};
     const bool rv = row < TR && bt * TR + row < B;
     if (rv) unpack4<T>(*reinterpret_cast<const Vec4*>(s0 + (size_t)(bt * TR + row) * ND + (size_t)n * D + k0), v);
-    lds_write<4>(hbuf[0], row, k0, v);
-    if (KW > 1 || TR < 16) {  // rows that are never rewritten must be finite in both buffers
-      if (!rv) lds_write<4>(hbuf[1], row, k0, v);
+    if constexpr (M44) {
+#pragma unroll
+      for (int i = 0; i < 4; ++i) {
+        reinterpret_cast<float*>(hbuf[0])[lds_index4(row, k0 + i)] = v[i];
+        if (!rv) reinterpret_cast<float*>(hbuf[1])[lds_index4(row, k0 + i)] = v[i];
+      }
+    } else {
+      lds_write<4>(hbuf[0], row, k0, v);
+      if (KW > 1 || TR < 16) {  // rows that are never rewritten must be finite in both buffers
+        if (!rv) lds_write<4>(hbuf[1], row, k0, v);
+      }
     }
   }
 
@@ -258,7 +288,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       if (KW > 1) {
         bool fail;
         if constexpr (PAIRS) fail = ll_gather_pairs<T, NP>(rLL, (unsigned)((t - 1) & 1) * LLW * 8u, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
-        else fail = ll_gather<T, NP>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
+        else fail = ll_gather<T, NP, M44>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
         if (barrier_or(fail, &dead_flag)) { dead = true; return; }
       } else {
         lds_barrier();
@@ -270,6 +300,30 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once
     // NACC accumulators per (tile, gate), used round robin over the k-steps, so that at least ~4
     // independent MFMA chains are in flight (a dependent MFMA waits ~3x longer than an independent one)
+    f32x4 acc[UTW][GR];
+    float ry44[M44 ? UTW : 1][4];  // 4x4x1 form: the lane's element, gates 0..3
+    if constexpr (M44) {
+      const float* hf = reinterpret_cast<const float*>(hbuf[cur]) + lane;
+      float ha[D / 16];
+#pragma unroll
+      for (int v = 0; v < D / 16; ++v) ha[v] = hf[64 * v];
+      __builtin_amdgcn_sched_barrier(0);
+      f32x4 ac[UTW][4];  // 4 independent accumulation chains per tile
+#pragma unroll
+      for (int v = 0; v < D / 16; ++v) {
+#pragma unroll
+        for (int u = 0; u < UTW; ++u) mfma_4x4x1_bcast16(ha[v], &rb[u][16 * v], ac[u], v == 0);
+      }
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) {
+        const f32x4 sum = (ac[u][0] + ac[u][1]) + (ac[u][2] + ac[u][3]);
+        // lane 4*blk + j holds (gate j, unit blk) of batch rows 0..3; after the transpose lane 4*blk + b holds
+        // gates 0..3 of (batch row b, unit blk): the element that Own<4> gives this lane
+        ry44[u][0] = sum[0]; ry44[u][1] = sum[1]; ry44[u][2] = sum[2]; ry44[u][3] = sum[3];
+        quad_transpose(ry44[u], lane);
+      }
+    }
+    if constexpr (!M44) {
     constexpr int NACC_ = UTW * GR >= 3 ? 1 : (UTW * GR == 2 ? 2 : 4);
     constexpr int NACC = NACC_ < KS ? NACC_ : KS;
     f32x4 accp[NACC][UTW][GR];
@@ -325,7 +379,6 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         if (j == NACC - 1) __builtin_amdgcn_sched_barrier(0);
       }
     }
-    f32x4 acc[UTW][GR];
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
@@ -334,6 +387,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
         for (int j = 1; j < NACC; ++j) acc[u][g] += accp[j][u][g];
       }
+    }  // !M44
 
     if constexpr (WX_LATE) {
       load_wx(wn, min(t + PD, Tn - 1));
@@ -344,7 +398,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #pragma unroll
       for (int u = 0; u < UTW; ++u)
 #pragma unroll
-        for (int g = 0; g < GR; ++g) sink += acc[u][g][0];
+        for (int g = 0; g < GR; ++g) sink += M44 ? ry44[u][g] : acc[u][g][0];
       asm volatile("" ::"v"(sink)); }
 #endif
     FRNN_STAMP(c2);
@@ -353,7 +407,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       float ryv[GR][E], wxv[GW][E];
 #pragma unroll
       for (int g = 0; g < GR; ++g) {
-        own_elems<TR>(acc[u][g], ryv[g]);
+        if constexpr (M44) ryv[g][0] = ry44[u][g];
+        else own_elems<TR>(acc[u][g], ryv[g]);
         if constexpr (!BIAS_C) {
 #pragma unroll
           for (int e = 0; e < E; ++e) ryv[g][e] += bown[u][g][e];
@@ -380,7 +435,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       // the new h first: it is what the next step (of every workgroup of the head) waits for
       // (the own slice goes straight to the LDS buffer of the next step: the workgroup does not poll it)
       if (KW > 1) ll_write<E>((T*)0, llbase, (unsigned)(bvalid ? (t & 1) : 2) * (unsigned)(LLW * 8), brow, ub[u] + esub, so[0], t, near_m);
-      lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
+      if constexpr (M44) reinterpret_cast<float*>(hbuf[cur ^ 1])[lds_index4(brow, ub[u] + esub)] = so[0][0];
+      else lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);

@@ -70,13 +70,17 @@ def test_recompute_with_clip_and_cut(gpu, options, function, B, T, N, D, dtype):
 
 
 @pytest.mark.parametrize("function", ["lstm", "gru"])
-def test_recompute_in_fp32_gives_the_bits_of_the_cached_path(gpu, function):
-    """fp32 storage: the stored h is what the forward pass fed to its product, the rebuild runs the same MFMA
-    chain and the same gate math, so every gradient must come out bit for bit as with the cache."""
+@pytest.mark.parametrize("tile_rows", [8, 4])
+def test_recompute_in_fp32_gives_the_bits_of_the_cached_path(gpu, function, tile_rows, monkeypatch):
+    """fp32 storage: the stored h is what the forward pass fed to its product.  With 8-row tiles the rebuild runs the
+    same MFMA chain and the same gate math as the forward pass, so every gradient must come out bit for bit as with
+    the cache.  With 4-row tiles the forward product runs on the 4x4x1 instruction (another summation order) and
+    the rebuild on the 16x16x4 one: equal to fp32 rounding."""
     from flashrnn_amd import FlashRNNConfig, flashrnn
 
     B, T, N, D = 7, 33, 2, 64
-    print(f"case recompute bits {function}", flush=True)
+    print(f"case recompute bits {function} rows {tile_rows}", flush=True)
+    monkeypatch.setenv("FRNN_TILE_ROWS", str(tile_rows))
     inp = make_inputs(function, B, T, N, D, 84, init="randn")
     res = []
     for rc in (False, True):
@@ -87,7 +91,10 @@ def test_recompute_in_fp32_gives_the_bits_of_the_cached_path(gpu, function):
         res.append((out,) + torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(gpu)))
     torch.cuda.synchronize()
     for name, a, c in zip(("states", "dWx", "dR", "db", "ds0"), *res):
-        assert torch.equal(a, c), f"{name}: max diff {(a - c).abs().max().item():.3e}"
+        if tile_rows == 8:
+            assert torch.equal(a, c), f"{name}: max diff {(a - c).abs().max().item():.3e}"
+        else:
+            assert float((a - c).abs().max()) <= 1e-5 * max(1.0, float(c.abs().max())), name
 
 
 def test_recompute_has_no_cache_and_refuses_what_it_cannot_do(gpu):
