@@ -122,6 +122,14 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
   constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
   constexpr unsigned ES = sizeof(T);
+  // fp32, 4-row batch tiles, several workgroups per head: the product runs on v_mfma_f32_4x4x1_16B_f32 with the 4
+  // batch rows on the 4-wide side (see the forward kernel).  Block = previous unit p of a destination tile, the 4
+  // columns of a block = 4 destination workgroups (the wave's tile position in each), A = dg of the own gate rows
+  // (the values of one block broadcast to all 16), one instruction per k: KDL instructions of 8 cycles per 4
+  // destinations instead of KDL / 4 of 32 per destination.
+  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && KW >= 2 && !RC &&
+                       bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)) == 0;  // (the whole operand in registers)
+  constexpr int NG4 = (KW + 3) / 4;  // groups of 4 destinations
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);
@@ -180,8 +188,28 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   constexpr int FRAG_REGS = (int)sizeof(Frag) / 4, RTF_REGS = KWR * UTW * KS * FRAG_REGS;
   constexpr int PIN_REGS = RC ? 0 : RTF_REGS > 160 ? (RTF_REGS < 232 ? RTF_REGS : 232) : 0;
   Frag rtf[KWR][UTW][KS];
+  // 4x4x1 form: lane 4*blk + j holds row p = (tile of destination 4q + j, unit blk) of R^T, one register per own k
+  float rtb[M44 ? NG4 : 1][M44 ? UTW : 1][M44 ? KDL : 1];
+  if constexpr (M44) {
+    const int blk = lane >> 2, j = lane & 3;
 #pragma unroll
-  for (int r = 0; r < KW; ++r) {
+    for (int q = 0; q < NG4; ++q) {
+      const int r = 4 * q + j;
+      const int x = (slice + (r < KW ? r : 0)) % KW;
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) {
+        const float* row = reinterpret_cast<const float*>(Rt) + ((size_t)n * D + (x * UT_WG + w * UTW + u) * 16 + blk) * (GR * D) + slice * DL;
+#pragma unroll
+        for (int kk = 0; kk < KDL; kk += 4) {
+          const float4 v = *reinterpret_cast<const float4*>(row + (kk / DL) * D + (kk % DL));
+          rtb[q][u][kk] = r < KW ? v.x : 0.f; rtb[q][u][kk + 1] = r < KW ? v.y : 0.f;
+          rtb[q][u][kk + 2] = r < KW ? v.z : 0.f; rtb[q][u][kk + 3] = r < KW ? v.w : 0.f;
+        }
+      }
+    }
+  }
+#pragma unroll
+  for (int r = 0; r < (M44 ? 0 : KW); ++r) {
     const int x = (slice + r) % KW;
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
@@ -514,7 +542,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
       if constexpr (!cut) {
 #pragma unroll
-        for (int g = 0; g < GR; ++g) lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
+        for (int g = 0; g < GR; ++g) {
+          if constexpr (M44) reinterpret_cast<float*>(gb)[lds_index4(brow, g * DL + (ub[u] + esub - slice * DL))] = dgr[g][0];
+          else lds_write<E>(gb, brow, g * DL + (ub[u] + esub - slice * DL), dgr[g]);
+        }
       }
     }
     if constexpr (RC) {
@@ -537,20 +568,43 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     // With 3 and more workgroups per head the products that other workgroups wait for come first
     // and are sent at once; the product for the own tiles follows while those words travel (it
     // needs all fragments still in registers: one chunk)
-    constexpr bool OWN_LAST = KW >= 3 && KS == chunk_of(KS);
+    constexpr bool OWN_LAST = KW >= 3 && KS == chunk_of(KS) && !M44;
     // More than 8 remote destinations (10 and more workgroups per head): their products run in groups
     // of 4 destinations (4 independent MFMA chains), each group sent as soon as it is complete, so that
     // 16 accumulator registers are live instead of 4 per destination (128 at 32 workgroups per head).
     constexpr bool GROUPED = OWN_LAST && KW - 1 > 8;
     constexpr int RI = 4;
     static_assert(!GROUPED || RLD % RI == 0, "LDS-resident destinations come in whole groups");
+    float p44[M44 ? NG4 : 1][M44 ? UTW : 1][4];  // 4x4x1 form: partial sums of the lane's element, destination 4q + i
+    if constexpr (M44) {
+      const float* gfl = reinterpret_cast<const float*>(gb) + lane;
+      float ga[KDL / 16];
+#pragma unroll
+      for (int v = 0; v < KDL / 16; ++v) ga[v] = gfl[64 * v];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int q = 0; q < NG4; ++q)
+#pragma unroll
+        for (int u = 0; u < UTW; ++u) {
+          f32x4 ac[4];
+#pragma unroll
+          for (int v = 0; v < KDL / 16; ++v) mfma_4x4x1_bcast16(ga[v], &rtb[q][u][16 * v], ac, v == 0);
+          const f32x4 sum = (ac[0] + ac[1]) + (ac[2] + ac[3]);
+          // lane 4*blk + j holds (destination 4q + j, unit blk) of batch rows 0..3; after the transpose lane
+          // 4*blk + b holds destinations 4q .. 4q+3 of (batch row b, unit blk): the element of this lane
+          p44[q][u][0] = sum[0]; p44[q][u][1] = sum[1]; p44[q][u][2] = sum[2]; p44[q][u][3] = sum[3];
+          quad_transpose(p44[q][u], lane);
+        }
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) ds[u][0][0] += p44[0][u][0];
+    }
     f32x4 accp[NACC][GROUPED ? 1 : KW][UTW];
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;
     constexpr int KC = chunk_of(KS);
     static_assert(KS % KC == 0, "k-steps must split into whole chunks");
     Frag gq[2][KC];
 #pragma unroll
-    for (int k = 0; k < KC; ++k) gq[0][k] = gf[k * 64];
+    for (int k = 0; k < (M44 ? 0 : KC); ++k) gq[0][k] = gf[k * 64];
     Frag la_next[RLD > 0 ? RLD : 1][UTW];
     if constexpr (RLD > 0 && !GROUPED) {
 #pragma unroll
@@ -630,7 +684,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
       }
     }
 #pragma unroll
-    for (int kc = 0; kc < (GROUPED ? 0 : KS / KC); ++kc) {
+    for (int kc = 0; kc < (GROUPED || M44 ? 0 : KS / KC); ++kc) {
       if (kc + 1 < KS / KC) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) gq[(kc + 1) & 1][k] = gf[((kc + 1) * KC + k) * 64];
@@ -666,10 +720,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     static_assert(NACC == 1, "one accumulator per tile");
     f32x4 acc[GROUPED ? 1 : KW][UTW];
 #pragma unroll
-    for (int r = OWN_LAST ? 1 : 0; r < (GROUPED ? 0 : KW); ++r)
+    for (int r = OWN_LAST ? 1 : 0; r < (GROUPED || M44 ? 0 : KW); ++r)
 #pragma unroll
       for (int u = 0; u < UTW; ++u) acc[r][u] = accp[0][r][u];
-    if constexpr (!OWN_LAST) {
+    if constexpr (!OWN_LAST && !M44) {
 #pragma unroll
       for (int u = 0; u < UTW; ++u) {
         float own[E];
@@ -695,7 +749,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #pragma unroll
         for (int u = 0; u < UTW; ++u) {
           float part[E];
-          own_elems<TR>(acc[r][u], part);
+          if constexpr (M44) part[0] = p44[r >> 2][u][r & 3];
+          else own_elems<TR>(acc[r][u], part);
           IW wv[E];
 #pragma unroll
           for (int e = 0; e < E; ++e) wv[e] = part_pack((PT*)0, part[e], t);

@@ -101,10 +101,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   // instruction computes 16 columns, 12 of them padding, at the same rate).  Block = unit of the tile, the 4
   // columns of a block = the gates of that unit, A = h (the values of one block broadcast to all 16), one
   // instruction per k: D instructions of 8 cycles per tile and step instead of G_r * D / 4 of 32.
-  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && GR >= 3;
+  constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
+  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && GR >= 3 && RLK == 0 && D <= 384;  // (the whole operand, D registers per tile, in registers)
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
   __shared__ int dead_flag, near_word;
-  constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
 
@@ -147,7 +147,6 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int PIN_REGS = RF_REGS > 160 ? (RF_REGS < 232 ? RF_REGS : 232) : 0;  // (160 registers, D = 320: measured no gain)
   Frag rf[UTW][GR][KSR];
   Frag* const rl = rlds + (size_t)w * RLK * UTW * GR * 64 + lane;
-  static_assert(!M44 || RLK == 0, "4x4x1 form: the whole operand in registers");
   // 4x4x1 form: lane 4*blk + j holds row (gate j, unit blk of the tile) of R, one register per k
   float rb[M44 ? UTW : 1][M44 ? D : 1];
   if constexpr (M44) {

@@ -42,10 +42,14 @@ struct Plan {
 #define FRNN_PLANS_SLSTM_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 4, 1, 3, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
+// fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave, so D = 512 is as far as one tile per
+// wave goes (2 waves per workgroup from D = 448 on, part of R in LDS); larger heads run on the alternating backend
 #define FRNN_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 8) X(448, 0, 2, 1, 14, 4) X(512, 0, 2, 1, 16, 4)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 4) X(448, 0, 2, 1, 14, 8) X(512, 0, 1, 1, 32, 4)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
@@ -54,9 +58,11 @@ struct Plan {
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 12, 1, 1, 4) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 8) X(512, 0, 4, 1, 8, 8)
 #define FRNN_BWD_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 8) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 8)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
@@ -67,11 +73,11 @@ struct Plan {
   X(256, 0, 16, 1, 1, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 8, 1, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 8, 1, 4, 16) X(640, 0, 4, 1, 10, 16) \
   X(768, 0, 8, 1, 6, 16) X(1024, 0, 8, 1, 8, 4)
 #define FRNN_PLANS_GR1_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 16) \
-  X(512, 0, 4, 2, 4, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 16) \
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 2, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 2, 4, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 8)
 #define FRNN_BWD_PLANS_GR1_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 8) \
-  X(512, 0, 4, 2, 4, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 8) \
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 2, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 2, 4, 8) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 16) X(1024, 0, 4, 1, 16, 8)
 
 // ---- reverse scan in recompute mode (no gate cache): R and R^T are both resident, so only the head
 // dims whose two operands fit the registers beside the working set; same tilings as above where those

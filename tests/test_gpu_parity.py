@@ -61,6 +61,24 @@ FUSED_SMALL = [
     ("slstm", 4, 6, 1, 640, "bfloat16"),
     ("gru", 6, 4, 1, 640, "bfloat16"),
     ("elman", 12, 5, 1, 640, "bfloat16"),
+    # fp32 beyond D = 256 (5 to 32 workgroups per head; from 384 on part of R / R^T lives in LDS)
+    ("lstm", 6, 5, 1, 160, "float32"),
+    ("gru", 5, 6, 2, 160, "float32"),
+    ("elman", 9, 5, 1, 160, "float32"),      # 10 waves
+    ("lstm", 5, 6, 1, 320, "float32"),
+    ("slstm", 7, 5, 1, 320, "float32"),
+    ("gru", 4, 5, 1, 320, "float32"),
+    ("lstm", 9, 4, 1, 384, "float32"),
+    ("gru", 6, 5, 1, 384, "float32"),
+    ("elman", 5, 6, 1, 384, "float32"),
+    ("lstm", 5, 5, 1, 448, "float32"),       # 14 workgroups of 2 waves
+    ("gru", 7, 4, 1, 448, "float32"),
+    ("lstm", 6, 6, 1, 512, "float32"),       # forward 16 workgroups of 2 waves, backward 32 of one wave
+    ("slstm", 4, 5, 1, 512, "float32"),
+    ("gru", 9, 4, 1, 512, "float32"),
+    ("elman", 7, 5, 1, 768, "float32"),
+    ("elman", 10, 4, 1, 1024, "float32"),
+    ("lstm", 37, 4, 1, 512, "float32"),      # 10 groups of 4 rows: two backward launches (8 groups of 32 workgroups each)
 ]
 
 
