@@ -10,6 +10,7 @@
 // transposed on their way into LDS (bf16; the fp32 MFMA takes them as they are).
 #include "frnn_grad.h"
 #include <cstdlib>
+#include <type_traits>
 
 namespace frnn {
 
@@ -50,60 +51,124 @@ __device__ __forceinline__ void gemm_tile_of(const GradGemmArgs& a, int TM, int&
 
 template <int WT>
 __device__ __forceinline__ void gemm_store_partial(const GradGemmArgs& a, int TM, int g, int n, int split, int dt, int pt,
-                                                   int wm, int wn, int r16, int q4, const f32x4 (&acc)[WT][WT]) {
+                                                   int wm, int wn, int r16, int q4, const f32x4 (&acc)[WT][WT], int span) {
   const int D = a.D;
   float* out = a.part + ((((size_t)split * a.GR + g) * a.N + n) * D) * D;
 #pragma unroll
   for (int i = 0; i < WT; ++i)
 #pragma unroll
     for (int j = 0; j < WT; ++j) {
-      const int d = dt * TM + wm * (TM / 2) + i * 16 + q4 * 4;
-      const int p = pt * TM + wn * (TM / 2) + j * 16 + r16;
+      const int d = dt * TM + wm * span + i * 16 + q4 * 4;  // span: units per wave
+      const int p = pt * TM + wn * span + j * 16 + r16;
 #pragma unroll
       for (int e = 0; e < 4; ++e) out[(size_t)(d + e) * D + p] = acc[i][j][e];
     }
 }
 
-// 16-bit storage types.  Both operands arrive with the contraction index as the slow one, so a stage
-// is transposed on its way into LDS: [unit][row pair], one dword = rows (2k, 2k+1) of a unit, 17 dwords
-// per unit (16 + 1 pad).  The odd stride puts the 64 lanes of a transposing store on 32 different banks
-// (a thread stores 4 adjacent units of one row pair, 16 threads cover 64 units, a wave 4 row pairs) and
-// keeps the fragment reads (4 consecutive dwords per lane) conflict-free; an 8-element row stride would
-// be a multiple of the bank count for every choice of padding that keeps 16-byte reads aligned
-// (measured: bank conflicts in 83 % of the LDS-active cycles, the kernel was LDS-bound).
-// Two stages alternate, so that one barrier per stage is enough: the global loads of stage s+1 are
-// issued before the MFMAs of stage s and stored to the other buffer after them.
-template <int TM> struct GemmStage16 {
-  static constexpr int LD = 17;
-  unsigned a[2][TM][LD], b[2][TM][LD];
-};
-
-template <typename T, int TM>
-__global__ void __launch_bounds__(256) grad_gemm16_kernel(const GradGemmArgs a) {
+// 16-bit storage types.  Both operands arrive with the contraction index as the slow one.  The stages are brought in
+// by direct global-to-LDS loads (global_load_lds_dwordx4: no registers, no LDS store instructions) and transposed on
+// their way OUT of LDS by ds_read_b64_tr_b16.  Workgroup tile TM x TM, WD x WD waves of (TM / WD)^2 each.
+//   LDS stage of one operand: [32 rows (b,t)][TM units], rows as they lie in memory.  A load instruction of a wave
+//   fills 1024 consecutive bytes (lane i writes bytes 16i..16i+15), which lane fetches which 16-byte chunk of the
+//   row is free to choose: the chunks of row r are stored at position (chunk ^ f(r)), f even, so that the
+//   transposing reads below, which touch 32 bytes of each of 8 rows at the same unit offset per pass, fall on 8
+//   different groups of 8 banks.
+//   ds_read_b64_tr_b16, as measured: in a group of 16 lanes, lane i receives element i % 4 of the 8-byte pieces
+//   that lanes i/4, i/4 + 4, i/4 + 8, i/4 + 12 point at.  Source lane s = a + 4j points at (row k0 + j, units
+//   u0 + 4a ..): lane i then holds rows k0 .. k0+3 of unit u0 + i, i.e. 4 consecutive k of its own MFMA row.  Two
+//   reads (k0 = 4q and 16 + 4q for lane group q) give the 8 k of a v_mfma_f32_16x16x32 operand; both operands use
+//   the same assignment of k to (group, element), which is all the instruction needs.
+//   NS stages are in flight: the loads of stage s + NS - 1 are issued right after the barrier that frees its
+//   buffer; one barrier per stage.
+template <typename T, int TM, int WD, int NS>
+__global__ void __launch_bounds__(64 * WD * WD) grad_gemm16_kernel(const GradGemmArgs a) {
   typedef ST<T> X;
   static_assert(sizeof(T) == 2, "16-bit storage types");
-  constexpr int WT = TM / 32;                     // MFMA tiles per wave per dimension
-  constexpr int TPR = TM >= 64 ? 16 : TM / 4;     // threads per row pair
-  constexpr int CH = TM / (4 * TPR);              // chunks of 4 units per thread and row
-  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];
-  GemmStage16<TM>& sm = *reinterpret_cast<GemmStage16<TM>*>(gemm_smem);
+  constexpr int NW = WD * WD, NT = 64 * NW;
+  constexpr int WT = TM / (16 * WD);    // MFMA tiles per wave per dimension
+  constexpr int CPR = TM / 8;           // 16-byte chunks per staged row
+  constexpr int KB = 32;                // rows (b,t) per stage
+  constexpr int OPB = KB * TM * 2;      // bytes of one operand of one stage
+  constexpr int IPW = CPR / NW;         // load instructions per wave and stage (CPR instructions: CPR/2 per operand)
+  static_assert(CPR >= NW && CPR % NW == 0 && NS >= 2, "every wave issues the same number of loads");
+  extern __shared__ __attribute__((aligned(16))) unsigned char gemm_smem[];  // [NS][operand][KB rows][TM units]
+  typedef __attribute__((address_space(3))) unsigned char lds_byte;
+  typedef short s16x4 __attribute__((ext_vector_type(4)));
+  typedef __attribute__((address_space(3))) s16x4 lds_s16x4;
+  lds_byte* const sm = (lds_byte*)gemm_smem;
 
   int g, dt, pt;
   gemm_tile_of(a, TM, g, dt, pt);
   const int n = blockIdx.y, split = blockIdx.z;
-  const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
-  const int wm = w >> 1, wn = w & 1;
+  const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int wm = w / WD, wn = w % WD;
   const int r16 = lane & 15, q4 = lane >> 4;
-  const int D = a.D, N = a.N, Tn = a.T;
+  const int N = a.N, Tn = a.T;
   const long rows = (long)a.B * Tn;
   const long r_begin = (long)split * a.rows_per_split;
   const long r_end = min(rows, r_begin + a.rows_per_split);
-  const size_t ND = (size_t)N * D;
+  const size_t ND = (size_t)N * a.D;
+  // (a row of 128 units fills the 64 banks once: 8 rows, 8 groups of 8 banks; shorter rows share them)
+  auto fz = [](int row) { return TM >= 128 ? 2 * (row % 8) : 2 * ((row / (128 / TM)) % (CPR / 2)); };
 
-  const T* __restrict__ G = static_cast<const T*>(a.gsrc[g]) + (size_t)n * D + dt * TM;
+  const T* __restrict__ G = static_cast<const T*>(a.gsrc[g]) + (size_t)n * a.D + dt * TM;
   const long gld = a.gld[g];
-  const T* __restrict__ H = static_cast<const T*>(a.states_h) + (size_t)n * D + pt * TM;
-  const T* __restrict__ H0 = static_cast<const T*>(a.s0_h) + (size_t)n * D + pt * TM;
+  const T* __restrict__ H = static_cast<const T*>(a.states_h) + (size_t)n * a.D + pt * TM;
+  const T* __restrict__ H0 = static_cast<const T*>(a.s0_h) + (size_t)n * a.D + pt * TM;
+
+  // This wave's load instructions: instruction q = w + NW*i of the stage; the first CPR/2 fill operand A (dG), the
+  // others operand B (h of the step before); instruction j of an operand fills chunk positions 64j .. 64j+63.
+  // A stage whose 32 rows are all valid and hold no first step of a sequence (t = 0, where h comes from the
+  // initial state) is affine in the row: the lane's offset never changes and the stage's base address, uniform,
+  // advances in scalar registers, so a load costs no vector instruction besides itself.  The other stages (one in
+  // T / 32, and the last of a split) compute their addresses per lane.
+  unsigned voff[IPW];  // this lane's byte offset from the stage base of its operand
+  int lrow[IPW], lchunk[IPW];
+#pragma unroll
+  for (int i = 0; i < IPW; ++i) {
+    const int q = w + NW * i, j = q % (CPR / 2);
+    const bool isb = q >= CPR / 2;  // uniform
+    const int P = 64 * j + lane;
+    lrow[i] = P / CPR; lchunk[i] = (P % CPR) ^ fz(lrow[i]);
+    voff[i] = (unsigned)(((size_t)lrow[i] * (isb ? ND : (size_t)gld) + lchunk[i] * 8) * sizeof(T));
+  }
+  auto dma = [&](const T* p, lds_byte* dst) __attribute__((always_inline)) {
+    // (as asm: the compiler, which cannot tell which stage a later LDS read belongs to, would put a wait for
+    // every load in flight in front of the fragment reads; the waits are placed by hand below)
+    asm volatile("s_mov_b32 m0, %1\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, off" ::"v"(p), "s"((unsigned)(size_t)dst) : "memory", "m0");
+  };
+  auto dma_affine = [&](const T* base, unsigned off, lds_byte* dst) __attribute__((always_inline)) {
+    asm volatile("s_mov_b32 m0, %2\n\ts_nop 0\n\tglobal_load_lds_dwordx4 %0, %1" ::"v"(off), "s"(base), "s"((unsigned)(size_t)dst) : "memory", "m0");
+  };
+  long next_seq = (long)(((unsigned)r_begin + (unsigned)Tn - 1u) / (unsigned)Tn) * Tn;  // (uniform) first row at or behind the stage's first that starts a sequence
+  // loads of the stage that begins at row r0 into buffer buf
+  auto issue = [&](long r0, int buf) __attribute__((always_inline)) {
+    while (next_seq < r0) next_seq += Tn;
+    const bool plain = r0 + KB <= r_end && next_seq >= r0 + KB;  // uniform
+    const T* const baseA = G + (size_t)r0 * gld;
+    const T* const baseB = H + (size_t)(r0 - 1) * ND;  // (before the tensor for r0 = 0, whose stage is never plain)
+#pragma unroll
+    for (int i = 0; i < IPW; ++i) {
+      const int q = w + NW * i, j = q % (CPR / 2);
+      const int isb = q >= CPR / 2 ? 1 : 0;  // uniform
+      lds_byte* dst = sm + (buf * 2 + isb) * OPB + j * 1024;
+      if (plain) {
+        dma_affine(isb ? baseB : baseA, voff[i], dst);
+      } else {
+        // rows beyond the end fetch the last valid row (and are zeroed in LDS afterwards)
+        long r = r0 + lrow[i];
+        r = r < r_end ? r : r_end - 1;
+        const T* p;
+        if (isb) {
+          const unsigned b = (unsigned)r / (unsigned)Tn;  // (B * T < 2^31, checked on the host)
+          p = ((unsigned)r - b * (unsigned)Tn > 0) ? H + (size_t)(r - 1) * ND : H0 + (size_t)b * ND;
+        } else {
+          p = G + (size_t)r * gld;
+        }
+        dma(p + lchunk[i] * 8, dst);
+      }
+    }
+  };
 
   f32x4 acc[WT][WT];
 #pragma unroll
@@ -111,69 +176,67 @@ __global__ void __launch_bounds__(256) grad_gemm16_kernel(const GradGemmArgs a) 
 #pragma unroll
     for (int j = 0; j < WT; ++j) acc[i][j] = f32x4{0.f, 0.f, 0.f, 0.f};
 
-  const int rp = tid / TPR, uc = (tid % TPR) * 4;
-  const bool active = rp < 16;
-  uint2 ga[CH][2], hb[CH][2];
-  auto fetch = [&](long r0) __attribute__((always_inline)) {
+  // fragment reads: lane (group q4, s = r16) points at row 4*q4 + s/4 (+16 for the second read), units 4*(s%4)..
+  const int krow = 4 * q4 + (r16 >> 2), sub = r16 & 3;
+  const int f1 = fz(krow);  // (= fz(krow + 16): the second read's address is the first's plus 16 rows)
+  const int ro1 = krow * (TM * 2) + (sub & 1) * 8;
+  const int ga0 = (wm * (TM / WD)) / 8 + (sub >> 1), gb0 = (wn * (TM / WD)) / 8 + (sub >> 1);
+  // byte offsets within a stage buffer (operand B: + OPB), the same for every stage
+  int oa1[WT], ob1[WT];
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-      const long r = r0 + 2 * rp + h;
-      const bool ok = active && r < r_end;
-      const long b = r / Tn, t = r - b * Tn;
-      const T* gp = G + (size_t)r * gld + uc;
-      const T* hp = (t > 0) ? H + (size_t)(r - 1) * ND + uc : H0 + (size_t)b * ND + uc;
+  for (int i = 0; i < WT; ++i) {
+    oa1[i] = ro1 + (((ga0 + 2 * i) ^ f1) << 4);
+    ob1[i] = OPB + ro1 + (((gb0 + 2 * i) ^ f1) << 4);
+  }
+  constexpr int O2 = 16 * TM * 2;
+
+  const int nst = (int)((r_end - r_begin + KB - 1) / KB);
 #pragma unroll
-      for (int c = 0; c < CH; ++c) {
-        ga[c][h] = make_uint2(0u, 0u); hb[c][h] = make_uint2(0u, 0u);
-        if (ok) {
-          ga[c][h] = *reinterpret_cast<const uint2*>(gp + c * 64);
-          hb[c][h] = *reinterpret_cast<const uint2*>(hp + c * 64);
-        }
+  for (int s = 0; s < NS - 1; ++s)
+    if (s < nst) issue(r_begin + (long)s * KB, s);
+  // one stage; `buf` is a compile-time constant (the loop below is unrolled over the NS buffers), so that the
+  // buffer's position goes into the offset field of the LDS reads
+  auto stage = [&](int s, auto BUF) __attribute__((always_inline)) {
+    constexpr int buf = decltype(BUF)::value;
+    // stage s has landed once at most the loads of the NS-2 stages behind it are in flight
+    if (s + NS - 2 < nst) asm volatile("s_waitcnt vmcnt(%0)" ::"n"(IPW * (NS - 2)) : "memory");
+    else asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    // every wave's part of stage s is there; every wave is done with the buffer of stage s - 1
+    // (a barrier that orders LDS only: __syncthreads() would wait for the loads in flight)
+    asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
+    if (s + NS - 1 < nst) issue(r_begin + (long)(s + NS - 1) * KB, (buf + NS - 1) % NS);
+    const long nvalid = r_end - (r_begin + (long)s * KB);
+    if (nvalid < KB) {  // (uniform; the last stage of a split only) rows beyond the end count as zero
+      for (int P = (int)nvalid * CPR + tid; P < KB * CPR; P += NT) {
+        *(__attribute__((address_space(3))) u32x4*)(sm + (buf * 2) * OPB + P * 16) = u32x4{0u, 0u, 0u, 0u};
+        *(__attribute__((address_space(3))) u32x4*)(sm + (buf * 2 + 1) * OPB + P * 16) = u32x4{0u, 0u, 0u, 0u};
       }
+      asm volatile("s_waitcnt lgkmcnt(0)\n\ts_barrier" ::: "memory");
     }
-  };
-  auto stage = [&](int buf) __attribute__((always_inline)) {
-    if (!active) return;
-#pragma unroll
-    for (int c = 0; c < CH; ++c) {
-      // element e of row 2rp in the low half, of row 2rp+1 in the high half
-      unsigned (*sa)[GemmStage16<TM>::LD] = &sm.a[buf][uc + c * 64];
-      unsigned (*sb)[GemmStage16<TM>::LD] = &sm.b[buf][uc + c * 64];
-      sa[0][rp] = (ga[c][0].x & 0xffffu) | (ga[c][1].x << 16);
-      sa[1][rp] = (ga[c][0].x >> 16) | (ga[c][1].x & 0xffff0000u);
-      sa[2][rp] = (ga[c][0].y & 0xffffu) | (ga[c][1].y << 16);
-      sa[3][rp] = (ga[c][0].y >> 16) | (ga[c][1].y & 0xffff0000u);
-      sb[0][rp] = (hb[c][0].x & 0xffffu) | (hb[c][1].x << 16);
-      sb[1][rp] = (hb[c][0].x >> 16) | (hb[c][1].x & 0xffff0000u);
-      sb[2][rp] = (hb[c][0].y & 0xffffu) | (hb[c][1].y << 16);
-      sb[3][rp] = (hb[c][0].y >> 16) | (hb[c][1].y & 0xffff0000u);
-    }
-  };
-  fetch(r_begin);
-  stage(0);
-  __syncthreads();
-  int cur = 0;
-  for (long r0 = r_begin; r0 < r_end; r0 += 32) {
-    const bool more = r0 + 32 < r_end;
-    if (more) fetch(r0 + 32);
+    lds_byte* const sb = sm + (buf * 2) * OPB;
     typename X::Frag af[WT], bfr[WT];
 #pragma unroll
     for (int i = 0; i < WT; ++i) {
-      const unsigned* pa = &sm.a[cur][wm * (TM / 2) + i * 16 + r16][q4 * 4];
-      const unsigned* pb = &sm.b[cur][wn * (TM / 2) + i * 16 + r16][q4 * 4];
-      const u32x4 va = {pa[0], pa[1], pa[2], pa[3]}, vb = {pb[0], pb[1], pb[2], pb[3]};
-      af[i] = __builtin_bit_cast(typename X::Frag, va);
-      bfr[i] = __builtin_bit_cast(typename X::Frag, vb);
+      const s16x4 a1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(sb + oa1[i]));
+      const s16x4 a2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(sb + oa1[i] + O2));
+      const s16x4 b1 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(sb + ob1[i]));
+      const s16x4 b2 = __builtin_amdgcn_ds_read_tr16_b64_v4i16((lds_s16x4*)(sb + ob1[i] + O2));
+      af[i] = __builtin_bit_cast(typename X::Frag, __builtin_shufflevector(a1, a2, 0, 1, 2, 3, 4, 5, 6, 7));
+      bfr[i] = __builtin_bit_cast(typename X::Frag, __builtin_shufflevector(b1, b2, 0, 1, 2, 3, 4, 5, 6, 7));
     }
+    __builtin_amdgcn_sched_barrier(0);  // all reads in front of the first MFMA: their latency is paid once
 #pragma unroll
     for (int i = 0; i < WT; ++i)
 #pragma unroll
       for (int j = 0; j < WT; ++j) acc[i][j] = X::mfma(af[i], bfr[j], acc[i][j]);
-    if (more) stage(cur ^ 1);
-    __syncthreads();  // the other buffer is complete, and this one has been read by every wave
-    cur ^= 1;
+  };
+  for (int s = 0; s < nst; s += NS) {
+    stage(s, std::integral_constant<int, 0>{});
+    if (s + 1 < nst) stage(s + 1, std::integral_constant<int, 1 % NS>{});
+    if (NS > 2 && s + 2 < nst) stage(s + 2, std::integral_constant<int, 2 % NS>{});
+    static_assert(NS <= 3, "the stage loop is written out for up to 3 buffers");
   }
-  gemm_store_partial<WT>(a, TM, g, n, split, dt, pt, wm, wn, r16, q4, acc);
+  gemm_store_partial<WT>(a, TM, g, n, split, dt, pt, wm, wn, r16, q4, acc, TM / WD);
 }
 
 // fp32 storage: the MFMA (16x16x4) takes the operands as they are stored, [row][unit]
@@ -188,6 +251,7 @@ __global__ void __launch_bounds__(256) grad_gemm32_kernel(const GradGemmArgs a) 
   typedef ST<T> X;
   constexpr int EV = TM / 8;           // elements per thread per staged row
   constexpr int WT = TM / 32;          // MFMA tiles per wave per dimension
+  constexpr int WD = 2;                // 2 x 2 waves
   __shared__ __attribute__((aligned(16))) GemmStage32<TM> sm;
 
   int g, dt, pt;
@@ -249,24 +313,27 @@ __global__ void __launch_bounds__(256) grad_gemm32_kernel(const GradGemmArgs a) 
         for (int j = 0; j < WT; ++j) acc[i][j] = X::mfma(af[i], bfr[j], acc[i][j]);
     }
   }
-  gemm_store_partial<WT>(a, TM, g, n, split, dt, pt, wm, wn, r16, q4, acc);
+  gemm_store_partial<WT>(a, TM, g, n, split, dt, pt, wm, wn, r16, q4, acc, TM / WD);
 }
 
-// side of the square workgroup tile: the largest of 128 (16-bit types only), 64, 32 that divides D
+// side of the square workgroup tile: the largest of 256, 128 (16-bit types only), 64, 32 that divides D
 static int gemm_tile_side(int dtype, int D) {
+  if (dtype != FRNN_F32 && D % 256 == 0) return 256;
   if (dtype != FRNN_F32 && D % 128 == 0) return 128;
   return (D % 64 == 0) ? 64 : 32;
 }
 
-// split-K factor.  A workgroup waits for its global loads once per stage, so the kernel lives on many
-// workgroups per compute unit (measured: time falls with the split count until about 8 per unit);
-// bounded by 4 stages per split and by 64 MiB of partial sums.
+// split-K factor.  Tiles of up to 128 units (workgroups of 4 waves): a workgroup waits for its loads once per stage,
+// so the kernel lives on many workgroups per compute unit (measured: time falls with the split count until about 8
+// per unit).  Tiles of 256 units (16 waves, 96 KB of LDS: one workgroup per compute unit, three stages in flight):
+// one workgroup per compute unit, all in one round (measured at D = 256, 768, 1024: best at 190-260 workgroups).
+// Bounded by 4 stages per split and by 64 MiB of partial sums.
 int grad_gemm_splits(int dtype, int B, int T, int N, int D, int GR) {
   const int TM = gemm_tile_side(dtype, D);
   const long tiles = (long)GR * (D / TM) * (D / TM) * N;
   const long chunks = ((long)B * T + 31) / 32;
   const long out_bytes = (long)GR * N * D * D * 4;
-  long s = (2048 + tiles - 1) / tiles;
+  long s = TM == 256 ? (256 + tiles / 2) / tiles : (2048 + tiles - 1) / tiles;
   if (s > 64) s = 64;
   if (s > (64l << 20) / out_bytes) s = (64l << 20) / out_bytes;
   if (s > chunks / 4) s = chunks / 4;
@@ -276,16 +343,24 @@ int grad_gemm_splits(int dtype, int B, int T, int N, int D, int GR) {
   return (int)s;
 }
 
-template <typename T, int TM>
+template <typename T, int TM, int WD>
 static int launch_gemm16(const GradGemmArgs& a, dim3 grid, hipStream_t st) {
-  const size_t lds = sizeof(GemmStage16<TM>);
+  constexpr int NS = 3;
+  const size_t lds = (size_t)NS * 2 * 32 * TM * 2;
   if (lds > 65536) {
-    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&grad_gemm16_kernel<T, TM>),
+    const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void*>(&grad_gemm16_kernel<T, TM, WD, NS>),
                                              hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
     if (e != hipSuccess) return (int)e;
   }
-  hipLaunchKernelGGL((grad_gemm16_kernel<T, TM>), grid, dim3(256), lds, st, a);
+  hipLaunchKernelGGL((grad_gemm16_kernel<T, TM, WD, NS>), grid, dim3(64 * WD * WD), lds, st, a);
   return (int)hipGetLastError();
+}
+template <typename T>
+static int launch_gemm16_any(int TM, const GradGemmArgs& a, dim3 grid, hipStream_t st) {
+  if (TM == 256) return launch_gemm16<T, 256, 4>(a, grid, st);
+  if (TM == 128) return launch_gemm16<T, 128, 2>(a, grid, st);
+  if (TM == 64) return launch_gemm16<T, 64, 2>(a, grid, st);
+  return launch_gemm16<T, 32, 2>(a, grid, st);
 }
 
 int launch_grad_gemm(int dtype, GradGemmArgs a, int splits, hipStream_t st) {
@@ -293,15 +368,8 @@ int launch_grad_gemm(int dtype, GradGemmArgs a, int splits, hipStream_t st) {
   const long chunks = ((long)a.B * a.T + 31) / 32;
   a.rows_per_split = (int)(((chunks + splits - 1) / splits) * 32);
   const dim3 grid(a.GR * (a.D / TM) * (a.D / TM), a.N, splits);
-  if (dtype == FRNN_BF16) {
-    if (TM == 128) return launch_gemm16<bf16_t, 128>(a, grid, st);
-    if (TM == 64) return launch_gemm16<bf16_t, 64>(a, grid, st);
-    return launch_gemm16<bf16_t, 32>(a, grid, st);
-  } else if (dtype == FRNN_F16) {
-    if (TM == 128) return launch_gemm16<half_t, 128>(a, grid, st);
-    if (TM == 64) return launch_gemm16<half_t, 64>(a, grid, st);
-    return launch_gemm16<half_t, 32>(a, grid, st);
-  }
+  if (dtype == FRNN_BF16) return launch_gemm16_any<bf16_t>(TM, a, grid, st);
+  if (dtype == FRNN_F16) return launch_gemm16_any<half_t>(TM, a, grid, st);
   if (TM == 64) hipLaunchKernelGGL((grad_gemm32_kernel<64>), grid, dim3(256), 0, st, a);
   else hipLaunchKernelGGL((grad_gemm32_kernel<32>), grid, dim3(256), 0, st, a);
   return (int)hipGetLastError();
