@@ -379,6 +379,39 @@ FRNN_SEL_DEFINE(unsigned, "global_store_dword")
 FRNN_SEL_DEFINE(u64, "global_store_dwordx2")
 #undef FRNN_SEL_DEFINE
 
+// The same for 4 destinations at once (4 uniform bases, one lane offset, N words each): the two switches of the lane
+// mask cost ~40 cycles per block, which adds up for a wave that sends to 31 other workgroups per step.
+#define FRNN_D(op, sc, d, e) op " %[o], %[v" #d #e "], %[b" #d "] offset:%[k" #e "] " sc "\n\t"
+#define FRNN_D1(op, sc, d) FRNN_D(op, sc, d, 0)
+#define FRNN_D2(op, sc, d) FRNN_D(op, sc, d, 0) FRNN_D(op, sc, d, 1)
+#define FRNN_D4(op, sc, d) FRNN_D(op, sc, d, 0) FRNN_D(op, sc, d, 1) FRNN_D(op, sc, d, 2) FRNN_D(op, sc, d, 3)
+#define FRNN_ALL(DN, op, sc) DN(op, sc, 0) DN(op, sc, 1) DN(op, sc, 2) DN(op, sc, 3)
+#define FRNN_VROW(d) [v##d##0] "v"(v[d][0])
+#define FRNN_VROW2(d) FRNN_VROW(d), [v##d##1] "v"(v[d][N > 1 ? 1 : 0])
+#define FRNN_VROW4(d) FRNN_VROW2(d), [v##d##2] "v"(v[d][N > 2 ? 2 : 0]), [v##d##3] "v"(v[d][N > 3 ? 3 : 0])
+#define FRNN_SEL4_DEFINE(W, op)                                                                                  \
+  template <int N, int STRIDE> __device__ __forceinline__ void ll_store_sel4(const void* const (&base)[4], unsigned voff, const W (&v)[4][N], u64 near) { \
+    static_assert(N == 1 || N == 2 || N == 4, "1, 2 or 4 words per lane and destination");                       \
+    static_assert(3 * STRIDE < 4096, "immediate offsets");                                                      \
+    u64 tmp;                                                                                                     \
+    if constexpr (N == 1)                                                                                        \
+      asm volatile(FRNN_SEL_HEAD FRNN_ALL(FRNN_D1, op, "sc0") FRNN_SEL_MID FRNN_ALL(FRNN_D1, op, "sc1") FRNN_SEL_TAIL \
+                   : [tmp] "=&s"(tmp) : [o] "v"(voff), [b0] "s"(base[0]), [b1] "s"(base[1]), [b2] "s"(base[2]), [b3] "s"(base[3]), \
+                     FRNN_VROW(0), FRNN_VROW(1), FRNN_VROW(2), FRNN_VROW(3), [k0] "n"(0), [nr] "s"(near) : "scc"); \
+    else if constexpr (N == 2)                                                                                   \
+      asm volatile(FRNN_SEL_HEAD FRNN_ALL(FRNN_D2, op, "sc0") FRNN_SEL_MID FRNN_ALL(FRNN_D2, op, "sc1") FRNN_SEL_TAIL \
+                   : [tmp] "=&s"(tmp) : [o] "v"(voff), [b0] "s"(base[0]), [b1] "s"(base[1]), [b2] "s"(base[2]), [b3] "s"(base[3]), \
+                     FRNN_VROW2(0), FRNN_VROW2(1), FRNN_VROW2(2), FRNN_VROW2(3), [k0] "n"(0), [k1] "n"(STRIDE), [nr] "s"(near) : "scc"); \
+    else                                                                                                         \
+      asm volatile(FRNN_SEL_HEAD FRNN_ALL(FRNN_D4, op, "sc0") FRNN_SEL_MID FRNN_ALL(FRNN_D4, op, "sc1") FRNN_SEL_TAIL \
+                   : [tmp] "=&s"(tmp) : [o] "v"(voff), [b0] "s"(base[0]), [b1] "s"(base[1]), [b2] "s"(base[2]), [b3] "s"(base[3]), \
+                     FRNN_VROW4(0), FRNN_VROW4(1), FRNN_VROW4(2), FRNN_VROW4(3),                                   \
+                     [k0] "n"(0), [k1] "n"(STRIDE), [k2] "n"(2 * STRIDE), [k3] "n"(3 * STRIDE), [nr] "s"(near) : "scc"); \
+  }
+FRNN_SEL4_DEFINE(unsigned, "global_store_dword")
+FRNN_SEL4_DEFINE(u64, "global_store_dwordx2")
+#undef FRNN_SEL4_DEFINE
+
 // largest divisor of n that is <= 8: k-steps whose LDS fragments are fetched together
 constexpr int chunk_of(int n) { for (int c = 8; c > 1; --c) if (n % c == 0) return c; return 1; }
 

@@ -617,6 +617,24 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     if constexpr (GROUPED) {
       const unsigned sslot = ((unsigned)(bvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
       auto send_group = [&](int r0, int nr, f32x4 (&ag)[RI][UTW]) __attribute__((always_inline)) {
+        if (nr == RI) {  // (compile-time at every call site) four destinations with one switch of the store form
+#pragma unroll
+          for (int u = 0; u < UTW; ++u) {
+            const void* base[RI];
+            IW wv[RI][E];
+#pragma unroll
+            for (int rr = 0; rr < RI; ++rr) {
+              const int x = (slice + r0 + rr) % KW;
+              base[rr] = inbox + (size_t)(((x * WAVES + w_u) * UTW + u) * KW + slice) * 256;
+              float part[E];
+              own_elems<TR>(ag[rr][u], part);
+#pragma unroll
+              for (int e = 0; e < E; ++e) wv[rr][e] = part_pack((PT*)0, part[e], t);
+            }
+            ll_store_sel4<E, 64 * (int)sizeof(IW)>(base, sslot, wv, near_m);
+          }
+          return;
+        }
 #pragma unroll
         for (int rr = 0; rr < RI; ++rr) {
           if (rr >= nr) continue;
