@@ -642,9 +642,8 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   // measured best, as in the forward call (exchange stores kept in the XCD's L2): the gated cells 0-2 units at every
   // head dim from 192 to 1024 (their dWx stores are issued between the send and the first probe, which is part of
   // their delay), elman D = 512 4, D = 1024 8; recompute mode sends its first probe behind the LDS reads of the
-  // rebuild: best without a delay, 2 units for the slstm
-  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", o.rc ? (fx == FRNN_SLSTM ? 2 : 0)
-                                                : c.GR == 1 ? (p.kw > 4 ? 8 : 4) : 2);
+  // rebuild: best without a delay for every cell
+  a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", o.rc ? 0 : c.GR == 1 ? (p.kw > 4 ? 8 : 4) : 2);
   a.g_clip = o.g_clip; a.cut = o.cut;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
