@@ -133,6 +133,40 @@ def run_gpu(w, backend, steps, warmup, device, recompute=False):
     return (t1 - t0) * 1e3 / steps, kern
 
 
+def run_with_linear(w, backend, steps, warmup, device):
+    """The reference's "withlinear" benchmark variants (speed_experiments/kernel_speed_benchmark.py:387-407): the input
+    projection Wx = Linear(x) in front of the recurrence, forward and backward through both.  The kernels read the
+    [B, T, G, N, D] tensor that the Linear writes as it is (a view of its [B, T, G*N*D] output): no permuted copy lies
+    between the two, which is the whole of the fusion that the reference measures.  Returns ms per step."""
+    import torch
+    from flashrnn_amd import FlashRNNConfig, flashrnn
+
+    _, dev = make_gpu_inputs(w, device)
+    B, T, N, D = w["B"], w["T"], w["N"], w["D"]
+    Gw = dev["Wx"].shape[2]
+    F = N * D
+    g = torch.Generator(device="cpu").manual_seed(w["seed"] + 7)
+    x = torch.randn((B, T, F), generator=g).to(device, dev["Wx"].dtype).requires_grad_(True)
+    W = (torch.randn((Gw * N * D, F), generator=g) / F ** 0.5).to(device, dev["Wx"].dtype).requires_grad_(True)
+    rest = [dev[k].requires_grad_(w["bwd"]) for k in ("R", "b", "states")]
+    cfg = FlashRNNConfig(backend=backend, function=w["function"], dtype=w["dtype"], head_dim=D, num_heads=N, batch_size=B)
+
+    def step():
+        Wx = torch.nn.functional.linear(x, W).view(B, T, Gw, N, D)
+        out, _ = flashrnn(Wx, *rest, config=cfg)
+        if w["bwd"]:
+            torch.autograd.grad(out, [x, W] + rest, grad_outputs=dev["dstates"])
+
+    for _ in range(warmup):
+        step()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        step()
+    torch.cuda.synchronize()
+    return (time.perf_counter() - t0) * 1e3 / steps
+
+
 def run_cpu_baseline(w, budget_s=20.0):
     """The CPU oracle (a port of the reference's vanilla backend) on the host cores, fp32, on a bounded
     sample: the first T_cpu time steps of the workload, T_cpu chosen from a 32-step probe so that one
@@ -272,6 +306,8 @@ def main():
     ap.add_argument("--backend", default=None, choices=["hip_fused", "hip"])
     ap.add_argument("--recompute", action="store_true",
                     help="hip_fused in recompute mode: no gate cache, the backward pass rebuilds the gates")
+    ap.add_argument("--with-linear", action="store_true",
+                    help="also time the step with the input projection Wx = Linear(x) in front (hidden size N*D)")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-alt", action="store_true", help="skip the other-backend comparison leg")
     ap.add_argument("--copy-calibration", action="store_true",
@@ -371,6 +407,10 @@ def main():
                                     "speedup_of_" + backend: ms_o / ms}
         except ValueError as e:  # no kernel of the other backend for this head dim
             out["other_backend"] = {"backend": other, "error": str(e)}
+    if args.with_linear:
+        ms_l = run_with_linear(w, backend, args.steps, args.warmup, device)
+        out["with_linear"] = {"ms_per_step": ms_l, "linear_ms": ms_l - ms,
+                              "note": "x [B,T,N*D] -> torch.nn.functional.linear -> view [B,T,G,N,D] -> flashrnn(); no copy in between"}
     if not args.no_cpu:
         out["cpu_baseline"] = run_cpu_baseline(w)
     print(json.dumps(out), flush=True)
