@@ -93,11 +93,16 @@ size_t frnn_fused_cache_bytes(int function, int dtype, int B, int T, int N, int 
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward);
 
 /* Concurrency: when a head spans several workgroups (frnn_fused_plan: wgs_per_head > 1) they wait for
- * each other inside the kernel and a launch may fill the device, so run one such call at a time per
- * device (calls on one stream are; the reference's cooperative launch has the same property), or set
- * FRNN_COOPERATIVE=1 in the environment: the kernels are then launched as cooperative kernels, which
- * the runtime runs one at a time (about 15 us more per launch).  Calls that overlap anyway cannot
- * hang: every wait is bounded and a wait that runs out is reported in the status word. */
+ * each other inside the kernel and must all be resident.  Launches of such kernels on different streams of
+ * one device are ordered behind each other by the library (an event wait on the device, nothing blocks on
+ * the host; the reference's cooperative launch gives the same guarantee, fused/flashrnn_fused_forward.cu:
+ * 893-911); FRNN_COOPERATIVE=1 in the environment launches them as cooperative kernels instead (about 15 us
+ * more per launch).  Kernels of other processes are not seen: every wait is bounded, and a wait that runs out
+ * is reported in the status word instead of hanging.
+ * The workgroups of a head exchange h (forward) and partial sums (backward) through tagged words in the
+ * workspace.  A launch places them on one XCD and the kernels check that at their start; the exchange stores
+ * then stay in that XCD's L2.  Where the check fails, or with FRNN_AGENT_STORES=1, they are written through to
+ * memory (slower, same results). */
 
 /* Forward over the whole sequence.  Replaces FlashRNNFuncFused::forward (fused/flashrnn.cc:68-144)
  * + ForwardPass::Run (fused/flashrnn_fused_forward.cu:772-975).
