@@ -411,6 +411,21 @@ FRNN_SEL_DEFINE(u64, "global_store_dwordx2")
 FRNN_SEL4_DEFINE(unsigned, "global_store_dword")
 FRNN_SEL4_DEFINE(u64, "global_store_dwordx2")
 #undef FRNN_SEL4_DEFINE
+#undef FRNN_VROW4
+#undef FRNN_VROW2
+#undef FRNN_VROW
+#undef FRNN_ALL
+#undef FRNN_D4
+#undef FRNN_D2
+#undef FRNN_D1
+#undef FRNN_D
+#undef FRNN_ST3
+#undef FRNN_ST2
+#undef FRNN_ST1
+#undef FRNN_ST0
+#undef FRNN_SEL_TAIL
+#undef FRNN_SEL_MID
+#undef FRNN_SEL_HEAD
 
 // largest divisor of n that is <= 8: k-steps whose LDS fragments are fetched together
 constexpr int chunk_of(int n) { for (int c = 8; c > 1; --c) if (n % c == 0) return c; return 1; }
