@@ -276,9 +276,15 @@ __device__ __forceinline__ bool poll_pairs(rsrc_t slot, unsigned soff, const int
         __hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != STATUS_OK) return true;
   }
 }
+// Word `off` of a vector of `tot` words in an LDS copy that starts `rot` words into the vector and wraps around
+// (tot = 0: no rotation)
+__device__ __forceinline__ unsigned lds_rotated(int off, int rot, int tot) {
+  const unsigned d = (unsigned)(off - rot);
+  return tot ? min(d, d + (unsigned)tot) : (unsigned)off;  // (off < rot: d wraps, d + tot is the index)
+}
 template <typename T, int NP>
 __device__ __forceinline__ bool ll_gather_pairs(rsrc_t slots, unsigned soff, const int* q, int t, T* lds_dst,
-                                                int* status, int spin_limit, int first_delay) {
+                                                int* status, int spin_limit, int first_delay, int rot = 0, int tot = 0) {
   constexpr int CH = NP < 16 ? NP : 16;  // words polled together
   static_assert(NP % CH == 0 && CH % 2 == 0, "poll list must split into whole chunks of pairs");
   bool fail = false;
@@ -293,7 +299,7 @@ __device__ __forceinline__ bool ll_gather_pairs(rsrc_t slots, unsigned soff, con
 #pragma unroll
       for (int i = 0; i < CH; i += 2)
         if (need[i])
-          *reinterpret_cast<uint2*>(reinterpret_cast<unsigned*>(lds_dst) + off[i]) =
+          *reinterpret_cast<uint2*>(reinterpret_cast<unsigned*>(lds_dst) + lds_rotated(off[i], rot, tot)) =
               make_uint2(ll_payload((T*)0, v[i]), ll_payload((T*)0, v[i + 1]));
     }
   }
@@ -304,7 +310,7 @@ __device__ __forceinline__ bool ll_gather_pairs(rsrc_t slots, unsigned soff, con
 // C4: the LDS vector is kept as [k][4 rows] (the fp32 4-row tiles, see lds_index4) instead of fragment order
 template <typename T, int NP, bool C4 = false>
 __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, T* lds_dst,
-                                          int* status, int spin_limit, int first_delay) {
+                                          int* status, int spin_limit, int first_delay, int rot = 0, int tot = 0) {
   constexpr int CH = NP < 16 ? NP : 16;  // words polled together
   static_assert(NP % CH == 0, "poll list must split into whole chunks");
   bool fail = false;
@@ -317,7 +323,7 @@ __device__ __forceinline__ bool ll_gather(const u64* slot, const int* q, int t, 
     if (!fail) {
 #pragma unroll
       for (int i = 0; i < CH; ++i)
-        if (need[i]) reinterpret_cast<unsigned*>(lds_dst)[C4 ? lds_index4_of_word(off[i]) : off[i]] = ll_payload((T*)0, v[i]);
+        if (need[i]) reinterpret_cast<unsigned*>(lds_dst)[C4 ? lds_index4_of_word(off[i]) : lds_rotated(off[i], rot, tot)] = ll_payload((T*)0, v[i]);
     }
   }
   return fail;

@@ -103,6 +103,19 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   // instruction per k: D instructions of 8 cycles per tile and step instead of G_r * D / 4 of 32.
   constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
   constexpr bool M44 = sizeof(T) == 4 && TR == 4 && GR >= 3 && RLK == 0 && D <= 384;  // (the whole operand, D registers per tile, in registers)
+  // Own slice first: of the h_(t-1) a step multiplies with, the workgroup's own D / KW units are in LDS as soon as
+  // its waves have finished step t-1; the k-steps over them run before the wait for the other workgroups' slices
+  // (behind one more LDS barrier) and leave the critical path.  Each workgroup keeps R and h rotated along k so
+  // that its own slice comes first: k-step ks of the loops below is k-step (ks + slice * KSO) % KS of the head.
+#ifdef FRNN_NO_OWN_FIRST
+  constexpr bool OWN_FIRST = false;
+#else
+  // (not for the fp32 kernels whose operand alone takes 256 registers and whose 16-row tiles keep 4 elements per
+  // lane: with the two-part product they spill)
+  constexpr bool OWN_FIRST = KW > 1 && KW <= 8 && !M44 && RLK == 0 && (D / KW) % X::KM == 0 &&
+                             !(sizeof(T) == 4 && UTW * GR * KS >= 256 && TR == 16);
+#endif
+  constexpr int KSO = OWN_FIRST ? (D / KW) / X::KM : 0;
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
   __shared__ int dead_flag, near_word;
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
@@ -146,6 +159,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int FRAG_REGS = (int)sizeof(Frag) / 4, RF_REGS = UTW * GR * KSR * FRAG_REGS;
   constexpr int PIN_REGS = RF_REGS > 160 ? (RF_REGS < 232 ? RF_REGS : 232) : 0;  // (160 registers, D = 320: measured no gain)
   Frag rf[UTW][GR][KSR];
+  const int rot_ks = OWN_FIRST ? slice * KSO : 0, rot_u = OWN_FIRST ? slice * (D / KW) : 0;  // rotation in k-steps, in units
   Frag* const rl = rlds + (size_t)w * RLK * UTW * GR * 64 + lane;
   // 4x4x1 form: lane 4*blk + j holds row (gate j, unit blk of the tile) of R, one register per k
   float rb[M44 ? UTW : 1][M44 ? D : 1];
@@ -169,7 +183,8 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       const T* row = R + ((size_t)(g * N + n) * D + ub[u] + r16) * D;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
-        const Frag f = load_frag<T>(row, ks, q4);
+        const int kh = OWN_FIRST ? (ks + rot_ks < KS ? ks + rot_ks : ks + rot_ks - KS) : ks;  // k-step of the head
+        const Frag f = load_frag<T>(row, kh, q4);
         if (ks < KSR) {
           rf[u][g][ks < KSR ? ks : 0] = f;
 #ifndef FRNN_NO_AGPR_PIN
@@ -231,9 +246,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         if (!rv) reinterpret_cast<float*>(hbuf[1])[lds_index4(row, k0 + i)] = v[i];
       }
     } else {
-      lds_write<4>(hbuf[0], row, k0, v);
+      const int kl = OWN_FIRST ? (k0 >= rot_u ? k0 - rot_u : k0 - rot_u + D) : k0;
+      lds_write<4>(hbuf[0], row, kl, v);
       if (KW > 1 || TR < 16) {  // rows that are never rewritten must be finite in both buffers
-        if (!rv) lds_write<4>(hbuf[1], row, k0, v);
+        if (!rv) lds_write<4>(hbuf[1], row, kl, v);
       }
     }
   }
@@ -243,6 +259,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   // per group: slot 0, slot 1, and a third area that swallows the stores of padded lanes
   u64* const llbase = a.ll + (size_t)(a.step ? 0 : grp) * 3 * LLW;
   const rsrc_t rLL = make_rsrc(llbase, (size_t)2 * LLW * 8);  // the two slots that are read
+  const int rot_w = rot_u * 16 / X::EPW;  // the rotation in words of the LDS vector (an exchange word holds 32 bits of it)
 
   // Wx is fetched PD steps ahead into a ring of PD + 1 register sets.  A head that exchanges
   // nothing (KW = 1) has steps shorter than a fetch from HBM takes (D = 64: 1100 cycles against
@@ -283,11 +300,35 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   auto step = [&](const int t, Dw<ND_> (&wc)[UTW][GW], Dw<ND_> (&wn)[UTW][GW]) __attribute__((always_inline)) {
     const int cur = t & 1;
     FRNN_STAMP(c0);
+    // NACC accumulators per (tile, gate), used round robin over the k-steps, so that at least ~4
+    // independent MFMA chains are in flight (a dependent MFMA waits ~3x longer than an independent one)
+    constexpr int NACC_ = UTW * GR >= 3 ? 1 : (UTW * GR == 2 ? 2 : 4);
+    constexpr int NACC = NACC_ < KS ? NACC_ : KS;
+    f32x4 accp[M44 ? 1 : NACC][UTW][GR];
+    if constexpr (OWN_FIRST) {
+      if (t > 0) lds_barrier();  // the own slice of h_(t-1), written by the gate math of every wave
+      const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane;
+      Frag ho[KSO];
+#pragma unroll
+      for (int k = 0; k < KSO; ++k) ho[k] = hf[k * 64];
+      __builtin_amdgcn_sched_barrier(0);
+#pragma unroll
+      for (int k = 0; k < KSO; ++k) {
+#pragma unroll
+        for (int u = 0; u < UTW; ++u)
+#pragma unroll
+          for (int g = 0; g < GR; ++g)
+            accp[k % NACC][u][g] = X::mfma(rf[u][g][k], ho[k],
+                                           k < NACC ? ((BIAS_C && k == 0) ? biasc[u][g] : f32x4{0.f, 0.f, 0.f, 0.f}) : accp[k % NACC][u][g]);
+        if (k % NACC == NACC - 1) __builtin_amdgcn_sched_barrier(0);
+      }
+      __builtin_amdgcn_sched_barrier(0);
+    }
     if (t > 0) {
       if (KW > 1) {
         bool fail;
-        if constexpr (PAIRS) fail = ll_gather_pairs<T, NP>(rLL, (unsigned)((t - 1) & 1) * LLW * 8u, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
-        else fail = ll_gather<T, NP, M44>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay);
+        if constexpr (PAIRS) fail = ll_gather_pairs<T, NP>(rLL, (unsigned)((t - 1) & 1) * LLW * 8u, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay, rot_w, OWN_FIRST ? LLW : 0);
+        else fail = ll_gather<T, NP, M44>(llbase + (size_t)((t - 1) & 1) * LLW, qpoll, t - 1, hbuf[cur], a.status, a.spin_limit, a.poll_delay, rot_w, OWN_FIRST ? LLW : 0);
         if (barrier_or(fail, &dead_flag)) { dead = true; return; }
       } else {
         lds_barrier();
@@ -297,8 +338,6 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     if constexpr (!WX_LATE) load_wx(wn, min(t + PD, Tn - 1));
 
     // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once
-    // NACC accumulators per (tile, gate), used round robin over the k-steps, so that at least ~4
-    // independent MFMA chains are in flight (a dependent MFMA waits ~3x longer than an independent one)
     f32x4 acc[UTW][GR];
     float ry44[M44 ? UTW : 1][4];  // 4x4x1 form: the lane's element, gates 0..3
     if constexpr (M44) {
@@ -323,12 +362,9 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       }
     }
     if constexpr (!M44) {
-    constexpr int NACC_ = UTW * GR >= 3 ? 1 : (UTW * GR == 2 ? 2 : 4);
-    constexpr int NACC = NACC_ < KS ? NACC_ : KS;
-    f32x4 accp[NACC][UTW][GR];
-    const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane;
-    constexpr int KC = chunk_of(KS);
-    static_assert(KS % KC == 0, "k-steps must split into whole chunks");
+    const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane + KSO * 64;  // (the own k-steps are done)
+    constexpr int KC = chunk_of(KS - KSO);
+    static_assert((KS - KSO) % KC == 0, "k-steps must split into whole chunks");
     Frag hq[2][KC];
 #pragma unroll
     for (int k = 0; k < KC; ++k) hq[0][k] = hf[k * 64];
@@ -342,15 +378,15 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
     __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-    for (int kc = 0; kc < KS / KC; ++kc) {
-      if (kc + 1 < KS / KC) {
+    for (int kc = 0; kc < (KS - KSO) / KC; ++kc) {
+      if (kc + 1 < (KS - KSO) / KC) {
 #pragma unroll
         for (int k = 0; k < KC; ++k) hq[(kc + 1) & 1][k] = hf[((kc + 1) * KC + k) * 64];
         __builtin_amdgcn_sched_barrier(0);
       }
 #pragma unroll
       for (int k = 0; k < KC; ++k) {
-        const int ks = kc * KC + k, j = ks % NACC;
+        const int ks = KSO + kc * KC + k, j = ks % NACC;
         // fragments kept in LDS: those of the next k-step are requested before this one's MFMAs
         Frag la[UTW][GR];
         if constexpr (RLK > 0) {
@@ -435,7 +471,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
       // (the own slice goes straight to the LDS buffer of the next step: the workgroup does not poll it)
       if (KW > 1) ll_write<E>((T*)0, llbase, (unsigned)(bvalid ? (t & 1) : 2) * (unsigned)(LLW * 8), brow, ub[u] + esub, so[0], t, near_m);
       if constexpr (M44) reinterpret_cast<float*>(hbuf[cur ^ 1])[lds_index4(brow, ub[u] + esub)] = so[0][0];
-      else lds_write<E>(hbuf[cur ^ 1], brow, ub[u] + esub, so[0]);
+      else lds_write<E>(hbuf[cur ^ 1], brow, ub[u] - rot_u + esub, so[0]);
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
