@@ -72,12 +72,15 @@ struct Plan {
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
   X(256, 0, 16, 1, 1, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 8, 1, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 8, 1, 4, 16) X(640, 0, 4, 1, 10, 16) \
   X(768, 0, 8, 1, 6, 16) X(1024, 0, 8, 1, 8, 4)
+// (fp32: a 16-unit tile costs D / 4 MFMAs of 32 cycles per step whatever the batch tile, so heads from D = 128 on are
+// spread over D / 64 workgroups with one tile per wave: D = 256 as one workgroup of 4 waves x 4 tiles took 8.0 ms
+// per 1024 steps forward + backward, as 4 workgroups it takes 2.7)
 #define FRNN_PLANS_GR1_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 16) \
-  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 2, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 2, 4, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 8)
 #define FRNN_BWD_PLANS_GR1_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 2, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 4, 3, 1, 16) X(256, 0, 4, 4, 1, 8) \
-  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 2, 3, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 2, 4, 8) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 16) X(1024, 0, 4, 1, 16, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 16) X(1024, 0, 4, 1, 16, 8)
 
 // ---- reverse scan in recompute mode (no gate cache): R and R^T are both resident, so only the head
 // dims whose two operands fit the registers beside the working set; same tilings as above where those
