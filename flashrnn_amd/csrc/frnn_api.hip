@@ -162,6 +162,20 @@ static int device_cus() {
 // of the device: with KW = 12 an XCD of 32 compute units holds 2 groups, the device 16, not 256 / 12 = 21.
 static int groups_per_launch(int kw) { return 8 * ((device_cus() / 8) / kw); }
 
+// The tiling of a call: the table's default for the head dim, or its small-batch alternative (variant 2) while all
+// groups of the call fit one launch with 4-row tiles.  FRNN_FUSED_VARIANT picks a variant by hand.
+static bool pick_plan(int function, int dtype, int B, int N, int D, int backward, Plan* p) {
+  const int variant = env_int("FRNN_FUSED_VARIANT", 0);
+  if (!find_plan(function, dtype, D, variant, backward, p)) return false;
+  if (variant == 0) {
+    Plan q;
+    if (find_plan(function, dtype, D, 2, backward, &q) && q.variant == 2 && q.kw > 1 &&
+        (long)N * ((B + 3) / 4) <= groups_per_launch(q.kw))
+      *p = q;
+  }
+  return true;
+}
+
 // Batch rows per group: 4, 8 or 16.  Fewer rows per tile mean less gate math per lane and fewer
 // words to poll per step (the larger costs of a step) at the price of more workgroups and copies
 // of R, so the smallest tile is used for which every workgroup of the call still gets a compute
@@ -425,7 +439,7 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
   int e = check_problem(function, dtype, B, 1, N, D);
   if (e) return e;
   Plan p;
-  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p))
+  if (!pick_plan(function, dtype, B, N, D, backward, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   if (waves) *waves = p.waves;
   if (tiles_per_wave) *tiles_per_wave = p.utw;
@@ -449,7 +463,7 @@ size_t frnn_fused_cache_bytes_opt(int function, int dtype, int B, int T, int N, 
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
   Plan p;
-  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward, &p)) return 0;
+  if (!pick_plan(function, dtype, B, N, D, backward, &p)) return 0;
   return backward ? carve_fused_bwd(nullptr, function, dtype, B, T, N, D, p).total
                   : carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
 }
@@ -459,7 +473,7 @@ size_t frnn_fused_workspace_bytes_opt(int function, int dtype, int B, int T, int
   Opts o;
   if (check_problem(function, dtype, B, T, N, D) || parse_opts(opt, function, &o)) return 0;
   Plan p;
-  if (!find_plan(o.fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), backward ? (o.rc ? 2 : 1) : 0, &p)) return 0;
+  if (!pick_plan(o.fx, dtype, B, N, D, backward ? (o.rc ? 2 : 1) : 0, &p)) return 0;
   return backward ? carve_fused_bwd(nullptr, o.fx, dtype, B, T, N, D, p).total
                   : carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
 }
@@ -487,7 +501,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   if (e) return e;
   const int fx = o.fx;
   Plan p;
-  if (!find_plan(fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
+  if (!pick_plan(fx, dtype, B, N, D, 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   e = check_fused_sizes(fx, dtype, B, T, N, D);
   if (e) return e;
@@ -569,7 +583,7 @@ int frnn_fused_forward_static(int function, int dtype, int training, int B, int 
   int e = check_problem(function, dtype, B, T, N, D);
   if (e) return e;
   Plan p;
-  if (!find_plan(function, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), 0, &p))
+  if (!pick_plan(function, dtype, B, N, D, 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   const size_t need = carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
   if (need > kStaticScratchBytes)
@@ -607,7 +621,7 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   const int fx = o.fx;
   const CellDims c = cell_dims(fx);
   Plan p;
-  if (!find_plan(fx, dtype, D, env_int("FRNN_FUSED_VARIANT", 0), o.rc ? 2 : 1, &p))
+  if (!pick_plan(fx, dtype, B, N, D, o.rc ? 2 : 1, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused%s kernel for function %d dtype %d head dim %d", o.rc ? " recompute-mode" : "",
                 function, dtype, D);
   e = check_fused_sizes(fx, dtype, B, T, N, D);

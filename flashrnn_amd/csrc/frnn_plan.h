@@ -9,8 +9,10 @@
 // compiler's resource report of every instantiation.
 //   R registers per lane = UTW * G_r * D / 8 (bf16) or UTW * G_r * D / 4 (f32); a workgroup of
 //   4 waves (one per SIMD) may use up to 512 VGPRs per lane, one of 8 waves 256, of 16 waves 128.
-// VARIANT 0 is the default; to try another tiling add an X(D, 1, ...) entry and run with
-// FRNN_FUSED_VARIANT=1.  The alternatives that were measured and lost (4 waves x 2 tiles for
+// VARIANT 0 is the default.  VARIANT 2, where a head dim has one, spreads the head over more workgroups: it is
+// used instead of the default while every workgroup of the call still gets a compute unit of its own with 4-row
+// batch tiles (measured faster there, slower once the device is full).  To try another tiling add an
+// X(D, 1, ...) entry and run with FRNN_FUSED_VARIANT=1.  The alternatives that were measured and lost (4 waves x 2 tiles for
 // D = 128, 2 x 8 waves or 8 x 2 waves for D = 256, ...) are not compiled in.
 // Forward and backward tile independently (the gate cache layout does not depend on the plan).
 #pragma once
@@ -32,6 +34,7 @@ struct Plan {
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 12, 1, 1, 4) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 #define FRNN_BWD_PLANS_GR4_BF16(X) \
+  X(160, 2, 2, 1, 5, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 4) X(192, 0, 4, 1, 3, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 // slstm backward: as above, but D = 160 as 5 workgroups of 2 waves (10 waves of 168 registers each spill at every tile height)
@@ -48,25 +51,28 @@ struct Plan {
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 8) X(448, 0, 2, 1, 14, 4) X(512, 0, 2, 1, 16, 4)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
+  X(64, 2, 2, 1, 2, 16) \
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 4) X(448, 0, 2, 1, 14, 8) X(512, 0, 1, 1, 32, 4)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 16) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_BWD_PLANS_GR3_BF16(X) \
+  X(192, 2, 4, 1, 3, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 12, 1, 1, 4) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_PLANS_GR3_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 8) X(512, 0, 4, 1, 8, 8)
 #define FRNN_BWD_PLANS_GR3_F32(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
+  X(64, 2, 2, 1, 2, 16) \
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 8) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 8)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
-  X(256, 0, 16, 1, 1, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 8, 3, 1, 4) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 2, 4, 16) X(640, 0, 4, 1, 10, 16) \
+  X(256, 0, 16, 1, 1, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 8, 3, 1, 4) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) \
   X(768, 0, 8, 1, 6, 16) X(1024, 0, 8, 1, 8, 8)
 #define FRNN_BWD_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
@@ -76,9 +82,11 @@ struct Plan {
 // spread over D / 64 workgroups with one tile per wave: D = 256 as one workgroup of 4 waves x 4 tiles took 8.0 ms
 // per 1024 steps forward + backward, as 4 workgroups it takes 2.7)
 #define FRNN_PLANS_GR1_F32(X) \
+  X(96, 2, 2, 1, 3, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 8)
 #define FRNN_BWD_PLANS_GR1_F32(X) \
+  X(96, 2, 2, 1, 3, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 16) X(1024, 0, 4, 1, 16, 8)
 

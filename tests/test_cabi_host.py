@@ -90,6 +90,21 @@ def test_plan_and_sizes(lib):
     assert lib.frnn_fused_workspace_bytes(L, 0, 8, 1024, 3, 2048, 0) == 0  # unsupported
 
 
+def test_small_batches_get_the_tiling_with_more_workgroups_per_head(lib):
+    """Where the table has a small-batch alternative for a head dim (gru bf16 D = 192 backward: 3 workgroups of 4
+    waves instead of one of 12), it is used while all groups of the call fit one launch with 4-row tiles, and the
+    workspace size follows the choice."""
+    G = _lib.FUNCTION_IDS["gru"]
+    out = [ctypes.c_int() for _ in range(4)]
+    plan = lambda B, backward: (lib.frnn_fused_plan(G, 0, B, 4, 192, backward, *[ctypes.byref(o) for o in out]),
+                                [o.value for o in out])[1]
+    assert plan(16, 1)[:3] == [4, 1, 3] and plan(1024, 1)[:3] == [12, 1, 1]
+    assert plan(16, 0)[:3] == [12, 1, 1]  # forward: one tiling
+    ws = lambda B: lib.frnn_fused_workspace_bytes(G, 0, B, 64, 4, 192, 1)
+    assert ws(16) > 256 + 64 * 1024  # exchange buffers of the 3-workgroup tiling
+    assert lib.frnn_fused_workspace_bytes(G, 0, 16, 64, 4, 192, 0) <= 1024  # one workgroup per head: the status word only
+
+
 def _fwd(lib, entry, function=0, dtype=0, B=8, T=4, N=1, D=64, Wx=FAKE, R=FAKE, b=FAKE, s0=FAKE, states=FAKE,
          cache=FAKE, ws=FAKE, ws_bytes=0, training=1):
     return getattr(lib, entry)(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, ws, ws_bytes, None)

@@ -79,6 +79,19 @@ FUSED_SMALL = [
     ("elman", 7, 5, 1, 768, "float32"),
     ("elman", 10, 4, 1, 1024, "float32"),
     ("lstm", 37, 4, 1, 512, "float32"),      # 10 groups of 4 rows: two backward launches (8 groups of 32 workgroups each)
+    # elman fp32 from D = 128 on: D / 64 workgroups of one tile per wave
+    ("elman", 6, 5, 2, 128, "float32"),
+    ("elman", 21, 4, 1, 192, "float32"),
+    ("elman", 9, 6, 2, 256, "float32"),
+    ("elman", 40, 4, 1, 512, "float32"),
+    # head dims with a small-batch tiling (more workgroups per head while the call fits one launch at 4-row tiles):
+    # these run on it, test_default_tiling_of_head_dims_with_a_small_batch_one on the other
+    ("gru", 14, 5, 2, 192, "bfloat16"),
+    ("lstm", 10, 5, 2, 160, "bfloat16"),
+    ("lstm", 9, 6, 3, 64, "float32"),
+    ("gru", 11, 5, 2, 64, "float32"),
+    ("elman", 8, 5, 1, 96, "float32"),
+    ("lstm", 12, 5, 1, 96, "float32"), ("gru", 70, 4, 2, 96, "float32"),   # backward: 3 workgroups of 2 waves
 ]
 
 
@@ -119,6 +132,26 @@ def test_fused_every_batch_tiling(gpu, monkeypatch, tile_rows, function, B, T, N
     print(f"case tiling rows={tile_rows} {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
     monkeypatch.setenv("FRNN_TILE_ROWS", str(tile_rows))
     check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=13, init="randn")
+
+
+# Head dims whose table holds two tilings: small calls run on the one with more workgroups per head (the cases
+# above), calls that fill the device on the default one, which FRNN_FUSED_VARIANT=1 (no such entry: the table's
+# default, and no switching) selects here at a small size; both with every batch tile height they are compiled for.
+TWO_TILINGS = [
+    ("gru", 14, 5, 2, 192, "bfloat16"), ("lstm", 10, 5, 2, 160, "bfloat16"), ("lstm", 9, 6, 3, 64, "float32"),
+    ("gru", 11, 5, 2, 64, "float32"), ("slstm", 7, 5, 2, 64, "float32"), ("elman", 8, 5, 1, 96, "float32"),
+]
+
+
+@pytest.mark.parametrize("function,B,T,N,D,dtype", TWO_TILINGS)
+@pytest.mark.parametrize("tile_rows", [4, 8, 16])
+@pytest.mark.parametrize("default_tiling", [True, False])
+def test_both_tilings_of_head_dims_with_a_small_batch_one(gpu, monkeypatch, default_tiling, tile_rows, function, B, T, N, D, dtype):
+    print(f"case two tilings default={default_tiling} rows={tile_rows} {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
+    monkeypatch.setenv("FRNN_TILE_ROWS", str(tile_rows))
+    if default_tiling:
+        monkeypatch.setenv("FRNN_FUSED_VARIANT", "1")
+    check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=17, init="randn")
 
 
 def test_fused_more_groups_than_one_launch_holds(gpu):

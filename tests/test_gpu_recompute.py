@@ -75,12 +75,15 @@ def test_recompute_in_fp32_gives_the_bits_of_the_cached_path(gpu, function, tile
     """fp32 storage: the stored h is what the forward pass fed to its product.  With 8-row tiles the rebuild runs the
     same MFMA chain and the same gate math as the forward pass, so every gradient must come out bit for bit as with
     the cache.  With 4-row tiles the forward product runs on the 4x4x1 instruction (another summation order) and
-    the rebuild on the 16x16x4 one: equal to fp32 rounding."""
+    the rebuild on the 16x16x4 one: equal to fp32 rounding.  (Both reverse kernels on the tiling that the two modes
+    share, one workgroup per head: a small call with the cache would otherwise run as 2 workgroups per head, which
+    sum the recurrent cotangent in another order.)"""
     from flashrnn_amd import FlashRNNConfig, flashrnn
 
     B, T, N, D = 7, 33, 2, 64
     print(f"case recompute bits {function} rows {tile_rows}", flush=True)
     monkeypatch.setenv("FRNN_TILE_ROWS", str(tile_rows))
+    monkeypatch.setenv("FRNN_FUSED_VARIANT", "1")  # (no such entry: the table's default tiling, no switching)
     inp = make_inputs(function, B, T, N, D, 84, init="randn")
     res = []
     for rc in (False, True):
