@@ -39,10 +39,12 @@ struct Plan {
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 // slstm backward: as above, but D = 160 as 5 workgroups of 2 waves (10 waves of 168 registers each spill at every tile height)
 #define FRNN_BWD_PLANS_SLSTM_BF16(X) \
+  X(128, 2, 4, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 // slstm: its heavier gate math tips D = 192 forward to 3 workgroups of 4 waves (1.19 against 1.26 ms)
 #define FRNN_PLANS_SLSTM_BF16(X) \
+  X(160, 2, 2, 1, 5, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 4, 1, 3, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
 // fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave, so D = 512 is as far as one tile per

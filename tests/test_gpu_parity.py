@@ -140,6 +140,7 @@ def test_fused_every_batch_tiling(gpu, monkeypatch, tile_rows, function, B, T, N
 TWO_TILINGS = [
     ("gru", 14, 5, 2, 192, "bfloat16"), ("lstm", 10, 5, 2, 160, "bfloat16"), ("lstm", 9, 6, 3, 64, "float32"),
     ("gru", 11, 5, 2, 64, "float32"), ("slstm", 7, 5, 2, 64, "float32"), ("elman", 8, 5, 1, 96, "float32"),
+    ("slstm", 9, 6, 2, 160, "bfloat16"), ("slstm", 6, 5, 3, 128, "bfloat16"),
 ]
 
 
