@@ -125,15 +125,19 @@ static bool near_stores_allowed() { return env_int("FRNN_AGENT_STORES", 0) == 0;
 // the data arrives depends on how long the other workgroups' gate math and stores take, so the best
 // value differs by cell and tiling.  Measured on MI355X (bf16, T = 1024, exchange stores kept in the XCD's
 // L2; a unit off costs up to 1-3 %, most curves are flat within 2 units):
-//   heads of up to 8 workgroups (own slice multiplied in front of the wait), 4-row tiles: lstm D=256 0, D=320 0,
-//   D=512 1; slstm D=192, 256 0; gru D=256, 384 1; elman D=512, 1024 0; 8- and 16-row tiles 2-4 (flat);
-//   lstm D=640 (10 workgroups) 5, D=768 (12) 6, D=1024 (32 workgroups of 2 waves) 3-6; gru D=1024 (16) 6.
+//   kernels that multiply the own slice in front of the wait, 4-row tiles: lstm D=256 0, D=320 0, D=512 1, D=640 1;
+//   slstm D=192, 256 0, D=640 1; gru D=256, 384, 640 1, D=768 2, D=1024 (16 workgroups) 6; elman D=512, 1024 0,
+//   D=640 2, fp32 0; 8- and 16-row tiles 2-4 (flat);
+//   the others: lstm D=768 (12 workgroups, part of R in LDS) 6, D=1024 (32 workgroups of 2 waves) 3-6.
 static int fwd_poll_delay_default(int function, int dtype, const Plan& p, int tile_rows) {
   if (p.kw <= 1) return 0;
   const bool elman = function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP;
-  // up to 8 workgroups per head the k-steps over the workgroup's own slice run in front of the wait (not in the fp32
-  // kernels of 4-row tiles, whose product has another form): little is left to sleep through
-  if (p.kw <= 8 && !(dtype == FRNN_F32 && tile_rows == 4 && !elman)) return elman ? 0 : tile_rows >= 8 ? 2 : (function == FRNN_GRU || p.kw > 5) ? 1 : 0;
+  // kernels that multiply the workgroup's own slice in front of the wait: little is left to sleep through
+  if (fwd_own_slice_first(cell_dims(function).GR, p.D, p.waves, p.utw, p.kw, tile_rows, dtype == FRNN_F32 ? 4 : 2)) {
+    if (elman) return p.kw > 8 && dtype != FRNN_F32 ? 2 : 0;
+    if (p.kw > 8) return p.kw >= 16 ? 6 : p.kw >= 12 ? 2 : 1;
+    return tile_rows >= 8 ? 2 : (function == FRNN_GRU || p.kw > 5) ? 1 : 0;
+  }
   if (elman) return p.waves > 4 ? 2 : 6;
   if (p.kw == 3) return 2;
   if (p.kw == 6) return 4;

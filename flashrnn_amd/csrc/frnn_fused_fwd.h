@@ -19,6 +19,7 @@
 // first MFMA of each gate.
 #pragma once
 #include "frnn_exchange.h"
+#include "frnn_plan.h"
 #include "frnn_pointwise.h"
 
 namespace frnn {
@@ -47,19 +48,6 @@ struct FwdArgs {
 #else
 #define FRNN_STAMP(var)
 #endif
-
-// Resident operand of the forward product: a wave holds UTW*G_r*KS fragments of R.  When they alone
-// would take more than 400 of the 512 registers a wave has at one wave per SIMD (LSTM D = 1024: all
-// 512), those of the last RLK k-steps live in LDS instead (as many as bring the rest down to 352, and
-// as fit beside the two h buffers) and are read back one k-step ahead as the A operand of their MFMAs.
-constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
-  const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4, FRB = esize == 4 ? 4 : 16;
-  const int KS = D / KM, per = UTW * GR * FR, regs = per * KS;
-  if (!(WAVES <= 4 && regs > 336)) return 0;
-  const int want = (regs - 320 + per - 1) / per;
-  const int room = (160 * 1024 - 2 * 16 * D * esize - 1024) / (WAVES * UTW * GR * 64 * FRB);
-  return want < room ? want : room;
-}
 
 template <typename T> __device__ __forceinline__ typename ST<T>::Frag load_frag(const T* row, int ks, int kq);
 template <> __device__ __forceinline__ bf16x8 load_frag<bf16_t>(const bf16_t* row, int ks, int kq) {
@@ -102,7 +90,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   // columns of a block = the gates of that unit, A = h (the values of one block broadcast to all 16), one
   // instruction per k: D instructions of 8 cycles per tile and step instead of G_r * D / 4 of 32.
   constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
-  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && GR >= 3 && RLK == 0 && D <= 384;  // (the whole operand, D registers per tile, in registers)
+  constexpr bool M44 = fwd_form_4x4x1(GR, D, WAVES, UTW, TR, (int)sizeof(T));  // (the whole operand, D registers per tile, in registers)
   // Own slice first: of the h_(t-1) a step multiplies with, the workgroup's own D / KW units are in LDS as soon as
   // its waves have finished step t-1; the k-steps over them run before the wait for the other workgroups' slices
   // (behind one more LDS barrier) and leave the critical path.  Each workgroup keeps R and h rotated along k so
@@ -110,10 +98,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
 #ifdef FRNN_NO_OWN_FIRST
   constexpr bool OWN_FIRST = false;
 #else
-  // (not for the fp32 kernels whose operand alone takes 256 registers and whose 16-row tiles keep 4 elements per
-  // lane: with the two-part product they spill)
-  constexpr bool OWN_FIRST = KW > 1 && KW <= 8 && !M44 && RLK == 0 && (D / KW) % X::KM == 0 &&
-                             !(sizeof(T) == 4 && UTW * GR * KS >= 256 && TR == 16);
+  constexpr bool OWN_FIRST = fwd_own_slice_first(GR, D, WAVES, UTW, KW, TR, (int)sizeof(T));
 #endif
   constexpr int KSO = OWN_FIRST ? (D / KW) / X::KM : 0;
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];

@@ -23,6 +23,35 @@ struct Plan {
   int cooperative = 0;  // host side only: launch the kernel as a cooperative one (see fused_*_tu.hip)
   int recompute = 0;    // host side only: the reverse kernel of recompute mode
 };
+
+// Resident operand of the forward product: a wave holds UTW*G_r*KS fragments of R.  When they alone
+// would take more than 400 of the 512 registers a wave has at one wave per SIMD (LSTM D = 1024: all
+// 512), those of the last RLK k-steps live in LDS instead (as many as bring the rest down to 352, and
+// as fit beside the two h buffers) and are read back one k-step ahead as the A operand of their MFMAs.
+constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
+  const int KM = esize == 4 ? 4 : 32, FR = esize == 4 ? 1 : 4, FRB = esize == 4 ? 4 : 16;
+  const int KS = D / KM, per = UTW * GR * FR, regs = per * KS;
+  if (!(WAVES <= 4 && regs > 336)) return 0;
+  const int want = (regs - 320 + per - 1) / per;
+  const int room = (160 * 1024 - 2 * 16 * D * esize - 1024) / (WAVES * UTW * GR * 64 * FRB);
+  return want < room ? want : room;
+}
+
+// Forward kernel, fp32 at 4-row tiles, cells with 3 or 4 recurrent gates: the product runs on v_mfma_f32_4x4x1_16B_f32
+// (see the kernel), when the whole operand, D registers per tile, fits the registers.
+constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esize) {
+  return esize == 4 && TR == 4 && GR >= 3 && fwd_lds_ksteps(GR, D, WAVES, UTW, esize) == 0 && D <= 384;
+}
+// Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
+// 2..16 workgroups whose operand is all in registers and whose slice is a whole number of k-steps; not the fp32
+// kernels whose operand alone takes 256 registers, at the tile heights where they keep 2 or 4 elements per lane
+// (with the two-part product they spill).  The host reads this for the delay of the first probe.
+constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize) {
+  const int KM = esize == 4 ? 4 : 32, KS = D / KM;
+  return KW > 1 && KW <= 16 && !fwd_form_4x4x1(GR, D, WAVES, UTW, TR, esize) &&
+         fwd_lds_ksteps(GR, D, WAVES, UTW, esize) == 0 && (D / KW) % KM == 0 &&
+         !(esize == 4 && UTW * GR * KS >= 256 && TR >= (KW > 8 ? 8 : 16));
+}
 }
 
 // Measured on MI355X (T = 1024, bf16): when the head fits one workgroup, one tile per wave and
