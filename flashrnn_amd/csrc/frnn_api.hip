@@ -72,6 +72,7 @@ static const Plan kFwd1F[] = {FRNN_PLANS_GR1_F32(FRNN_ROW)};
 static const Plan kBwd4B[] = {FRNN_BWD_PLANS_GR4_BF16(FRNN_ROW)};
 static const Plan kBwdSB[] = {FRNN_BWD_PLANS_SLSTM_BF16(FRNN_ROW)};
 static const Plan kBwd4F[] = {FRNN_BWD_PLANS_GR4_F32(FRNN_ROW)};
+static const Plan kBwdSF[] = {FRNN_BWD_PLANS_SLSTM_F32(FRNN_ROW)};
 static const Plan kBwd3B[] = {FRNN_BWD_PLANS_GR3_BF16(FRNN_ROW)};
 static const Plan kBwd3F[] = {FRNN_BWD_PLANS_GR3_F32(FRNN_ROW)};
 static const Plan kBwd1B[] = {FRNN_BWD_PLANS_GR1_BF16(FRNN_ROW)};
@@ -93,7 +94,10 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kFwd3B) else PICK(kFwd3F) }
     else { if (dtype != FRNN_F32) PICK(kFwd1B) else PICK(kFwd1F) }
   } else if (backward == 1) {
-    if (GR == 4) { if (dtype == FRNN_F32) PICK(kBwd4F) else if (function == FRNN_SLSTM) PICK(kBwdSB) else PICK(kBwd4B) }
+    if (GR == 4) {
+      if (dtype == FRNN_F32) { if (function == FRNN_SLSTM) PICK(kBwdSF) else PICK(kBwd4F) }
+      else if (function == FRNN_SLSTM) PICK(kBwdSB) else PICK(kBwd4B)
+    }
     else if (GR == 3) { if (dtype != FRNN_F32) PICK(kBwd3B) else PICK(kBwd3F) }
     else { if (dtype != FRNN_F32) PICK(kBwd1B) else PICK(kBwd1F) }
   } else {  // reverse scan in recompute mode
@@ -128,14 +132,14 @@ static bool near_stores_allowed() { return env_int("FRNN_AGENT_STORES", 0) == 0;
 //   kernels that multiply the own slice in front of the wait, 4-row tiles: lstm D=256 0, D=320 0, D=512 1, D=640 1;
 //   slstm D=192, 256 0, D=640 1; gru D=256, 384, 640 1, D=768 2, D=1024 (16 workgroups) 6; elman D=512, 1024 0,
 //   D=640 2, fp32 0; 8- and 16-row tiles 2-4 (flat);
-//   the others: lstm D=768 (12 workgroups, part of R in LDS) 6, D=1024 (32 workgroups of 2 waves) 3-6.
+//   lstm, slstm D=768 (12 workgroups) 0-1;  the others: lstm D=1024 (32 workgroups of 2 waves) 3-6.
 static int fwd_poll_delay_default(int function, int dtype, const Plan& p, int tile_rows) {
   if (p.kw <= 1) return 0;
   const bool elman = function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP;
   // kernels that multiply the workgroup's own slice in front of the wait: little is left to sleep through
   if (fwd_own_slice_first(cell_dims(function).GR, p.D, p.waves, p.utw, p.kw, tile_rows, dtype == FRNN_F32 ? 4 : 2)) {
     if (elman) return p.kw > 8 && dtype != FRNN_F32 ? 2 : 0;
-    if (p.kw > 8) return p.kw >= 16 ? 6 : p.kw >= 12 ? 2 : 1;
+    if (p.kw > 8) return p.kw >= 16 ? 6 : p.kw < 12 ? 1 : function == FRNN_GRU ? 2 : 0;
     return tile_rows >= 8 ? 2 : (function == FRNN_GRU || p.kw > 5) ? 1 : 0;
   }
   if (elman) return p.waves > 4 ? 2 : 6;

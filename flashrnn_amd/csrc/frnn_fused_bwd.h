@@ -127,9 +127,11 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   // columns of a block = 4 destination workgroups (the wave's tile position in each), A = dg of the own gate rows
   // (the values of one block broadcast to all 16), one instruction per k: KDL instructions of 8 cycles per 4
   // destinations instead of KDL / 4 of 32 per destination.
-  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && KW >= 2 && !RC &&
-                       bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)) == 0;  // (the whole operand in registers)
   constexpr int NG4 = (KW + 3) / 4;  // groups of 4 destinations
+  // (the whole operand, a register per destination group and own gate row, in the registers of a wave: wherever the
+  // 16x16x4 form keeps it there too, and up to 320 registers at one wave per SIMD)
+  constexpr bool M44 = sizeof(T) == 4 && TR == 4 && KW >= 2 && !RC &&
+                       (bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)) == 0 || (WAVES <= 4 && NG4 * UTW * KDL <= 320));
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);

@@ -52,6 +52,9 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
 #elif FRNN_DT != 1
 #define FRNN_TU_PLANS FRNN_PLANS_GR4_BF16
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_BF16
+#elif FRNN_F == 1
+#define FRNN_TU_PLANS FRNN_PLANS_GR4_F32
+#define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_SLSTM_F32
 #else
 #define FRNN_TU_PLANS FRNN_PLANS_GR4_F32
 #define FRNN_TU_BWD_PLANS FRNN_BWD_PLANS_GR4_F32

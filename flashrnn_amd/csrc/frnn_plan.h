@@ -38,18 +38,19 @@ constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
 }
 
 // Forward kernel, fp32 at 4-row tiles, cells with 3 or 4 recurrent gates: the product runs on v_mfma_f32_4x4x1_16B_f32
-// (see the kernel), when the whole operand, D registers per tile, fits the registers.
+// (see the kernel), when the whole operand, D registers per tile in that form, fits the registers of a wave
+// (workgroups of up to 4 waves: 512 registers each).
 constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esize) {
-  return esize == 4 && TR == 4 && GR >= 3 && fwd_lds_ksteps(GR, D, WAVES, UTW, esize) == 0 && D <= 384;
+  return esize == 4 && TR == 4 && GR >= 3 && WAVES <= 4 && UTW * D <= 384;
 }
 // Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
-// 2..16 workgroups whose operand is all in registers and whose slice is a whole number of k-steps; not the fp32
+// 2..16 workgroups (up to 12 where part of the operand lives in LDS) whose slice is a whole number of k-steps; not the fp32
 // kernels whose operand alone takes 256 registers, at the tile heights where they keep 2 or 4 elements per lane
 // (with the two-part product they spill).  The host reads this for the delay of the first probe.
 constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize) {
   const int KM = esize == 4 ? 4 : 32, KS = D / KM;
   return KW > 1 && KW <= 16 && !fwd_form_4x4x1(GR, D, WAVES, UTW, TR, esize) &&
-         fwd_lds_ksteps(GR, D, WAVES, UTW, esize) == 0 && (D / KW) % KM == 0 &&
+         (fwd_lds_ksteps(GR, D, WAVES, UTW, esize) == 0 || KW <= 12) && (D / KW) % KM == 0 &&
          !(esize == 4 && UTW * GR * KS >= 256 && TR >= (KW > 8 ? 8 : 16));
 }
 }
@@ -82,6 +83,12 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 8) X(448, 0, 2, 1, 14, 4) X(512, 0, 2, 1, 16, 4)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
+  X(320, 2, 1, 1, 20, 4) \
+  X(64, 2, 2, 1, 2, 16) \
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 4) X(448, 0, 2, 1, 14, 8) X(512, 0, 1, 1, 32, 4)
+// slstm fp32 backward: the same without the 20-workgroup tiling of D = 320 (with four states its kernel spills)
+#define FRNN_BWD_PLANS_SLSTM_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 4) X(448, 0, 2, 1, 14, 8) X(512, 0, 1, 1, 32, 4)

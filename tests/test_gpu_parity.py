@@ -141,6 +141,7 @@ TWO_TILINGS = [
     ("gru", 14, 5, 2, 192, "bfloat16"), ("lstm", 10, 5, 2, 160, "bfloat16"), ("lstm", 9, 6, 3, 64, "float32"),
     ("gru", 11, 5, 2, 64, "float32"), ("slstm", 7, 5, 2, 64, "float32"), ("elman", 8, 5, 1, 96, "float32"),
     ("slstm", 9, 6, 2, 160, "bfloat16"), ("slstm", 6, 5, 3, 128, "bfloat16"),
+    ("lstm", 6, 5, 1, 320, "float32"),       # backward: 20 workgroups of one wave / 5 of 4 waves
 ]
 
 
