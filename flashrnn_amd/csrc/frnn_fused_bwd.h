@@ -209,6 +209,19 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
         }
       }
     }
+#ifndef FRNN_NO_AGPR_PIN
+    // what does not fit the architectural VGPRs beside the working set is pinned to accumulation registers, where the
+    // MFMA reads it in place (left to the register allocator it is copied back before every use)
+    // (384 registers: the 152 that would stay in VGPRs leave too little for the working set; left alone there)
+    constexpr int ALL44 = NG4 * UTW * KDL, PIN44 = ALL44 > 344 ? 0 : ALL44 - 112 > 232 ? 232 : ALL44 - 112;
+#pragma unroll
+    for (int q = 0; q < NG4; ++q)
+#pragma unroll
+      for (int u = 0; u < UTW; ++u)
+#pragma unroll
+        for (int kk = 0; kk < KDL; ++kk)
+          if (ALL44 - 1 - ((q * UTW + u) * KDL + kk) < PIN44) asm volatile("" : "+a"(rtb[q][u][kk]));
+#endif
   }
 #pragma unroll
   for (int r = 0; r < (M44 ? 0 : KW); ++r) {

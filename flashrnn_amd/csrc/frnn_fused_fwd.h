@@ -159,6 +159,14 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         rb[u][k] = j < GR ? v.x : 0.f; rb[u][k + 1] = j < GR ? v.y : 0.f;
         rb[u][k + 2] = j < GR ? v.z : 0.f; rb[u][k + 3] = j < GR ? v.w : 0.f;
       }
+#ifndef FRNN_NO_AGPR_PIN
+      // (as for the fragments below: what does not fit the architectural VGPRs beside the working set is pinned to
+      // accumulation registers, where the MFMA reads it in place, instead of being copied back before every use)
+      constexpr int PIN44 = UTW * D - 128 > 232 ? 232 : UTW * D - 128;
+#pragma unroll
+      for (int k = 0; k < D; ++k)
+        if (u * D + (D - 1 - k) < PIN44) asm volatile("" : "+a"(rb[u][k]));
+#endif
     }
   }
 #pragma unroll
