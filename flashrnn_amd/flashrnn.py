@@ -130,6 +130,32 @@ class FlashRNNConfig:
             self.hidden_dim = self.num_heads * self.head_dim
 
 
+def _raw_stream(device: torch.device) -> int:
+    """The current stream of `device` as the integer handle that the C ABI takes."""
+    get = getattr(torch._C, "_cuda_getCurrentRawStream", None)  # (no Stream object is built: several microseconds per call)
+    if get is not None:
+        return get(device.index if device.index is not None else torch.cuda.current_device())
+    return torch.cuda.current_stream(device).cuda_stream
+
+
+class _on_device:
+    """`with torch.cuda.device(d)` that does nothing when d is already the current device (the usual case)."""
+
+    def __init__(self, device: torch.device):
+        self._ctx = None
+        if device.index is not None and device.index != torch.cuda.current_device():
+            self._ctx = torch.cuda.device(device)
+
+    def __enter__(self):
+        if self._ctx is not None:
+            self._ctx.__enter__()
+
+    def __exit__(self, *exc):
+        if self._ctx is not None:
+            self._ctx.__exit__(*exc)
+        return False
+
+
 def _entry(backend: str, name: str):
     prefix = "frnn_fused_" if backend == "hip_fused" else "frnn_alt_"
     return getattr(_lib.load_library(), prefix + name)
@@ -165,7 +191,8 @@ class _StatusLog:
     completed are read at the start of every later call (forward or backward, any stream), and a non-zero
     one raises RuntimeError there.  ``check_status()`` waits for the entries still pending (their events
     only) and does the same.  Entries made under stream capture are not logged: a replay repeats the
-    kernels, not this bookkeeping."""
+    kernels, not this bookkeeping.  The pinned words and events of entries that have been read are used again
+    (except the most recent entry of each kind, which ``last()`` may still be asked for)."""
 
     def __init__(self):
         import collections
@@ -174,13 +201,16 @@ class _StatusLog:
         self._lock = threading.Lock()
         self._pending = collections.deque()
         self._last = {}
+        self._free = []
 
     def log(self, kind: str, ws: torch.Tensor, what: str):
         if torch.cuda.is_current_stream_capturing():
             return
-        host = torch.empty(1, dtype=torch.int32, pin_memory=True)
+        with self._lock:
+            host, ev = self._free.pop() if self._free else (None, None)
+        if host is None:
+            host, ev = torch.empty(1, dtype=torch.int32, pin_memory=True), torch.cuda.Event()
         host.copy_(ws[:4].view(torch.int32), non_blocking=True)
-        ev = torch.cuda.Event()
         ev.record()
         entry = (kind, what, host, ev)
         with self._lock:
@@ -201,6 +231,8 @@ class _StatusLog:
                 if ev.query():
                     if int(host[0]) != 0:
                         failed.append(f"{kind} of {what}")
+                    if self._last.get(kind) is not entry and len(self._free) < 64:
+                        self._free.append((host, ev))
                 else:
                     keep.append(entry)
             self._pending.extend(keep)
@@ -268,7 +300,7 @@ class _FlashRNNFunction(torch.autograd.Function):
         R_k = R.detach().to(kdt).contiguous()
         b_k = b.detach().to(kdt).contiguous()
         s0_k = s0.detach().to(kdt).reshape(S, B, N, D).contiguous()
-        with torch.cuda.device(Wx.device):
+        with _on_device(Wx.device):
             rc = _entry(cfg.backend, "supported")(f_id, d_id, B, N, D)
             if rc == 0 and cfg.recompute_gates:
                 if cfg.backend != "hip_fused":
@@ -281,7 +313,7 @@ class _FlashRNNFunction(torch.autograd.Function):
             cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx.device)
             ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 0)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx.device)
-            stream = torch.cuda.current_stream().cuda_stream
+            stream = _raw_stream(Wx.device)
             rc = _entry(cfg.backend, "forward_opt")(
                 f_id, d_id, int(training), B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(),
                 s0_k.data_ptr(), states.data_ptr(), cache.data_ptr() if training else None,
@@ -310,14 +342,14 @@ class _FlashRNNFunction(torch.autograd.Function):
         dev = states.device
         _status.poll()
         ds = dstates.to(kdt).contiguous()
-        with torch.cuda.device(dev):
+        with _on_device(dev):
             dWx = torch.empty((B, T, Gw, N, D), dtype=kdt, device=dev)
             ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
             dR = torch.empty((Gr, N, D, D), dtype=torch.float32, device=dev)
             db = torch.empty((Gt, N, D), dtype=torch.float32, device=dev)
             ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 1)
             ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
-            stream = torch.cuda.current_stream().cuda_stream
+            stream = _raw_stream(dev)
             if cfg.recompute_gates:
                 rc = _lib.load_library().frnn_fused_backward_recompute(
                     f_id, d_id, B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(),
@@ -477,11 +509,11 @@ def flashrnn_step(
                               or not carry.is_contiguous() or carry.device != Wx.device):
         raise TypeError(f"carry must be a contiguous float32 tensor [{S},{B},{N},{D}] on the device of Wx")
     f_id, d_id = _lib.FUNCTION_IDS[config.function], _lib.DTYPE_IDS[config.dtype]
-    with torch.cuda.device(Wx.device):
+    with _on_device(Wx.device):
         out = torch.empty((S, B, 1, N, D), dtype=kdt, device=Wx.device)
         rc = _entry(config.backend, "step")(
             f_id, d_id, B, N, D, Wx.data_ptr(), R.data_ptr(), b.data_ptr(), states.data_ptr(), out.data_ptr(),
-            carry.data_ptr() if carry is not None else None, torch.cuda.current_stream().cuda_stream, _options(config))
+            carry.data_ptr() if carry is not None else None, _raw_stream(Wx.device), _options(config))
         if rc != 0:
             _raise(rc, f"{config.backend} step")
     return out
