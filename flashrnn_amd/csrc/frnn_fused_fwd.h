@@ -61,7 +61,8 @@ template <> __device__ __forceinline__ float load_frag<float>(const float* row, 
 }
 
 template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR>
-__global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) {
+__global__ void __launch_bounds__((WAVES + (fwd_producer_wave(Cell<F>::GR, D, WAVES, UTW, KW, TR, (int)sizeof(T)) ? 1 : 0)) * 64)
+fused_fwd_kernel(const FwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
@@ -103,6 +104,10 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr int KSO = OWN_FIRST ? (D / KW) / X::KM : 0;
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
   __shared__ int dead_flag, near_word;
+  // Wx of one step for the whole workgroup, two buffers by step parity: [tile][gate][batch row][16 units]
+  constexpr bool PW = fwd_producer_wave(GR, D, WAVES, UTW, KW, TR, (int)sizeof(T));
+  constexpr int WBUF = UT_WG * GW * TR * 16;
+  __shared__ __attribute__((aligned(16))) T wbuf[PW ? 2 * WBUF + 8 : 1];  // (+ 16 bytes that swallow the writes of lanes without a piece)
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
 
@@ -128,6 +133,62 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
   constexpr int NCP = CacheBlk<T, NCA>::NCP, NWC = CacheBlk<T, NCA>::template Words<E>::value;
   const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * (NC ? NCP : 0) * ES);
+
+  // ---- the producer wave (see fwd_producer_wave): the workgroup's last wave.  It takes part in every barrier of the
+  //      compute waves, in the same order and under the same conditions (all of them wave-uniform values that every
+  //      wave reads from LDS behind a barrier).  Wx of step s travels in register set s % 3; iteration t (the compute
+  //      waves are in step t and read buffer t & 1) writes Wx(t+1) into the other buffer, which the compute waves read
+  //      behind the barriers of step t+1, and then sends for Wx(t+3) --------------------------------------------------
+  if constexpr (PW) {
+    if (w == WAVES) {
+      constexpr int CH_TOT = UT_WG * GW * TR * 2, NCH = (CH_TOT + 63) / 64;  // 16-byte pieces (8 units) per step, per lane
+      unsigned pv[NCH]; int pl[NCH];
+#pragma unroll
+      for (int i = 0; i < NCH; ++i) {
+        const int c = lane + 64 * i, half = c & 1, pr = (c >> 1) % TR, pg = ((c >> 1) / TR) % GW, ptile = (c >> 1) / (TR * GW);
+        const bool ok = c < CH_TOT && bt * TR + pr < B;
+        pv[i] = ok ? ((((unsigned)(bt * TR + pr) * Tn * GW + pg) * ND + n * D + slice * (D / KW) + ptile * 16 + half * 8) * ES) : kInvalidOff;
+        pl[i] = c < CH_TOT ? ((ptile * GW + pg) * TR + pr) * 16 + half * 8 : -1;  // (-1: the spare 16 bytes behind the buffers)
+      }
+      Dw<4> set[3][NCH];
+      auto fetch = [&](Dw<4> (&dst)[NCH], int s_) __attribute__((always_inline)) {
+        const int sc = s_ < Tn ? s_ : Tn - 1;
+#pragma unroll
+        for (int i = 0; i < NCH; ++i) dst[i] = buf_load<4>(rWx, pv[i], (unsigned)sc * GW * ND * ES);
+      };
+      auto put = [&](const Dw<4> (&src)[NCH], int s_) __attribute__((always_inline)) {
+        // (no branch on the lane: behind one the compiler waits for every load in flight, the latest ones included)
+#pragma unroll
+        for (int i = 0; i < NCH; ++i)
+          *reinterpret_cast<uint4*>(wbuf + (pl[i] >= 0 ? (s_ & 1) * WBUF + pl[i] : 2 * WBUF)) = make_uint4(src[i].v[0], src[i].v[1], src[i].v[2], src[i].v[3]);
+      };
+      fetch(set[0], 0); fetch(set[1], 1); fetch(set[2], 2);
+      put(set[0], 0);
+      __syncthreads();  // (the one of the prologue below)
+      bool pdead = __builtin_amdgcn_readfirstlane(near_word) < 0;
+      auto iter = [&](int t, const Dw<4> (&next)[NCH], Dw<4> (&refill)[NCH]) __attribute__((always_inline)) {
+        if (t > 0) {
+          if constexpr (OWN_FIRST) lds_barrier();
+          if (barrier_or(false, &dead_flag)) { pdead = true; return; }
+        }
+        put(next, t + 1);
+        fetch(refill, t + 3);
+      };
+      int t = 0;
+      for (; t + 2 < Tn && !pdead; t += 3) {
+        iter(t, set[1], set[0]);
+        if (pdead) break;
+        iter(t + 1, set[2], set[1]);
+        if (pdead) break;
+        iter(t + 2, set[0], set[2]);
+      }
+      if (!pdead && t < Tn) {
+        iter(t, set[1], set[0]);
+        if (!pdead && t + 1 < Tn) iter(t + 1, set[2], set[1]);
+      }
+      return;
+    }
+  }
 
   int ub[UTW];
   unsigned wx_v[UTW], st_v[UTW], ca_v[UTW];  // per-lane byte offsets; out of range for padded rows
@@ -266,6 +327,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
   constexpr bool WX_LATE = KW == 1;
   Dw<ND_> wx[PD + 1][UTW][GW];
   auto load_wx = [&](Dw<ND_> (&dst)[UTW][GW], int t) __attribute__((always_inline)) {
+    if constexpr (PW) return;  // (the producer wave's job)
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
@@ -329,6 +391,15 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
     }
     FRNN_STAMP(c1);
     if constexpr (!WX_LATE) load_wx(wn, min(t + PD, Tn - 1));
+    Dw<ND_> wcl[PW ? UTW : 1][PW ? GW : 1];  // this step's Wx from the producer wave's buffer
+    if constexpr (PW) {
+      static_assert(E == 1 && ND_ == 1, "4-row tiles: one element per lane and tile");
+      const unsigned short* const wb = reinterpret_cast<const unsigned short*>(wbuf) + cur * WBUF;
+#pragma unroll
+      for (int u = 0; u < UTW; ++u)
+#pragma unroll
+        for (int g = 0; g < GW; ++g) wcl[u][g].v[0] = wb[(((w * UTW + u) * GW + g) * TR + brow) * 16 + esub];
+    }
 
     // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once
     f32x4 acc[UTW][GR];
@@ -443,7 +514,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_fwd_kernel(const FwdArgs a) 
         }
       }
 #pragma unroll
-      for (int g = 0; g < GW; ++g) unpack<E>(wc[u][g], wxv[g], (T*)0);
+      for (int g = 0; g < GW; ++g) unpack<E>(PW ? wcl[PW ? u : 0][PW ? g : 0] : wc[u][g], wxv[g], (T*)0);
       float cv[NCA][E];
       float so[S][E];
 #pragma unroll

@@ -24,12 +24,14 @@ int fused_fwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const FwdArgs& a, hipStream
   if (p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                                 \
     auto kern = fwd_kernel_for<Dv, W, U, K, MTR>(a.tile_rows);                                \
     if (!kern) return FRNN_E_UNSUPPORTED;                                                     \
+    /* (one more wave where the kernel has a producer wave: the same predicate as in the kernel) */ \
+    const dim3 block((W + (fwd_producer_wave(Cell<FRNN_F>::GR, Dv, W, U, K, a.tile_rows, (int)sizeof(FRNN_TU_T)) ? 1 : 0)) * 64); \
     if (K > 1 && p.cooperative) {                                                             \
       FwdArgs aa = a;                                                                         \
       void* args[] = {(void*)&aa};                                                            \
-      return (int)hipLaunchCooperativeKernel((const void*)kern, grid, dim3(W * 64), args, 0, st); \
+      return (int)hipLaunchCooperativeKernel((const void*)kern, grid, block, args, 0, st);    \
     }                                                                                         \
-    hipLaunchKernelGGL(kern, grid, dim3(W * 64), 0, st, a);                                   \
+    hipLaunchKernelGGL(kern, grid, block, 0, st, a);                                          \
     return (int)hipGetLastError();                                                            \
   }
   FRNN_TU_PLANS(FRNN_CASE)
