@@ -393,12 +393,17 @@ fused_fwd_kernel(const FwdArgs a) {
     if constexpr (!WX_LATE) load_wx(wn, min(t + PD, Tn - 1));
     Dw<ND_> wcl[PW ? UTW : 1][PW ? GW : 1];  // this step's Wx from the producer wave's buffer
     if constexpr (PW) {
-      static_assert(E == 1 && ND_ == 1, "4-row tiles: one element per lane and tile");
-      const unsigned short* const wb = reinterpret_cast<const unsigned short*>(wbuf) + cur * WBUF;
+      // (the lane's E consecutive units of a gate: 2, 4 or 8 bytes)
+      const T* const wb = wbuf + cur * WBUF;
 #pragma unroll
       for (int u = 0; u < UTW; ++u)
 #pragma unroll
-        for (int g = 0; g < GW; ++g) wcl[u][g].v[0] = wb[(((w * UTW + u) * GW + g) * TR + brow) * 16 + esub];
+        for (int g = 0; g < GW; ++g) {
+          const T* const src = wb + (((w * UTW + u) * GW + g) * TR + brow) * 16 + esub;
+          if constexpr (E == 1) wcl[u][g].v[0] = *reinterpret_cast<const unsigned short*>(src);
+          else if constexpr (E == 2) wcl[u][g].v[0] = *reinterpret_cast<const unsigned*>(src);
+          else { const uint2 v = *reinterpret_cast<const uint2*>(src); wcl[u][g].v[0] = v.x; wcl[u][g].v[1] = v.y; }
+        }
     }
 
     // h fragments are read KC k-steps ahead of the MFMAs that use them, so LDS latency is paid once

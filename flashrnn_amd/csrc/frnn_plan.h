@@ -48,11 +48,11 @@ constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esi
 // issued in front of the wait delays the probe (a wave's memory operations return in order).  The producer wave has a
 // queue of its own: it loads the Wx of the whole workgroup three steps ahead and writes the Wx of the next step into an
 // LDS buffer, from which the compute waves take their elements with LDS reads.  For the kernels with steps of ~2000 cycles
-// (16-bit types, 4-row tiles, heads of several workgroups of 4 waves) that stay within the 256 registers a wave has when
+// (16-bit types, 4- and 8-row tiles, heads of several workgroups of 4 waves) that stay within the 256 registers a wave has when
 // five share four SIMDs, and for the cells with four gates: LSTM D = 256 forward 0.944 -> 0.887 ms per 1024 steps, sLSTM
 // D = 192 0.961 -> 0.914; the GRU (three loads per step to save) measured +1.5 % to -0.8 %, Elman the same to 0.3 %.
 constexpr bool fwd_producer_wave(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize) {
-  return esize == 2 && GR == 4 && KW > 1 && TR == 4 && WAVES == 4 && UTW * GR * (D / 32) * 4 <= 160;
+  return esize == 2 && GR == 4 && KW > 1 && TR <= 8 && WAVES == 4 && UTW * GR * (D / 32) * 4 <= (TR == 4 ? 160 : 128);
 }
 // Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
 // 2..16 workgroups (up to 12 where part of the operand lives in LDS) whose slice is a whole number of k-steps; not the fp32
