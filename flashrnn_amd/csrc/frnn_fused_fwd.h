@@ -165,11 +165,12 @@ fused_fwd_kernel(const FwdArgs a) {
       fetch(set[0], 0); fetch(set[1], 1); fetch(set[2], 2);
       put(set[0], 0);
       __syncthreads();  // (the one of the prologue below)
-      bool pdead = __builtin_amdgcn_readfirstlane(near_word) < 0;
+      bool pdead = KW > 1 && __builtin_amdgcn_readfirstlane(near_word) < 0;
       auto iter = [&](int t, const Dw<4> (&next)[NCH], Dw<4> (&refill)[NCH]) __attribute__((always_inline)) {
         if (t > 0) {
           if constexpr (OWN_FIRST) lds_barrier();
-          if (barrier_or(false, &dead_flag)) { pdead = true; return; }
+          if constexpr (KW > 1) { if (barrier_or(false, &dead_flag)) { pdead = true; return; } }
+          else lds_barrier();
         }
         put(next, t + 1);
         fetch(refill, t + 3);

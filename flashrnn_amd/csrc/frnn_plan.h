@@ -49,9 +49,11 @@ constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esi
 // queue of its own: it loads the Wx of the whole workgroup three steps ahead and writes the Wx of the next step into an
 // LDS buffer, from which the compute waves take their elements with LDS reads.  For the kernels with steps of ~2000 cycles
 // (16-bit types, 4- and 8-row tiles, heads of several workgroups of 4 waves) that stay within the 256 registers a wave has when
-// five share four SIMDs, and for the cells with four gates: LSTM D = 256 forward 0.944 -> 0.887 ms per 1024 steps, sLSTM
+// five share four SIMDs (heads of one workgroup of up to 8 waves, where every load is on the chain: the gated cells,
+// GRU B16 T2048 N4 D128 forward 0.915 -> 0.826 ms), and for the cells with four gates: LSTM D = 256 forward 0.944 -> 0.887 ms per 1024 steps, sLSTM
 // D = 192 0.961 -> 0.914; the GRU (three loads per step to save) measured +1.5 % to -0.8 %, Elman the same to 0.3 %.
 constexpr bool fwd_producer_wave(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize) {
+  if (KW == 1) return esize == 2 && GR >= 3 && TR == 4 && WAVES <= 8 && UTW == 1;  // (heads of one workgroup: every load is on the chain)
   return esize == 2 && GR == 4 && KW > 1 && TR <= 8 && WAVES == 4 && UTW * GR * (D / 32) * 4 <= (TR == 4 ? 160 : 128);
 }
 // Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
