@@ -98,7 +98,8 @@ template <> __device__ __forceinline__ float load_frag_at<float>(const float* p)
 // are rebuilt from the stored (rounded) m_(t-2); the larger of the two is still exactly 1, the other carries
 // the rounding error of m_(t-2) as a relative error (2^-9 |m| for bf16).
 template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool RC = false>
-__global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) {
+__global__ void __launch_bounds__((WAVES + (bwd_producer_wave(Cell<F>::GR, Cell<F>::NC, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC) ? 1 : 0)) * 64)
+fused_bwd_kernel(const BwdArgs a) {
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
@@ -172,6 +173,95 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
   const rsrc_t rDw = make_rsrc(a.dWx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rDx = make_rsrc(a.dgx, (size_t)B * Tn * ND * ES);
   const rsrc_t rWx = make_rsrc(a.Wx, RC ? (size_t)B * Tn * GW * ND * ES : 0);
+
+  // ---- the producer wave (see bwd_producer_wave): the workgroup's last wave.  It takes part in every barrier of the
+  //      compute waves, in the same order and under the same conditions (wave-uniform values that every wave reads from
+  //      LDS behind a barrier, and kernel arguments).  Iterations count the reverse steps: iteration i is step
+  //      T-1-i.  The operands of iteration j travel in register set j % 3; during iteration i the compute waves read
+  //      those of iteration i+1 from buffer (i+1) & 1 (behind the barrier of the step) and this wave writes those of
+  //      iteration i+2 into the other buffer and sends for those of iteration i+4 --------------------------------------
+  constexpr bool PW = bwd_producer_wave(GR, NC, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC);
+  // one buffer: [cache: tile][row][16 units][NCP values] [s_(t-1): state][tile][row][16 units] [cotangent: the same]
+  constexpr int PB_CA = NC > 0 ? UT_WG * TR * 16 * NCP : 0, PB_ST = S * UT_WG * TR * 16, PB = PB_CA + 2 * PB_ST;
+  static_assert(!PW || 2 * PB * (int)sizeof(T) + 16 == bwd_producer_bytes(NC, S, UT_WG, TR, (int)sizeof(T)), "hand-over buffer size");
+  T* const pbuf = reinterpret_cast<T*>(smem_raw + bwd_lds_bytes(GR, D, WAVES, UTW, KW, (int)sizeof(T)));
+  if constexpr (PW) {
+    if (w == WAVES) {
+      constexpr int CPR = NCP * 2;  // 16-byte pieces per (tile, batch row) of the cache
+      constexpr int CP_TOT = NC > 0 ? UT_WG * TR * CPR : 0, NPC = (CP_TOT + 63) / 64;
+      constexpr int SP_TOT = S * UT_WG * TR * 2, NPS = (SP_TOT + 63) / 64;  // pieces of 8 units of one state, tile and row
+      unsigned cvo[NPC > 0 ? NPC : 1], svo[NPS], s0o[NPS]; int cl[NPC > 0 ? NPC : 1], sl[NPS];
+#pragma unroll
+      for (int i = 0; i < NPC; ++i) {
+        const int c = lane + 64 * i, q = c % CPR, pr = (c / CPR) % TR, ptile = c / (CPR * TR);
+        const bool ok = c < CP_TOT && bt * TR + pr < B;
+        cvo[i] = ok ? ((((unsigned)(slice * UT_WG + ptile) * Bpad + bt * TR + pr) * 16) * NCP * ES + q * 16) : kInvalidOff;
+        cl[i] = c < CP_TOT ? ((ptile * TR + pr) * 16) * NCP + q * 8 : -1;
+      }
+#pragma unroll
+      for (int i = 0; i < NPS; ++i) {
+        const int c = lane + 64 * i, half = c & 1, pr = (c >> 1) % TR, ptile = ((c >> 1) / TR) % UT_WG, pk = (c >> 1) / (TR * UT_WG);
+        const bool ok = c < SP_TOT && bt * TR + pr < B;
+        const unsigned col = n * D + slice * DL + ptile * 16 + half * 8;
+        svo[i] = ok ? ((((unsigned)(pk * B + bt * TR + pr) * Tn) * ND + col) * ES) : kInvalidOff;   // + t * ND * ES
+        s0o[i] = ok ? (((unsigned)(pk * B + bt * TR + pr) * ND + col) * ES) : kInvalidOff;
+        sl[i] = c < SP_TOT ? ((pk * UT_WG + ptile) * TR + pr) * 16 + half * 8 : -1;
+      }
+      struct Ops { Dw<4> ca[NPC > 0 ? NPC : 1], sp[NPS], dso[NPS]; };
+      Ops set[3];
+      auto fetch = [&](Ops& o, int j) __attribute__((always_inline)) {
+        const int t = Tn - 1 - j > 0 ? Tn - 1 - j : 0;  // (beyond the last step: the operands of step 0 again, unused)
+        const bool first = t == 0;
+        const rsrc_t rPrev = first ? rS0 : rSt;
+#pragma unroll
+        for (int i = 0; i < NPC; ++i) o.ca[i] = buf_load<4>(rCa, cvo[i], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
+#pragma unroll
+        for (int i = 0; i < NPS; ++i) {
+          o.dso[i] = buf_load<4>(rDs, svo[i], (unsigned)t * ND * ES);
+          o.sp[i] = buf_load<4>(rPrev, first ? s0o[i] : svo[i], first ? 0u : (unsigned)(t - 1) * ND * ES);
+        }
+      };
+      // (no branch on the lane: behind one the compiler waits for every load in flight, the latest ones included;
+      // lanes without a piece write to the 16 spare bytes behind the buffers)
+      auto put = [&](const Ops& o, int j) __attribute__((always_inline)) {
+        T* const pb = pbuf + (j & 1) * PB;
+        T* const spare = pbuf + 2 * PB;
+#pragma unroll
+        for (int i = 0; i < NPC; ++i)
+          *reinterpret_cast<uint4*>(cl[i] >= 0 ? pb + cl[i] : spare) = make_uint4(o.ca[i].v[0], o.ca[i].v[1], o.ca[i].v[2], o.ca[i].v[3]);
+#pragma unroll
+        for (int i = 0; i < NPS; ++i) {
+          *reinterpret_cast<uint4*>(sl[i] >= 0 ? pb + PB_CA + sl[i] : spare) = make_uint4(o.sp[i].v[0], o.sp[i].v[1], o.sp[i].v[2], o.sp[i].v[3]);
+          *reinterpret_cast<uint4*>(sl[i] >= 0 ? pb + PB_CA + PB_ST + sl[i] : spare) = make_uint4(o.dso[i].v[0], o.dso[i].v[1], o.dso[i].v[2], o.dso[i].v[3]);
+        }
+      };
+      fetch(set[1], 1); fetch(set[2], 2); fetch(set[0], 3);
+      put(set[1], 1);
+      __syncthreads();  // (the one of the prologue below)
+      bool pdead = KW > 1 && __builtin_amdgcn_readfirstlane(near_word) < 0;
+      if (!a.cut) {
+        auto iter = [&](int i, const Ops& next, Ops& refill) __attribute__((always_inline)) {
+          if (barrier_or(false, dead_flag)) { pdead = true; return; }
+          put(next, i + 2);
+          fetch(refill, i + 4);
+        };
+        int i = 0;
+        for (; i + 2 < Tn && !pdead; i += 3) {
+          iter(i, set[2], set[1]);
+          if (pdead) break;
+          iter(i + 1, set[0], set[2]);
+          if (pdead) break;
+          iter(i + 2, set[1], set[0]);
+        }
+        if (!pdead && i < Tn) {
+          iter(i, set[2], set[1]);
+          if (!pdead && i + 1 < Tn) iter(i + 1, set[0], set[2]);
+        }
+      }
+      if (!pdead) barrier_or(false, dead_flag);  // (the one behind the time loop)
+      return;
+    }
+  }
 
   int ub[UTW];
   unsigned wx_v[UTW], st_v[UTW], s0_v[UTW], ca_v[UTW];
@@ -349,7 +439,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
 #ifdef FRNN_PD
   constexpr int PD = RC ? 2 : KW == 1 ? FRNN_PD : 1;
 #else
-  constexpr int PD = RC ? 2 : KW > 1 || WAVES >= 8 ? 1 : 3;  // measured: with 8 waves and more, other waves hide the fetch
+  constexpr int PD = RC ? 2 : KW > 1 || WAVES >= 8 || PW ? 1 : 3;  // measured: with 8 waves and more, other waves hide the fetch
 #endif
   Pre pre[PD + 1];
   auto load_pre = [&](Pre& p, int t) __attribute__((always_inline)) {
@@ -499,7 +589,7 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     FRNN_STAMP(c0);
     // (readfirstlane: the compiler otherwise forms max(t - PD, 0) with a saturating VALU subtract
     // and then wraps a buffer load that uses it as a scalar offset into a waterfall loop)
-    load_pre(pn, __builtin_amdgcn_readfirstlane(t >= PD ? t - PD : 0));
+    if constexpr (!(PW && !cut)) load_pre(pn, __builtin_amdgcn_readfirstlane(t >= PD ? t - PD : 0));
     // dWx_t (and the GRU's g-gate cotangent).  With an exchange the stores are issued after the
     // partial sums are sent, where they fill the wait for the other workgroups instead of delaying
     // the barrier (a vector memory instruction costs ~30 cycles to issue)
@@ -576,6 +666,25 @@ __global__ void __launch_bounds__(WAVES * 64) fused_bwd_kernel(const BwdArgs a) 
     // the barrier also spreads a failed wait of the previous step to the whole workgroup
     if (barrier_or(fail, dead_flag)) { dead = true; return; }
     FRNN_STAMP(c2);
+    if constexpr (PW) {
+      // the operands of step t-1 from the producer wave's buffer (behind this step's barrier; used in the next step)
+      static_assert(E == 1 && ND_ == 1 && PD == 1, "4-row tiles: one element per lane and tile, one step ahead");
+      const T* const pb = pbuf + ((Tn - t) & 1) * PB;
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) {
+        const int el = ((w * UTW + u) * TR + brow) * 16 + esub;
+        if constexpr (NC > 0) {
+          const unsigned* const pc_ = reinterpret_cast<const unsigned*>(pb) + el * NWC;
+#pragma unroll
+          for (int i = 0; i < NWC; ++i) pn.cache[u].v[i] = pc_[i];
+        }
+#pragma unroll
+        for (int k = 0; k < S; ++k) {
+          pn.sp[u][k].v[0] = reinterpret_cast<const unsigned short*>(pb + PB_CA)[k * UT_WG * TR * 16 + el];
+          pn.dso[u][k].v[0] = reinterpret_cast<const unsigned short*>(pb + PB_CA + PB_ST)[k * UT_WG * TR * 16 + el];
+        }
+      }
+    }
 
     // one accumulator per tile: splitting a lone chain over several accumulators (as the forward
     // kernel does) measured 3-8 % slower here, before and after the barrier was made LDS-only

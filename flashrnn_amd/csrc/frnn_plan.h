@@ -56,6 +56,22 @@ constexpr bool fwd_producer_wave(int GR, int D, int WAVES, int UTW, int KW, int 
   if (KW == 1) return esize == 2 && GR >= 3 && TR == 4 && WAVES <= 8 && UTW == 1;  // (heads of one workgroup: every load is on the chain)
   return esize == 2 && GR == 4 && KW > 1 && TR <= 8 && WAVES == 4 && UTW * GR * (D / 32) * 4 <= (TR == 4 ? 160 : 128);
 }
+// Backward kernel: the same producer wave for the operands of a step (gate cache, s_(t-1), the cotangent of the
+// states), for the heads that run as one workgroup: there every load of the compute waves is on the chain of dependent
+// steps, and a step (~1600 cycles) is shorter than a fetch from HBM, which their one-step prefetch therefore waits for
+// (a timing-only build without these loads runs GRU D = 128 backward 35 % faster).  The producer wave loads four steps
+// ahead and leaves the operands of the next step in LDS.  Not in recompute mode, and not for truncated backpropagation
+// (no barrier per step to hand over at: that variant of the step keeps its own loads).
+constexpr bool bwd_producer_wave(int GR, int nc, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
+  // (nc = 5, the sLSTM: its 8-wave kernel spills at the 170 registers that nine waves leave each)
+  return esize == 2 && !rc && GR >= 3 && KW == 1 && TR == 4 && (WAVES <= 6 || (WAVES <= 8 && nc <= 4)) && UTW == 1;
+}
+// LDS bytes of the hand-over buffers of that wave (two steps): the gate cache (nc values per element, padded to an even
+// number), s_(t-1) and the cotangent (s states each) of the workgroup's UT_WG tiles of TR rows x 16 units, and 16
+// spare bytes
+constexpr int bwd_producer_bytes(int nc, int s, int ut_wg, int TR, int esize) {
+  return 2 * ut_wg * TR * 16 * ((nc + 1) / 2 * 2 + 2 * s) * esize + 16;
+}
 // Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
 // 2..16 workgroups (up to 12 where part of the operand lives in LDS) whose slice is a whole number of k-steps; not the fp32
 // kernels whose operand alone takes 256 registers, at the tile heights where they keep 2 or 4 elements per lane

@@ -18,7 +18,10 @@ template <>
 int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream_t st) {
   const dim3 grid(grid_for(a.groups, p.kw));
   const bool rc = p.recompute != 0;
-  const size_t lds = bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T), rc) + 16;
+  // (one more wave and its hand-over buffers where the kernel has a producer wave: the same predicate as in the kernel)
+  const bool pw = bwd_producer_wave(Cell<FRNN_F>::GR, Cell<FRNN_F>::NC, p.D, p.waves, p.utw, p.kw, a.tile_rows, (int)sizeof(FRNN_TU_T), rc);
+  const size_t lds = bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T), rc) + 16 +
+                     (pw ? bwd_producer_bytes(Cell<FRNN_F>::NC, Cell<FRNN_F>::S, p.waves * p.utw, a.tile_rows, (int)sizeof(FRNN_TU_T)) : 0);
 #define FRNN_CASE_(RCV, Dv, VAR, W, U, K, MTR)                                                          \
   if (rc == RCV && p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                               \
     auto kern = bwd_kernel_for<Dv, W, U, K, MTR, RCV>(a.tile_rows);                                      \
@@ -30,9 +33,9 @@ int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream
     if (K > 1 && p.cooperative) { /* see fused_fwd_tu.hip */                                             \
       BwdArgs aa = a;                                                                                    \
       void* args[] = {(void*)&aa};                                                                       \
-      return (int)hipLaunchCooperativeKernel((const void*)kern, grid, dim3(W * 64), args, lds, st);      \
+      return (int)hipLaunchCooperativeKernel((const void*)kern, grid, dim3((W + (pw ? 1 : 0)) * 64), args, lds, st);      \
     }                                                                                                    \
-    hipLaunchKernelGGL(kern, grid, dim3(W * 64), lds, st, a);                                            \
+    hipLaunchKernelGGL(kern, grid, dim3((W + (pw ? 1 : 0)) * 64), lds, st, a);                                            \
     return (int)hipGetLastError();                                                                       \
   }
 #define FRNN_CASE(Dv, VAR, W, U, K, MTR) FRNN_CASE_(false, Dv, VAR, W, U, K, MTR)
