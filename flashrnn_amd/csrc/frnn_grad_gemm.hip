@@ -41,9 +41,26 @@ int launch_transpose_r(int dtype, const void* R, void* Rt, int N, int D, int GR,
 // dR GEMM.  Workgroup tile TM (units d of one gate) x TM (previous units p), 4 waves in 2 x 2,
 // 32 rows (b,t) per LDS stage; grid (tiles, N, splits).
 // ---------------------------------------------------------------------------------------------
-__device__ __forceinline__ void gemm_tile_of(const GradGemmArgs& a, int TM, int& g, int& dt, int& pt) {
+// Which tile of which (head, split) a workgroup computes.  All tiles of one (head, split) read the same rows of h, and
+// the tiles of one gate row the same rows of dG, so they should run at the same time behind the same L2: the device hands
+// consecutive workgroups to its 8 XCDs in turn (each with an L2 of its own), so the workgroups of one XCD, every 8th in
+// launch order, take the tiles of one (head, split) after another.  Without this each of the 4 gate tiles of LSTM D = 64
+// and D = 256 ran on an XCD of its own and h came from HBM four times (3.2 GB per launch instead of 2.0 at B = 256,
+// T = 1024).  The last (head, split) pairs, less than 8, keep the plain order.
+__device__ __forceinline__ void gemm_tile_of(const GradGemmArgs& a, int TM, int& g, int& dt, int& pt, int& n, int& split) {
   const int tiles = a.D / TM;
-  int tile = blockIdx.x;
+  const int per_pair = gridDim.x, pairs = gridDim.y * gridDim.z;
+  const int lin = blockIdx.x + per_pair * (blockIdx.y + gridDim.y * blockIdx.z);
+  int tile, pair;
+  if (lin < (pairs / 8) * 8 * per_pair) {
+    const int j = lin / 8;
+    tile = j % per_pair;
+    pair = (j / per_pair) * 8 + lin % 8;
+  } else {
+    tile = lin % per_pair;
+    pair = lin / per_pair;
+  }
+  n = pair % a.N; split = pair / a.N;
   pt = tile % tiles; tile /= tiles;
   dt = tile % tiles;
   g = tile / tiles;
@@ -98,8 +115,8 @@ __global__ void __launch_bounds__(64 * WD * WD) grad_gemm16_kernel(const GradGem
   lds_byte* const sm = (lds_byte*)gemm_smem;
 
   int g, dt, pt;
-  gemm_tile_of(a, TM, g, dt, pt);
-  const int n = blockIdx.y, split = blockIdx.z;
+  int n, split;
+  gemm_tile_of(a, TM, g, dt, pt, n, split);
   const int tid = threadIdx.x, lane = tid & 63, w = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int wm = w / WD, wn = w % WD;
   const int r16 = lane & 15, q4 = lane >> 4;
@@ -255,8 +272,8 @@ __global__ void __launch_bounds__(256) grad_gemm32_kernel(const GradGemmArgs a) 
   __shared__ __attribute__((aligned(16))) GemmStage32<TM> sm;
 
   int g, dt, pt;
-  gemm_tile_of(a, TM, g, dt, pt);
-  const int n = blockIdx.y, split = blockIdx.z;
+  int n, split;
+  gemm_tile_of(a, TM, g, dt, pt, n, split);
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int wm = w >> 1, wn = w & 1;
   const int r16 = lane & 15, q4 = lane >> 4;
