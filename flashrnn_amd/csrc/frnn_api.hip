@@ -188,13 +188,15 @@ static bool pick_plan(int function, int dtype, int B, int N, int D, int backward
 // words to poll per step (the larger costs of a step) at the price of more workgroups and copies
 // of R, so the smallest tile is used for which every workgroup of the call still gets a compute
 // unit of its own.  Heads that run as one small workgroup (up to 4 waves, no exchange) may share a
-// compute unit three at a time: one workgroup's gate math then runs while another waits for memory
-// (measured at B = 128..256: LSTM D = 32 2.74 -> 2.17 ms, D = 64 3.72 -> 3.35; not so with 8 waves).
+// compute unit four at a time (eight of up to 2 waves): one workgroup's gate math then runs while another
+// waits for memory, and only the 4-row kernels have the producer wave (measured, LSTM bf16 T = 1024, 4-row
+// against 8-row tiles: B = 340 N = 12 D = 64, 1020 workgroups, 4.07 against 4.80 ms; B = 336 N = 24 D = 32,
+// 2016 workgroups, 4.63 against 4.98; with 8 waves, D = 128, a gain for the LSTM and a loss for the GRU).
 // `largest` is the tallest tile the tiling is compiled for (Plan::max_tr: taller ones would spill registers).
 static int tile_rows_for(int B, int N, int kw, int waves, int largest) {
   const int forced = env_int("FRNN_TILE_ROWS", 0);
   if (forced == 4 || forced == 8 || forced == 16) return forced < largest ? forced : largest;
-  const long room = kw > 1 ? groups_per_launch(kw) : (long)device_cus() * (waves <= 4 ? 3 : 1);
+  const long room = kw > 1 ? groups_per_launch(kw) : (long)device_cus() * (waves <= 2 ? 8 : waves <= 4 ? 4 : 1);
   for (int tr = 4; tr < largest; tr *= 2)
     if ((long)N * ((B + tr - 1) / tr) <= room) return tr;
   return largest;

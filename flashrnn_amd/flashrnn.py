@@ -453,7 +453,7 @@ _FUSED_TENSOR_LIMIT = 1 << 31  # the fused kernels address each tensor with 32-b
 def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     """Batch rows are independent, so a fused problem one of whose tensors (Wx, the states or the gate cache)
     would reach 2 GiB runs as several calls over ranges of the batch; autograd sums dR and db over the ranges.
-    Wx[b0:b1] is a view (the batch is its leading axis); the outputs of the ranges are concatenated."""
+    A range of Wx is a view (the batch is its leading axis); the outputs of the ranges are concatenated."""
     B, T, Gw, N, D = Wx.shape
     if config.backend != "hip_fused":
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
@@ -465,8 +465,10 @@ def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     if rows >= B:
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
     rows = max(16, rows // 16 * 16) if rows >= 16 else rows  # whole batch tiles
-    outs = [_FlashRNNFunction.apply(Wx[b0:b0 + rows], R, b, states[:, b0:b0 + rows], config, training)
-            for b0 in range(0, B, rows)]
+    # (split, not slices: its backward is one concatenation of the ranges' gradients, where every slice's backward
+    # would fill a zero tensor of the full size and autograd would then add those up)
+    outs = [_FlashRNNFunction.apply(wx_r, R, b, st_r, config, training)
+            for wx_r, st_r in zip(torch.split(Wx, rows, dim=0), torch.split(states, rows, dim=1))]
     return torch.cat(outs, dim=1)
 
 
