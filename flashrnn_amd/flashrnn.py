@@ -465,6 +465,9 @@ def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     if rows >= B:
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
     rows = max(16, rows // 16 * 16) if rows >= 16 else rows  # whole batch tiles
+    if rows >= 16:  # ranges of about the same size, still whole tiles
+        n_ranges = -(-B // rows)
+        rows = min(rows, -(-B // (16 * n_ranges)) * 16)
     # (split, not slices: its backward is one concatenation of the ranges' gradients, where every slice's backward
     # would fill a zero tensor of the full size and autograd would then add those up)
     outs = [_FlashRNNFunction.apply(wx_r, R, b, st_r, config, training)
