@@ -278,6 +278,84 @@ def fused_plan(function: str, dtype: str, B: int, N: int, D: int, backward: bool
     return tuple(o.value for o in out)
 
 
+def _cast_inputs(Wx, R, b, s0, cfg: FlashRNNConfig):
+    """The inputs in the kernel type and the kernels' layouts, as the reference's custom_fwd(cast_inputs=...) does
+    (flashrnn.py:690-695); s0 comes back as [S,B,N,D]."""
+    kdt = DTYPE_DICT[cfg.dtype]
+    if not cfg.enable_automatic_mixed_precision:
+        for name, x in (("Wx", Wx), ("R", R), ("b", b), ("states", s0)):
+            if x.dtype != kdt:
+                raise TypeError(f"{name} is {x.dtype}, the kernel type is {kdt} and "
+                                "enable_automatic_mixed_precision is off")
+    S, B = cfg.num_states, Wx.shape[0]
+    N, D = Wx.shape[3], Wx.shape[4]
+    return (Wx.detach().to(kdt).contiguous(), R.detach().to(kdt).contiguous(), b.detach().to(kdt).contiguous(),
+            s0.detach().to(kdt).reshape(S, B, N, D).contiguous())
+
+
+def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
+    """One forward call of the library on kernel-typed, contiguous tensors: (states [S,B,T,N,D], gate cache)."""
+    kdt = DTYPE_DICT[cfg.dtype]
+    f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
+    B, T, Gw, N, D = Wx_k.shape
+    S = cfg.num_states
+    with _on_device(Wx_k.device):
+        rc = _entry(cfg.backend, "supported")(f_id, d_id, B, N, D)
+        if rc == 0 and cfg.recompute_gates:
+            if cfg.backend != "hip_fused":
+                raise ValueError("recompute_gates is an option of the hip_fused backend")
+            rc = _lib.load_library().frnn_fused_recompute_supported(f_id, d_id, B, N, D)
+        if rc != 0:
+            _raise(rc, f"{cfg.backend} backend")
+        states = torch.empty((S, B, T, N, D), dtype=kdt, device=Wx_k.device)
+        cache_bytes = _entry(cfg.backend, "cache_bytes_opt")(f_id, d_id, B, T, N, D, _options(cfg)) if training else 0
+        cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx_k.device)
+        ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 0)
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx_k.device)
+        stream = _raw_stream(Wx_k.device)
+        rc = _entry(cfg.backend, "forward_opt")(
+            f_id, d_id, int(training), B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(),
+            s0_k.data_ptr(), states.data_ptr(), cache.data_ptr() if training else None,
+            ws.data_ptr(), ws.numel(), stream, _options(cfg))
+        if rc != 0:
+            _raise(rc, f"{cfg.backend} forward")
+        if cfg.backend == "hip_fused":
+            _status.log("forward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+    return states, cache
+
+
+def _run_backward(cfg: FlashRNNConfig, R_k, b_k, s0_k, states, cache, Wx_k, ds, dWx):
+    """One backward call of the library; ds [S,B,T,N,D] contiguous in the kernel type, dWx [B,T,G_w,N,D] is written.
+    Returns (dR, db, ds0 [S,B,N,D]); dR and db are fp32."""
+    kdt = DTYPE_DICT[cfg.dtype]
+    f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
+    S, B, T, N, D = states.shape
+    Gr, Gt = cfg.num_gates_r, cfg.num_gates_t
+    dev = states.device
+    with _on_device(dev):
+        ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
+        dR = torch.empty((Gr, N, D, D), dtype=torch.float32, device=dev)
+        db = torch.empty((Gt, N, D), dtype=torch.float32, device=dev)
+        ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 1)
+        ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
+        stream = _raw_stream(dev)
+        if cfg.recompute_gates:
+            rc = _lib.load_library().frnn_fused_backward_recompute(
+                f_id, d_id, B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(),
+                states.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
+                ws.data_ptr(), ws.numel(), stream, _options(cfg))
+        else:
+            rc = _entry(cfg.backend, "backward_opt")(
+                f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
+                cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
+                ws.data_ptr(), ws.numel(), stream, _options(cfg))
+        if rc != 0:
+            _raise(rc, f"{cfg.backend} backward")
+        if cfg.backend == "hip_fused":
+            _status.log("backward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+    return dR, db, ds0
+
+
 class _FlashRNNFunction(torch.autograd.Function):
     """forward(Wx [B,T,G_w,N,D], R [G_r,N,D,D], b [G_t,N,D], s0 [S,B,1,N,D]) -> states [S,B,T,N,D]."""
 
@@ -285,45 +363,10 @@ class _FlashRNNFunction(torch.autograd.Function):
     def forward(ctx, Wx, R, b, s0, cfg: FlashRNNConfig, training: bool):
         if not Wx.is_cuda:
             raise RuntimeError("flashrnn_amd runs on a GPU only (got a CPU tensor); there is no CPU fallback")
-        kdt = DTYPE_DICT[cfg.dtype]
-        f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
-        B, T, Gw, N, D = Wx.shape
-        S = cfg.num_states
         _status.poll()
-        if not cfg.enable_automatic_mixed_precision:
-            for name, x in (("Wx", Wx), ("R", R), ("b", b), ("states", s0)):
-                if x.dtype != kdt:
-                    raise TypeError(f"{name} is {x.dtype}, the kernel type is {kdt} and "
-                                    "enable_automatic_mixed_precision is off")
-        # cast to the kernel type as the reference's custom_fwd(cast_inputs=...) does (:690-695)
-        Wx_k = Wx.detach().to(kdt).contiguous()
-        R_k = R.detach().to(kdt).contiguous()
-        b_k = b.detach().to(kdt).contiguous()
-        s0_k = s0.detach().to(kdt).reshape(S, B, N, D).contiguous()
-        with _on_device(Wx.device):
-            rc = _entry(cfg.backend, "supported")(f_id, d_id, B, N, D)
-            if rc == 0 and cfg.recompute_gates:
-                if cfg.backend != "hip_fused":
-                    raise ValueError("recompute_gates is an option of the hip_fused backend")
-                rc = _lib.load_library().frnn_fused_recompute_supported(f_id, d_id, B, N, D)
-            if rc != 0:
-                _raise(rc, f"{cfg.backend} backend")
-            states = torch.empty((S, B, T, N, D), dtype=kdt, device=Wx.device)
-            cache_bytes = _entry(cfg.backend, "cache_bytes_opt")(f_id, d_id, B, T, N, D, _options(cfg)) if training else 0
-            cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx.device)
-            ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 0)
-            ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=Wx.device)
-            stream = _raw_stream(Wx.device)
-            rc = _entry(cfg.backend, "forward_opt")(
-                f_id, d_id, int(training), B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(),
-                s0_k.data_ptr(), states.data_ptr(), cache.data_ptr() if training else None,
-                ws.data_ptr(), ws.numel(), stream, _options(cfg))
-            if rc != 0:
-                _raise(rc, f"{cfg.backend} forward")
-            if cfg.backend == "hip_fused":
-                _status.log("forward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+        Wx_k, R_k, b_k, s0_k = _cast_inputs(Wx, R, b, s0, cfg)
+        states, cache = _run_forward(Wx_k, R_k, b_k, s0_k, cfg, training)
         ctx.cfg, ctx.training = cfg, training
-        ctx.dims = (B, T, N, D)
         # (recompute mode reads Wx again in the backward pass; it is the caller's tensor unless it was cast)
         ctx.save_for_backward(R_k, b_k, s0_k, states, cache, Wx_k if cfg.recompute_gates else cache)
         return states
@@ -335,38 +378,69 @@ class _FlashRNNFunction(torch.autograd.Function):
             raise RuntimeError("FlashRNN backward can only be called in training mode")
         cfg = ctx.cfg
         R_k, b_k, s0_k, states, cache, Wx_k = ctx.saved_tensors
-        kdt = DTYPE_DICT[cfg.dtype]
-        f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
-        B, T, N, D = ctx.dims
-        S, Gw, Gr, Gt = cfg.num_states, cfg.num_gates_w, cfg.num_gates_r, cfg.num_gates_t
-        dev = states.device
+        S, B, T, N, D = states.shape
         _status.poll()
-        ds = dstates.to(kdt).contiguous()
-        with _on_device(dev):
-            dWx = torch.empty((B, T, Gw, N, D), dtype=kdt, device=dev)
-            ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
-            dR = torch.empty((Gr, N, D, D), dtype=torch.float32, device=dev)
-            db = torch.empty((Gt, N, D), dtype=torch.float32, device=dev)
-            ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 1)
-            ws = torch.empty(max(ws_bytes, 256), dtype=torch.uint8, device=dev)
-            stream = _raw_stream(dev)
-            if cfg.recompute_gates:
-                rc = _lib.load_library().frnn_fused_backward_recompute(
-                    f_id, d_id, B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(),
-                    states.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
-                    ws.data_ptr(), ws.numel(), stream, _options(cfg))
-            else:
-                rc = _entry(cfg.backend, "backward_opt")(
-                    f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
-                    cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
-                    ws.data_ptr(), ws.numel(), stream, _options(cfg))
-            if rc != 0:
-                _raise(rc, f"{cfg.backend} backward")
-            if cfg.backend == "hip_fused":
-                _status.log("backward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+        ds = dstates.to(states.dtype).contiguous()
+        with _on_device(states.device):
+            dWx = torch.empty((B, T, cfg.num_gates_w, N, D), dtype=states.dtype, device=states.device)
+        dR, db, ds0 = _run_backward(cfg, R_k, b_k, s0_k, states, cache, Wx_k, ds, dWx)
         # dR / db stay fp32: autograd casts them to the dtype of the leaf they belong to, so fp32
         # master weights receive unrounded gradients
         return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None
+
+
+class _FlashRNNRangesFunction(torch.autograd.Function):
+    """The same over ranges of `rows` batch rows, one library call each (see _apply_in_batch_ranges).  A range of Wx
+    and of dWx is contiguous (the batch is their leading axis), so the calls read and write the full tensors in
+    place; the state tensors [S,B,...] are copied range by range."""
+
+    @staticmethod
+    def forward(ctx, Wx, R, b, s0, cfg: FlashRNNConfig, training: bool, rows: int):
+        if not Wx.is_cuda:
+            raise RuntimeError("flashrnn_amd runs on a GPU only (got a CPU tensor); there is no CPU fallback")
+        _status.poll()
+        Wx_k, R_k, b_k, s0_k = _cast_inputs(Wx, R, b, s0, cfg)
+        B, T, _, N, D = Wx_k.shape
+        S = cfg.num_states
+        with _on_device(Wx_k.device):
+            states = torch.empty((S, B, T, N, D), dtype=Wx_k.dtype, device=Wx_k.device)
+        saved = []
+        for b0 in range(0, B, rows):
+            b1 = min(B, b0 + rows)
+            s0_r = s0_k[:, b0:b1].contiguous()
+            states_r, cache_r = _run_forward(Wx_k[b0:b1], R_k, b_k, s0_r, cfg, training)
+            states[:, b0:b1].copy_(states_r)
+            saved += [s0_r, states_r, cache_r]
+        ctx.cfg, ctx.training, ctx.rows = cfg, training, rows
+        ctx.save_for_backward(R_k, b_k, Wx_k if cfg.recompute_gates else R_k, *saved)
+        return states
+
+    @staticmethod
+    @torch.autograd.function.once_differentiable
+    def backward(ctx, dstates):
+        if not ctx.training:
+            raise RuntimeError("FlashRNN backward can only be called in training mode")
+        cfg, rows = ctx.cfg, ctx.rows
+        R_k, b_k, Wx_k, *saved = ctx.saved_tensors
+        S, _, T, N, D = dstates.shape
+        B = sum(saved[3 * i].shape[1] for i in range(len(saved) // 3))
+        kdt = DTYPE_DICT[cfg.dtype]
+        _status.poll()
+        ds = dstates.to(kdt)
+        with _on_device(dstates.device):
+            dWx = torch.empty((B, T, cfg.num_gates_w, N, D), dtype=kdt, device=dstates.device)
+            ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dstates.device)
+        dR = db = None
+        for i, b0 in enumerate(range(0, B, rows)):
+            b1 = min(B, b0 + rows)
+            s0_r, states_r, cache_r = saved[3 * i:3 * i + 3]
+            wx_r = Wx_k[b0:b1] if cfg.recompute_gates else Wx_k
+            dR_r, db_r, ds0_r = _run_backward(cfg, R_k, b_k, s0_r, states_r, cache_r, wx_r,
+                                              ds[:, b0:b1].contiguous(), dWx[b0:b1])
+            ds0[:, b0:b1].copy_(ds0_r)
+            dR = dR_r if dR is None else dR.add_(dR_r)
+            db = db_r if db is None else db.add_(db_r)
+        return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None, None
 
 
 def _get_config(Wx, R, b, function, backend, dtype) -> FlashRNNConfig:
@@ -452,8 +526,8 @@ _FUSED_TENSOR_LIMIT = 1 << 31  # the fused kernels address each tensor with 32-b
 
 def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     """Batch rows are independent, so a fused problem one of whose tensors (Wx, the states or the gate cache)
-    would reach 2 GiB runs as several calls over ranges of the batch; autograd sums dR and db over the ranges.
-    A range of Wx is a view (the batch is its leading axis); the outputs of the ranges are concatenated."""
+    would reach 2 GiB runs as several library calls over ranges of the batch (_FlashRNNRangesFunction), dR and db
+    summed over the ranges."""
     B, T, Gw, N, D = Wx.shape
     if config.backend != "hip_fused":
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
@@ -468,11 +542,7 @@ def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     if rows >= 16:  # ranges of about the same size, still whole tiles
         n_ranges = -(-B // rows)
         rows = min(rows, -(-B // (16 * n_ranges)) * 16)
-    # (split, not slices: its backward is one concatenation of the ranges' gradients, where every slice's backward
-    # would fill a zero tensor of the full size and autograd would then add those up)
-    outs = [_FlashRNNFunction.apply(wx_r, R, b, st_r, config, training)
-            for wx_r, st_r in zip(torch.split(Wx, rows, dim=0), torch.split(states, rows, dim=1))]
-    return torch.cat(outs, dim=1)
+    return _FlashRNNRangesFunction.apply(Wx, R, b, states, config, training, rows)
 
 
 def flashrnn_step(
