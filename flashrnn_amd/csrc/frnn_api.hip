@@ -527,10 +527,12 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   FusedFwdWs w = carve_fused_fwd(workspace, dtype, B, N, D, p);
   if (!step) {
     if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
-    prof_begin("fill_zero_kernel", st);
-    e = launch_fill_zero(workspace, w.zero_bytes, st);
-    prof_end(st);
-    if (e) return hip_fail(e, "workspace clear");
+    if (p.kw > 1) {  // (a head of one workgroup has no exchange words, and its kernel sets the status word itself)
+      prof_begin("fill_zero_kernel", st);
+      e = launch_fill_zero(workspace, w.zero_bytes, st);
+      prof_end(st);
+      if (e) return hip_fail(e, "workspace clear");
+    }
   } else {
     const size_t one_group = 256 + (p.kw > 1 ? (size_t)3 * 16 * D / (dtype == FRNN_F32 ? 1 : 2) * 8 + 256 : 0);
     if (workspace_bytes < one_group) return fail(FRNN_E_WORKSPACE, "step scratch %zu < %zu bytes", workspace_bytes, one_group);
@@ -643,10 +645,12 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   const FusedBwdWs w = carve_fused_bwd(workspace, fx, dtype, B, T, N, D, p);
   if (workspace_bytes < w.total) return fail(FRNN_E_WORKSPACE, "workspace %zu < %zu bytes", workspace_bytes, w.total);
   hipStream_t st = (hipStream_t)stream;
-  prof_begin("fill_zero_kernel", st);
-  e = launch_fill_zero(workspace, w.zero_bytes, st);
-  prof_end(st);
-  if (e) return hip_fail(e, "workspace clear");
+  if (p.kw > 1) {  // (as in the forward call)
+    prof_begin("fill_zero_kernel", st);
+    e = launch_fill_zero(workspace, w.zero_bytes, st);
+    prof_end(st);
+    if (e) return hip_fail(e, "workspace clear");
+  }
   prof_begin("transpose_r_kernel", st);
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   prof_end(st);

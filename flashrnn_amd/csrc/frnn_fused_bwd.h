@@ -388,6 +388,8 @@ fused_bwd_kernel(const BwdArgs a) {
     for (int idx = tid; idx < (2 * 16 * D * (int)sizeof(T)) / 4; idx += NT) reinterpret_cast<unsigned*>(hb0)[idx] = 0u;
   }
   if (tid == 0) dead_flag_word = 0;
+  // (as in the forward kernel: the status word of a call whose workgroups never wait is set here, not by a clearing kernel)
+  if constexpr (KW == 1) { if (blockIdx.x == 0 && tid == 0) *a.status = 0; }
 
   float ds[UTW][E][S];
   float dbacc[UTW][E][GT];

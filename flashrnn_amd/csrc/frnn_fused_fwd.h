@@ -128,6 +128,9 @@ fused_fwd_kernel(const FwdArgs a) {
   const T* __restrict__ s0 = static_cast<const T*>(a.s0);
   const unsigned ND = (unsigned)N * D;
   if (tid == 0) dead_flag = 0;
+  // (a head of one workgroup never waits, so nothing else writes its call's status word: the host launches no clearing
+  // kernel for such a call and the word is set here)
+  if constexpr (KW == 1) { if (blockIdx.x == 0 && tid == 0) *a.status = 0; }
 
   const rsrc_t rWx = make_rsrc(a.Wx, (size_t)B * Tn * GW * ND * ES);
   const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
