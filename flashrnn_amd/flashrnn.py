@@ -12,6 +12,7 @@ for the backward pass (:746) or slice dWx (:789-796).
 """
 from __future__ import annotations
 
+import functools
 import os
 from dataclasses import dataclass
 from typing import Optional, Sequence, Union
@@ -217,6 +218,11 @@ class _StatusLog:
             self._pending.append(entry)
             self._last[kind] = entry
 
+    def note_ok(self, kind: str):
+        """A call that cannot fail this way (heads of one workgroup: nothing waits): nothing to fetch."""
+        with self._lock:
+            self._last[kind] = None
+
     def poll(self, wait: bool = False):
         if torch.cuda.is_current_stream_capturing():
             return  # (querying an event is not allowed while this thread captures)
@@ -278,6 +284,20 @@ def fused_plan(function: str, dtype: str, B: int, N: int, D: int, backward: bool
     return tuple(o.value for o in out)
 
 
+@functools.lru_cache(maxsize=None)
+def _heads_wait_cached(function: str, dtype: str, B: int, N: int, D: int, backward: bool, variant) -> bool:
+    return fused_plan(function, dtype, B, N, D, backward)[2] > 1
+
+
+def _heads_wait(cfg: FlashRNNConfig, B: int, N: int, D: int, backward: bool) -> bool:
+    """Whether the heads of this fused call run as several workgroups that wait for each other: only then can the
+    status word of the call become non-zero, and only then is it fetched (a copy on the stream per call).  The
+    recompute-mode reverse kernels have tilings of their own, so their calls always fetch it."""
+    if cfg.recompute_gates and backward:
+        return True
+    return _heads_wait_cached(cfg.function, cfg.dtype, B, N, D, backward, os.environ.get("FRNN_FUSED_VARIANT"))
+
+
 def _cast_inputs(Wx, R, b, s0, cfg: FlashRNNConfig):
     """The inputs in the kernel type and the kernels' layouts, as the reference's custom_fwd(cast_inputs=...) does
     (flashrnn.py:690-695); s0 comes back as [S,B,N,D]."""
@@ -320,7 +340,10 @@ def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
         if rc != 0:
             _raise(rc, f"{cfg.backend} forward")
         if cfg.backend == "hip_fused":
-            _status.log("forward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+            if _heads_wait(cfg, B, N, D, False):
+                _status.log("forward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+            else:
+                _status.note_ok("forward")
     return states, cache
 
 
@@ -352,7 +375,10 @@ def _run_backward(cfg: FlashRNNConfig, R_k, b_k, s0_k, states, cache, Wx_k, ds, 
         if rc != 0:
             _raise(rc, f"{cfg.backend} backward")
         if cfg.backend == "hip_fused":
-            _status.log("backward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+            if _heads_wait(cfg, B, N, D, True):
+                _status.log("backward", ws, f"{cfg.function} B{B} T{T} N{N} D{D}")
+            else:
+                _status.note_ok("backward")
     return dR, db, ds0
 
 
