@@ -87,13 +87,6 @@ def make_gpu_inputs(w, device):
     return inp, dev
 
 
-def _launches_per_step(w, backend):
-    """Profile entries one step produces (see the prof_begin calls of the C library)."""
-    if backend == "hip_fused":
-        return 2 + (5 if w["bwd"] else 0)
-    return 1 + (5 if w["bwd"] else 0)
-
-
 def run_gpu(w, backend, steps, warmup, device, recompute=False):
     """Returns (ms_per_step, {kernel name: (avg ms, launches per step)})."""
     import torch
@@ -115,6 +108,12 @@ def run_gpu(w, backend, steps, warmup, device, recompute=False):
     for _ in range(warmup):
         step()
     torch.cuda.synchronize()
+    # profile entries that one step produces (it depends on the tiling: heads of one workgroup have no clearing launch)
+    lib.frnn_profile_enable(1)
+    step()
+    torch.cuda.synchronize()
+    entries_per_step = max(1, lib.frnn_profile_count())
+    lib.frnn_profile_enable(0)
     # HIP events around every kernel launch, recorded on the launch stream inside the timed
     # region; the library keeps the most recent 64 launches, read after the region ends
     lib.frnn_profile_enable(1)
@@ -128,7 +127,7 @@ def run_gpu(w, backend, steps, warmup, device, recompute=False):
     for i in range(held):
         per_kernel.setdefault(lib.frnn_profile_name(i).decode(), []).append(lib.frnn_profile_ms(i))
     lib.frnn_profile_enable(0)
-    calls = max(1, min(steps, held // max(1, _launches_per_step(w, backend))))
+    calls = max(1, min(steps, held // entries_per_step))
     kern = {k: (sum(v) / len(v), max(1, round(len(v) / calls))) for k, v in per_kernel.items()}
     return (t1 - t0) * 1e3 / steps, kern
 
