@@ -279,3 +279,13 @@ def test_slstm_mixed_fresh_and_running_elements(gpu):
         for k in range(4):
             assert_close(f"{backend} state {k}", got[k], per[k], "float32", "state")
         assert float((got[0].double() - whole[0]).abs().max()) > 1e-2
+
+
+@pytest.mark.parametrize("function,B,T,N,D,dtype", [
+    ("lstm", 336, 24, 12, 64, "bfloat16"), ("slstm", 300, 16, 12, 64, "bfloat16"), ("lstm", 340, 16, 24, 32, "bfloat16"),
+    ("gru", 336, 24, 12, 64, "float16"), ("lstm", 160, 16, 12, 64, "float32")])
+def test_small_heads_at_large_batches(gpu, function, B, T, N, D, dtype):
+    """Heads of one workgroup keep 4-row tiles while at most four workgroups (eight of up to two waves) share a
+    compute unit: here 1008, 900, 2040, 1008 and 480 workgroups in one launch."""
+    print(f"case large batch {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
+    check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=5, init="randn")
