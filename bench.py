@@ -413,9 +413,6 @@ def main():
     if not args.no_cpu:
         out["cpu_baseline"] = run_cpu_baseline(w)
     print(json.dumps(out), flush=True)
-    # (a process that ends within milliseconds of a backward pass can die in PyTorch's shutdown, after its work is
-    # done: the autograd worker thread is still waiting for the interpreter lock; let it finish)
-    time.sleep(0.05)
 
 
 if __name__ == "__main__":

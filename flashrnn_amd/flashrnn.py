@@ -12,6 +12,7 @@ for the backward pass (:746) or slice dWx (:789-796).
 """
 from __future__ import annotations
 
+import atexit
 import functools
 import os
 from dataclasses import dataclass
@@ -256,8 +257,72 @@ class _StatusLog:
         entry[3].synchronize()
         return int(entry[2][0])
 
+    def drain(self) -> list:
+        """Waits for every pending entry, then lets go of all events and pinned words (while the HIP runtime is
+        still up).  Returns the descriptions of the calls whose status word was set."""
+        with self._lock:
+            pending, self._pending = list(self._pending), type(self._pending)()
+            self._last, self._free = {}, []
+        failed = []
+        for kind, what, host, ev in pending:
+            ev.synchronize()
+            if int(host[0]) != 0:
+                failed.append(f"{kind} of {what}")
+        return failed
+
 
 _status = _StatusLog()
+# devices on which a backward pass of this package ran: their autograd worker threads are what _teardown orders
+_backward_devices = set()
+_used_devices = set()  # every device a call of this package launched kernels on
+
+
+def _teardown() -> None:
+    """Runs once, from atexit, before the interpreter starts to finalise.  Never raises.
+
+    Why it exists.  A process that ended within milliseconds of a backward pass died now and then with
+    "terminate called without an active exception" (exit status 134) after all its work was done.  torch >= 2.10
+    releases the Python wrapper of a tensor on whatever thread drops the last other C++ reference to it
+    (c10::intrusive_ptr: decref_pyobject() noexcept on the 2 -> 1 transition), and that needs the interpreter
+    lock.  CPython 3.10 ends any thread that is waiting for the lock when finalisation begins with
+    pthread_exit(); the forced unwinding then meets the noexcept frame and C++ answers with std::terminate().
+    The one foreign thread that handles this package's tensors is the autograd engine's worker thread of the
+    device: after ``torch.autograd.grad`` / ``backward`` has returned to the caller it may still have the tail
+    of its loop iteration to run (it wakes the caller first and lets go of the finished graph task, whose
+    result holds the gradient tensors, afterwards), and on a busy machine that tail can be preempted for
+    milliseconds.
+
+    What it does.  (1) waits for the device work of every device this package used; (2) drains the status
+    log: events and pinned words are released now, by this thread; (3) sends one trivial backward pass through
+    the worker thread of every device a backward pass of this package ran on.  The worker takes tasks one at
+    a time, so when that pass has come back the worker has finished every iteration before it, all its
+    references to this package's tensors are gone, and what the trivial pass itself leaves behind holds no
+    Python-wrapped tensor (it accumulates into .grad, nothing is captured)."""
+    try:
+        if not torch.cuda.is_available() or not torch.cuda.is_initialized():
+            return
+        devices = sorted(_backward_devices)
+        _backward_devices.clear()
+        for index in sorted(_used_devices):
+            torch.cuda.synchronize(index)
+        failed = _status.drain()
+        if failed:
+            import sys
+
+            print("flashrnn_amd: a bounded wait between workgroups ran out in: " + "; ".join(failed)
+                  + " (outputs of those calls were NaN)", file=sys.stderr)
+        for index in devices:
+            with torch.enable_grad():
+                x = torch.zeros(1, device=torch.device("cuda", index), requires_grad=True)
+                (x * 1.0).backward(torch.zeros_like(x))
+            del x
+    except Exception:  # (at exit there is nobody left to tell)
+        pass
+
+
+# (registered when the package is imported, i.e. after torch: exit functions run last-in first-out, so this one runs
+# while everything torch registered for exit is still in place)
+atexit.register(_teardown)
 
 
 def check_status() -> None:
@@ -319,6 +384,7 @@ def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
     f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
     B, T, Gw, N, D = Wx_k.shape
     S = cfg.num_states
+    _used_devices.add(Wx_k.device.index if Wx_k.device.index is not None else torch.cuda.current_device())
     with _on_device(Wx_k.device):
         rc = _entry(cfg.backend, "supported")(f_id, d_id, B, N, D)
         if rc == 0 and cfg.recompute_gates:
@@ -405,6 +471,7 @@ class _FlashRNNFunction(torch.autograd.Function):
         cfg = ctx.cfg
         R_k, b_k, s0_k, states, cache, Wx_k = ctx.saved_tensors
         S, B, T, N, D = states.shape
+        _backward_devices.add(states.device.index if states.device.index is not None else torch.cuda.current_device())
         _status.poll()
         ds = dstates.to(states.dtype).contiguous()
         with _on_device(states.device):
@@ -451,6 +518,7 @@ class _FlashRNNRangesFunction(torch.autograd.Function):
         S, _, T, N, D = dstates.shape
         B = sum(saved[3 * i].shape[1] for i in range(len(saved) // 3))
         kdt = DTYPE_DICT[cfg.dtype]
+        _backward_devices.add(dstates.device.index if dstates.device.index is not None else torch.cuda.current_device())
         _status.poll()
         ds = dstates.to(kdt)
         with _on_device(dstates.device):

@@ -65,10 +65,7 @@ def hip_run(function, inp, dtype, backend, device, backward=True, options=None):
     out, last = flashrnn(*leaves, config=config)
     grads = None
     if backward:
-        # (the cotangent keeps a reference here until the call is over: a temporary would be handed to the autograd
-        # engine's worker thread to release, which needs the interpreter lock and can outlive a short test process)
-        cot = inp["dstates"].to(device).to(out.dtype)
-        grads = torch.autograd.grad(out, leaves, grad_outputs=cot)
+        grads = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(device).to(out.dtype))
         grads = [g.float().cpu() for g in grads]
     torch.cuda.synchronize()
     check_status()  # raises if a bounded wait between workgroups ran out in any fused call so far
