@@ -292,6 +292,71 @@ def run_steps(device, n_steps=256):
     return out
 
 
+def run_decode(device, n_tokens=256):
+    """The resident decode kernel (FlashRNNDecoder): microseconds per token, (a) one token per post, eager; (b) the
+    same replayed from a HIP graph of 64 chained posts, each of which ends when it has collected its token: the
+    device-side cost of a token whose input depends on the previous output; (c) 16 tokens per post, replayed: the
+    rate at which the resident kernel serves tokens that are already there."""
+    import torch
+    from flashrnn_amd import FlashRNNDecoder
+    from oracle import make_inputs
+
+    out = []
+    side = torch.cuda.Stream()
+    for function, N, D in (("lstm", 3, 256), ("lstm", 4, 192), ("lstm", 12, 64), ("gru", 4, 128), ("slstm", 4, 192)):
+        for B in (1, 8):
+            inp = make_inputs(function, B, 16, N, D, 7, init="randn", round_to=torch.bfloat16)
+            x = {k: v.to(device, torch.bfloat16).contiguous() for k, v in inp.items()}
+            wx1, wx16 = x["Wx"][:, :1].contiguous(), x["Wx"].contiguous()
+            S = x["states"].shape[0]
+            o1 = torch.empty((S, B, 1, N, D), dtype=torch.bfloat16, device=device)
+            o16 = torch.empty((S, B, 16, N, D), dtype=torch.bfloat16, device=device)
+            side.wait_stream(torch.cuda.current_stream())
+            with torch.cuda.stream(side):  # (graph capture needs a stream other than the default one)
+                dec = FlashRNNDecoder(x["R"], x["b"], x["states"], function=function, slots=16, idle_polls=1 << 23)
+                for _ in range(20):
+                    dec.step(wx1, out=o1)
+                side.synchronize()
+                t0 = time.perf_counter()
+                for _ in range(n_tokens):
+                    dec.step(wx1, out=o1)
+                side.synchronize()
+                eager = (time.perf_counter() - t0) / n_tokens * 1e6
+
+                graphs = []  # (kept until the session is closed: destroying a graph frees memory, which waits for the device)
+
+                def replayed(wx, o, launches):
+                    # (capture_begin / capture_end: the torch.cuda.graph context manager synchronises the device)
+                    g = torch.cuda.CUDAGraph()
+                    graphs.append(g)
+                    g.capture_begin()
+                    for _ in range(launches):
+                        dec.step(wx, out=o)
+                    g.capture_end()
+                    for _ in range(3):
+                        g.replay()
+                    side.synchronize()
+                    reps = 8
+                    t0 = time.perf_counter()
+                    for _ in range(reps):
+                        g.replay()
+                    side.synchronize()
+                    return (time.perf_counter() - t0) / (reps * launches * wx.shape[1]) * 1e6
+
+                one = replayed(wx1, o1, 64)
+                many = replayed(wx16, o16, 16)
+                dec.close()
+                side.synchronize()
+                graphs.clear()
+            c = dec.control()
+            assert not c["wait_expired"] and not c["collect_gave_up"], c
+            out.append({"cell": f"{function} bf16 B{B} N{N} D{D}", "backend": "hip_fused, resident kernel",
+                        "eager_us_per_token": eager, "graph_replay_us_per_token": one,
+                        "graph_replay_us_per_token_16_per_post": many, "tokens_served": c["tokens_served"]})
+    torch.cuda.current_stream().wait_stream(side)
+    return out
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -340,12 +405,13 @@ def main():
         return
     if args.workload == "step":
         rows = run_steps(device)
+        decode_rows = run_decode(device)
         ref = rows[0]
         print(json.dumps({"metric": "microseconds per single decoding step (flashrnn_step, fp32 carry)", "value": ref["graph_replay_us_per_step"],
                           "unit": "us/step", "n_gpus": 1, "steps": 256, "warmup": 20, "ms_per_step": ref["graph_replay_us_per_step"] / 1e3,
                           "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16", "data": "synthetic",
                           "config": {"workload": "step: value is " + ref["cell"] + " on " + ref["backend"] + ", graph replay"},
-                          "steps_table": rows}))
+                          "steps_table": rows, "resident_decode_table": decode_rows}))
         return
     w = WORKLOADS[args.workload]
     backend = args.backend or ("hip" if args.workload == "C5" else "hip_fused")

@@ -6,8 +6,10 @@ There is no CPU path: calls fail loudly without the HIP library or a GPU.
 """
 from .flashrnn import (  # noqa: F401
     FlashRNNConfig,
+    FlashRNNDecoder,
     check_status,
     flashrnn,
+    flashrnn_decode,
     flashrnn_step,
     fused_plan,
     last_status,
@@ -16,6 +18,6 @@ from .flashrnn import (  # noqa: F401
 )
 from ._lib import build_library, library_path, load_library  # noqa: F401
 
-__all__ = ["flashrnn", "flashrnn_step", "make_carry", "FlashRNNConfig", "rnn_function_registry", "fused_plan",
+__all__ = ["flashrnn", "flashrnn_step", "flashrnn_decode", "FlashRNNDecoder", "make_carry", "FlashRNNConfig", "rnn_function_registry", "fused_plan",
            "last_status", "check_status",
            "load_library", "library_path", "build_library"]

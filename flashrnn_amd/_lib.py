@@ -20,8 +20,12 @@ E_ARG, E_UNSUPPORTED, E_NULL, E_ALIGN, E_WORKSPACE, E_DEVICE = -1, -2, -3, -4, -
 class Options(ctypes.Structure):
     """frnn_options of include/flashrnn_hip.h (0 / False = option off)."""
 
-    _fields_ = [("forward_clipval", ctypes.c_float), ("gradient_recurrent_clipval", ctypes.c_float),
-                ("gradient_recurrent_cut", c_int), ("recompute", c_int)]
+    _fields_ = [("struct_size", ctypes.c_uint), ("forward_clipval", ctypes.c_float),
+                ("gradient_recurrent_clipval", ctypes.c_float), ("gradient_recurrent_cut", c_int), ("recompute", c_int)]
+
+    def __init__(self, forward_clipval=0.0, gradient_recurrent_clipval=0.0, gradient_recurrent_cut=0, recompute=0):
+        super().__init__(ctypes.sizeof(Options), forward_clipval, gradient_recurrent_clipval, gradient_recurrent_cut,
+                         recompute)
 
 
 _P6 = [c_int] * 6
@@ -58,6 +62,12 @@ _SIGNATURES = {
     "frnn_fused_backward_recompute": (c_int, _P6 + [c_void_p] * 11 + [c_size_t, c_void_p, POINTER(Options)]),
     "frnn_fused_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),
     "frnn_alt_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),
+    "frnn_streams_overlap": (c_int, [c_void_p, c_void_p]),
+    "frnn_fused_decode_mailbox_bytes": (c_size_t, _P6),
+    "frnn_fused_decode_mailbox_layout": (c_int, _P6 + [POINTER(c_size_t)] * 4),
+    "frnn_fused_decode_open": (c_int, [c_int] * 5 + [c_void_p] * 5 + [c_size_t, c_int, c_int, c_int, c_void_p, c_void_p, POINTER(Options)]),
+    "frnn_fused_decode_step": (c_int, [c_int] * 6 + [c_void_p] * 3 + [c_size_t, c_int, c_void_p]),
+    "frnn_fused_decode_close": (c_int, [c_void_p] * 3),
     "frnn_fused_forward_static_max_bytes": (c_size_t, []),
     "frnn_fused_forward_static": (c_int, [c_int] * 7 + [c_void_p] * 7 + [POINTER(Options)]),
 }

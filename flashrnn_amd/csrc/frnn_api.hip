@@ -2,6 +2,7 @@
 // workspace carving, launch sequencing.  No device allocation, no hidden streams, no
 // device-wide synchronisation.
 #include <stdarg.h>
+#include <stddef.h>
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
@@ -13,6 +14,7 @@
 #include "frnn_fused_fwd.h"
 #include "frnn_grad.h"
 #include "frnn_launch.h"
+#include "frnn_mailbox.h"
 
 namespace frnn {
 
@@ -213,6 +215,8 @@ static int tile_rows_for(int B, int N, int kw, int waves, int largest) {
 // capture are left alone (a captured launch is replayed later, when this order means nothing): overlapping
 // replays are the caller's to order.  Kernels of other processes are not seen; there the bounded waits and
 // the status word remain the safety net.
+// The event is recorded on the launching stream itself, right behind the launch (gate_leave); a later launch on
+// another stream waits for that event.  `last` is only ever compared, never used: the stream it names may be gone.
 struct LaunchGate { std::mutex mu; hipEvent_t ev = nullptr; hipStream_t last = nullptr; bool have = false; };
 static LaunchGate g_gate[64];
 static bool stream_capturing(hipStream_t st) {
@@ -229,17 +233,20 @@ static LaunchGate* gate_enter(int kw, hipStream_t st) {
   if (stream_capturing(st)) return nullptr;
   LaunchGate* g = &g_gate[dev];
   g->mu.lock();
-  if (g->have && g->last != st && !stream_capturing(g->last)) {
-    if (!g->ev && hipEventCreateWithFlags(&g->ev, hipEventDisableTiming) != hipSuccess) { g->ev = nullptr; (void)hipGetLastError(); }
-    // (a stream that no longer exists has no work left to wait for: errors are dropped)
-    if (g->ev && hipEventRecord(g->ev, g->last) == hipSuccess) (void)hipStreamWaitEvent(st, g->ev, 0);
-    (void)hipGetLastError();
+  if (g->have && g->last != st) {
+    if (hipStreamWaitEvent(st, g->ev, 0) != hipSuccess) (void)hipGetLastError();
   }
   return g;
 }
-static void gate_leave(LaunchGate* g, hipStream_t st) {
+// record == false: the launch is not one that later launches should queue behind (the resident decode kernel, which
+// stays on the device until its session ends)
+static void gate_leave(LaunchGate* g, hipStream_t st, bool launched_ok = true, bool record = true) {
   if (!g) return;
-  g->last = st; g->have = true;
+  if (launched_ok && record) {
+    if (!g->ev && hipEventCreateWithFlags(&g->ev, hipEventDisableTiming) != hipSuccess) { g->ev = nullptr; (void)hipGetLastError(); }
+    if (g->ev && hipEventRecord(g->ev, st) == hipSuccess) { g->last = st; g->have = true; }
+    else { g->have = false; (void)hipGetLastError(); }
+  }
   g->mu.unlock();
 }
 
@@ -250,13 +257,17 @@ struct Opts { float h_clip, g_clip; int cut; int fx; int rc; };
 static int parse_opts(const frnn_options* o, int function, Opts* out) {
   out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0; out->fx = function; out->rc = 0;
   if (!o) return 0;
+  // (the struct may grow at its end: struct_size says how much of it the caller's build knows)
+  if (o->struct_size < offsetof(frnn_options, recompute))
+    return fail(FRNN_E_ARG, "frnn_options.struct_size = %u: set it to sizeof(frnn_options) (%zu here)", o->struct_size, sizeof(frnn_options));
+  const int recompute = o->struct_size >= offsetof(frnn_options, recompute) + sizeof(int) ? o->recompute : 0;
   if (o->forward_clipval != o->forward_clipval || o->gradient_recurrent_clipval != o->gradient_recurrent_clipval ||
       o->forward_clipval < 0.f || o->gradient_recurrent_clipval < 0.f)
     return fail(FRNN_E_ARG, "clip values must be positive, or 0 for none (got %g, %g)", (double)o->forward_clipval,
                 (double)o->gradient_recurrent_clipval);
   out->h_clip = o->forward_clipval; out->g_clip = o->gradient_recurrent_clipval; out->cut = o->gradient_recurrent_cut != 0;
   if (function == FRNN_ELMAN && out->h_clip > 0.f) out->fx = FRNN_ELMAN_CLIP;
-  out->rc = o->recompute != 0 && function != FRNN_ELMAN;  // (elman caches nothing, or one value under forward_clipval)
+  out->rc = recompute != 0 && function != FRNN_ELMAN;  // (elman caches nothing, or one value under forward_clipval)
   return 0;
 }
 
@@ -381,7 +392,13 @@ static int weight_grads(int function, int dtype, int B, int T, int N, int D, con
 // allocate.  Every device the library runs on holds its own copy of the array until the process ends; in
 // host code the array's name is only a handle for hipGetSymbolAddress, the address itself is looked up
 // once per device (with that device current) and kept.
+// The array has two areas: the first kStaticForwardBytes serve frnn_fused_forward_static, the rest is where the
+// single-step kernels (frnn_fused_step) put their status word and the exchange words that nobody reads, so that a
+// step on one stream cannot touch the live exchange of a static forward call on another.
 static constexpr size_t kStaticScratchBytes = (size_t)4 << 20;
+static constexpr size_t kStaticStepBytes = (size_t)512 << 10;
+static constexpr size_t kStaticProbeBytes = 256;  // the two words of frnn_streams_overlap, at the very end
+static constexpr size_t kStaticForwardBytes = kStaticScratchBytes - kStaticStepBytes - kStaticProbeBytes;
 static __device__ __align__(256) unsigned char g_static_scratch[kStaticScratchBytes];
 static std::mutex g_scratch_mu;
 static void* g_scratch_ptr[64] = {nullptr};
@@ -399,6 +416,54 @@ static int static_scratch(void** out) {
   }
   *out = g_scratch_ptr[dev];
   return 0;
+}
+
+// ---- resident decode kernel: tiling, residency, mailbox layout ---------------------------------------------
+struct DecodePlan { Plan p; MbLayout l; int groups; };
+// Tiling, residency and mailbox layout of a decode session; 0 or an error code (message set).
+static int decode_plan(int function, int dtype, int B, int N, int D, int slots, DecodePlan* out) {
+  int e = check_problem(function, dtype, B, 1, N, D);
+  if (e) return e;
+  if (slots != 2 && slots != 4 && slots != 8 && slots != 16) return fail(FRNN_E_ARG, "slots must be 2, 4, 8 or 16 (got %d)", slots);
+  if (!find_plan(function, dtype, D, 0, 0, &out->p))
+    return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
+  const Plan& p = out->p;
+  out->groups = N * ((B + 3) / 4);
+  // every workgroup of the session stays on the device until the session ends: all of them must fit at once
+  const long room = p.kw > 1 ? groups_per_launch(p.kw) : (long)device_cus() * (p.waves <= 4 ? 2 : 1);
+  if (out->groups > room)
+    return fail(FRNN_E_UNSUPPORTED, "a decode session of %d groups (N * ceil(B / 4)) does not fit the device at once (room for %ld "
+                "with %d workgroup(s) per head)", out->groups, room, p.kw);
+  const CellDims c = cell_dims(function);
+  const size_t llw = (size_t)16 * D / (dtype == FRNN_F32 ? 1 : 2);
+  out->l = mb_layout(dtype, B, N, D, c.GW, c.S, slots, p.kw > 1 ? (size_t)out->groups * 3 * llw * 8 : 0,
+                     p.kw > 1 ? (size_t)out->groups * 32 * 4 : 0);
+  if ((size_t)slots * out->l.in_slot >= ((size_t)1 << 31) || (size_t)slots * out->l.out_slot >= ((size_t)1 << 31))
+    return fail(FRNN_E_ARG, "the inbox of this session reaches 2 GiB");
+  return 0;
+}
+template <typename T> static int exchange_launch(int function, const MbExchangeArgs& x, dim3 grid, hipStream_t st) {
+  switch (function) {
+    case FRNN_LSTM:  hipLaunchKernelGGL((decode_exchange_kernel<T, 4, 2>), grid, dim3(256), 0, st, x); break;
+    case FRNN_SLSTM: hipLaunchKernelGGL((decode_exchange_kernel<T, 4, 4>), grid, dim3(256), 0, st, x); break;
+    case FRNN_GRU:   hipLaunchKernelGGL((decode_exchange_kernel<T, 3, 1>), grid, dim3(256), 0, st, x); break;
+    default:         hipLaunchKernelGGL((decode_exchange_kernel<T, 1, 1>), grid, dim3(256), 0, st, x); break;
+  }
+  return (int)hipGetLastError();
+}
+template <int F> static int fused_dec_dispatch(int dtype, const Plan& p, const FwdArgs& a, hipStream_t st) {
+  return dtype == FRNN_BF16 ? fused_dec_launch<F, FRNN_BF16>(p, a, st)
+       : dtype == FRNN_F16 ? fused_dec_launch<F, FRNN_F16>(p, a, st) : fused_dec_launch<F, FRNN_F32>(p, a, st);
+}
+// `second` waits (on the device) for everything queued on `first` so far
+static int order_streams(hipStream_t first, hipStream_t second) {
+  hipEvent_t ev;
+  hipError_t e = hipEventCreateWithFlags(&ev, hipEventDisableTiming);
+  if (e != hipSuccess) return (int)e;
+  e = hipEventRecord(ev, first);
+  if (e == hipSuccess) e = hipStreamWaitEvent(second, ev, 0);
+  (void)hipEventDestroy(ev);  // (the wait keeps what it needs)
+  return (int)e;
 }
 
 }  // namespace frnn
@@ -555,6 +620,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
   a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(fx, dtype, p, tr));
   a.h_clip = o.h_clip;
+  a.mailbox = nullptr; a.inbox_off = a.outbox_off = a.in_slot = a.out_slot = 0; a.slots = 1; a.idle_limit = 0;
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);
@@ -573,7 +639,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
     prof_end(st);
     if (e) break;
   }
-  gate_leave(gate, st);
+  gate_leave(gate, st, e == 0);
   return e ? hip_fail(e, "fused forward launch") : 0;
 }
 
@@ -585,7 +651,7 @@ int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, 
                             workspace_bytes, stream, opt);
 }
 
-size_t frnn_fused_forward_static_max_bytes(void) { return kStaticScratchBytes; }
+size_t frnn_fused_forward_static_max_bytes(void) { return kStaticForwardBytes; }
 
 int frnn_fused_forward_static(int function, int dtype, int training, int B, int T, int N, int D,
                               const void* Wx, const void* R, const void* b, const void* s0,
@@ -598,14 +664,14 @@ int frnn_fused_forward_static(int function, int dtype, int training, int B, int 
   if (!pick_plan(function, dtype, B, N, D, 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
   const size_t need = carve_fused_fwd(nullptr, dtype, B, N, D, p).total;
-  if (need > kStaticScratchBytes)
+  if (need > kStaticForwardBytes)
     return fail(FRNN_E_WORKSPACE, "this problem needs %zu bytes of workspace, the static scratch array holds %zu: "
-                "use frnn_fused_forward_opt with a workspace of the caller", need, kStaticScratchBytes);
+                "use frnn_fused_forward_opt with a workspace of the caller", need, kStaticForwardBytes);
   void* ws = nullptr;
   e = static_scratch(&ws);
   if (e) return e;
   return fused_forward_impl(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, ws,
-                            kStaticScratchBytes, stream, opt);
+                            kStaticForwardBytes, stream, opt);
 }
 
 int frnn_fused_backward(int function, int dtype, int B, int T, int N, int D,
@@ -695,7 +761,7 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
     prof_end(st);
     if (e) break;
   }
-  gate_leave(gate, st);
+  gate_leave(gate, st, e == 0);
   if (e) return hip_fail(e, "fused backward launch");
   return weight_grads(fx, dtype, B, T, N, D, s0, states, dWx, w.dgx, w.part, w.splits, w.dbp, bt, dR, db, st);
 }
@@ -705,7 +771,7 @@ int frnn_fused_backward_opt(int function, int dtype, int B, int T, int N, int D,
                             const void* cache, const void* dstates,
                             void* dWx, void* ds0, float* dR, float* db,
                             void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
-  if (opt && opt->recompute && function != FRNN_ELMAN) {
+  if (opt && opt->struct_size >= sizeof(frnn_options) && opt->recompute && function != FRNN_ELMAN) {
     g_err[0] = 0;
     return fail(FRNN_E_ARG, "recompute mode has no gate cache: call frnn_fused_backward_recompute, which takes Wx");
   }
@@ -719,7 +785,8 @@ int frnn_fused_backward_recompute(int function, int dtype, int B, int T, int N, 
                                   void* workspace, size_t workspace_bytes, void* stream, const frnn_options* opt) {
   frnn_options o2;
   memset(&o2, 0, sizeof(o2));
-  if (opt) o2 = *opt;
+  if (opt) memcpy(&o2, opt, opt->struct_size < sizeof(o2) ? opt->struct_size : sizeof(o2));
+  o2.struct_size = sizeof(o2);
   o2.recompute = 1;
   if (Wx && Wx == dWx) { g_err[0] = 0; return fail(FRNN_E_ARG, "dWx must not be Wx: the scan reads Wx two steps ahead of its dWx stores"); }
   return fused_backward_impl(function, dtype, B, T, N, D, Wx, R, b, s0, states, nullptr, dstates, dWx, ds0, dR, db,
@@ -733,6 +800,148 @@ int frnn_fused_recompute_supported(int function, int dtype, int B, int N, int D)
   if (function != FRNN_ELMAN && !find_plan(function, dtype, D, 0, 2, &p))
     return fail(FRNN_E_UNSUPPORTED, "no recompute-mode kernel for function %d dtype %d head dim %d", function, dtype, D);
   return 0;
+}
+
+// ---- resident decode kernel -------------------------------------------------------------------------------
+
+int frnn_streams_overlap(void* stream, void* kernel_stream) {
+  g_err[0] = 0;
+  hipStream_t st = (hipStream_t)stream, ks = (hipStream_t)kernel_stream;
+  if (st == ks) return 0;
+  if (stream_capturing(st) || stream_capturing(ks)) return fail(FRNN_E_ARG, "streams under capture cannot be probed");
+  void* ws = nullptr;
+  int e = static_scratch(&ws);
+  if (e) return e;
+  int* words = (int*)(static_cast<unsigned char*>(ws) + kStaticScratchBytes - kStaticProbeBytes);
+  static std::mutex mu;  // (one probe at a time: they share the two words)
+  std::lock_guard<std::mutex> lk(mu);
+  hipError_t h = hipStreamSynchronize(st);  // work queued on `stream` earlier must not be mistaken for the resident kernel
+  if (h == hipSuccess) h = (hipError_t)launch_fill_zero(words, kStaticProbeBytes, st);
+  if (h == hipSuccess) h = (hipError_t)order_streams(st, ks);
+  if (h != hipSuccess) return hip_fail((int)h, "overlap probe setup");
+  // a kernel that waits on `kernel_stream` (at most ~3 ms) for a word that a kernel on `stream` sets
+  hipLaunchKernelGGL(overlap_spin_kernel, dim3(1), dim3(64), 0, ks, words, 20000);
+  h = hipGetLastError();
+  if (h == hipSuccess) { hipLaunchKernelGGL(decode_ctrl_store_kernel, dim3(1), dim3(64), 0, st, words, 1); h = hipGetLastError(); }
+  int host[2] = {0, 0};
+  if (h == hipSuccess) h = hipStreamSynchronize(ks);
+  if (h == hipSuccess) h = hipMemcpyAsync(host, words, sizeof(host), hipMemcpyDeviceToHost, st);
+  if (h == hipSuccess) h = hipStreamSynchronize(st);
+  if (h != hipSuccess) return hip_fail((int)h, "overlap probe");
+  return host[1] == 1 ? 1 : 0;
+}
+
+size_t frnn_fused_decode_mailbox_bytes(int function, int dtype, int B, int N, int D, int slots) {
+  DecodePlan dp;
+  if (decode_plan(function, dtype, B, N, D, slots, &dp)) return 0;
+  return dp.l.total;
+}
+
+int frnn_fused_decode_mailbox_layout(int function, int dtype, int B, int N, int D, int slots,
+                                     size_t* inbox_offset, size_t* inbox_slot_bytes,
+                                     size_t* outbox_offset, size_t* outbox_slot_bytes) {
+  g_err[0] = 0;
+  DecodePlan dp;
+  int e = decode_plan(function, dtype, B, N, D, slots, &dp);
+  if (e) return e;
+  if (inbox_offset) *inbox_offset = dp.l.inbox_off;
+  if (inbox_slot_bytes) *inbox_slot_bytes = dp.l.in_slot;
+  if (outbox_offset) *outbox_offset = dp.l.outbox_off;
+  if (outbox_slot_bytes) *outbox_slot_bytes = dp.l.out_slot;
+  return 0;
+}
+
+int frnn_fused_decode_open(int function, int dtype, int B, int N, int D,
+                           const void* R, const void* b, const void* s_in, float* carry,
+                           void* mailbox, size_t mailbox_bytes, int slots, int max_tokens, int idle_polls,
+                           void* stream, void* kernel_stream, const frnn_options* opt) {
+  g_err[0] = 0;
+  DecodePlan dp;
+  int e = decode_plan(function, dtype, B, N, D, slots, &dp);
+  if (e) return e;
+  Opts o;
+  e = parse_opts(opt, function, &o);
+  if (e) return e;
+  if (max_tokens <= 0 || idle_polls <= 0) return fail(FRNN_E_ARG, "max_tokens and idle_polls must be positive (got %d, %d)", max_tokens, idle_polls);
+  CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s_in) CHECK_PTR(mailbox)
+  if (((uintptr_t)mailbox) & 255) return fail(FRNN_E_ALIGN, "mailbox is not 256-byte aligned");
+  if (carry && (((uintptr_t)carry) & 15)) return fail(FRNN_E_ALIGN, "carry is not 16-byte aligned");
+  if (mailbox_bytes < dp.l.total) return fail(FRNN_E_WORKSPACE, "mailbox %zu < %zu bytes", mailbox_bytes, dp.l.total);
+  hipStream_t st = (hipStream_t)stream, ks = (hipStream_t)kernel_stream;
+  if (st == ks) return fail(FRNN_E_ARG, "kernel_stream must be a stream of its own: the resident kernel occupies it until the session ends");
+  if (stream_capturing(st) || stream_capturing(ks)) return fail(FRNN_E_ARG, "a decode session cannot be opened under stream capture");
+  if (env_int("FRNN_DECODE_NO_PROBE", 0) == 0) {
+    e = frnn_streams_overlap(stream, kernel_stream);
+    if (e < 0) return e;
+    if (e == 0)
+      return fail(FRNN_E_DEVICE, "kernels on `stream` do not run while one on `kernel_stream` is running (the two share a hardware "
+                  "queue): pick another kernel_stream (frnn_streams_overlap tells which pairs work)");
+  }
+  // the mailbox starts at zero (no token has tag 0); cleared on the caller's stream, which also orders the clear in
+  // front of the caller's first post, and the resident kernel behind it and behind whatever produced R, b and s_in
+  e = launch_fill_zero(mailbox, dp.l.zero_bytes, st);
+  if (e) return hip_fail(e, "mailbox clear");
+  e = order_streams(st, ks);
+  if (e) return hip_fail(e, "ordering the kernel stream behind the caller's");
+  const Plan& p = dp.p;
+  unsigned char* mb = static_cast<unsigned char*>(mailbox);
+  FwdArgs a;
+  a.Wx = nullptr; a.R = R; a.b = b; a.s0 = s_in; a.states = nullptr; a.cache = nullptr;
+  a.ll = (u64*)(mb + dp.l.exch_off); a.status = (int*)mb + MB_STATUS;
+  a.xcd = (p.kw > 1 && near_stores_allowed()) ? (int*)(mb + dp.l.xcd_off) : nullptr;
+  a.carry = carry; a.step = 0;
+  a.B = B; a.T = max_tokens; a.N = N; a.grp0 = 0; a.groups = dp.groups; a.groups_total = dp.groups; a.tile_rows = 4;
+  a.training = 0;
+  a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(function, dtype, p, 4));
+  a.h_clip = o.h_clip;
+  a.mailbox = mailbox; a.inbox_off = dp.l.inbox_off; a.outbox_off = dp.l.outbox_off;
+  a.in_slot = dp.l.in_slot; a.out_slot = dp.l.out_slot; a.slots = slots; a.idle_limit = idle_polls;
+  a.trace = nullptr;
+  LaunchGate* gate = gate_enter(p.kw, ks);
+  switch (function) {
+    case FRNN_LSTM:  e = fused_dec_dispatch<FRNN_LSTM>(dtype, p, a, ks); break;
+    case FRNN_SLSTM: e = fused_dec_dispatch<FRNN_SLSTM>(dtype, p, a, ks); break;
+    case FRNN_GRU:   e = fused_dec_dispatch<FRNN_GRU>(dtype, p, a, ks); break;
+    default:         e = fused_dec_dispatch<FRNN_ELMAN>(dtype, p, a, ks); break;
+  }
+  gate_leave(gate, ks, e == 0, false);
+  return e ? hip_fail(e, "resident decode kernel launch") : 0;
+}
+
+int frnn_fused_decode_step(int function, int dtype, int B, int N, int D, int count,
+                           const void* Wx, void* s_out, void* mailbox, size_t mailbox_bytes, int slots, void* stream) {
+  g_err[0] = 0;
+  DecodePlan dp;
+  int e = decode_plan(function, dtype, B, N, D, slots, &dp);
+  if (e) return e;
+  if (count <= 0 || count > slots) return fail(FRNN_E_ARG, "count must be between 1 and slots = %d (got %d)", slots, count);
+  CHECK_PTR(Wx) CHECK_PTR(s_out) CHECK_PTR(mailbox)
+  if (mailbox_bytes < dp.l.total) return fail(FRNN_E_WORKSPACE, "mailbox %zu < %zu bytes", mailbox_bytes, dp.l.total);
+  MbExchangeArgs x;
+  x.Wx = Wx; x.s_out = s_out; x.mailbox = mailbox;
+  x.inbox_off = dp.l.inbox_off; x.outbox_off = dp.l.outbox_off; x.in_slot = dp.l.in_slot; x.out_slot = dp.l.out_slot;
+  x.B = B; x.N = N; x.D = D; x.count = count; x.slots = slots;
+  x.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
+  const dim3 grid((unsigned)(((size_t)B * N * D + 255) / 256));
+  hipStream_t st = (hipStream_t)stream;
+  prof_begin("decode_exchange_kernel", st);
+  e = dtype == FRNN_BF16 ? exchange_launch<bf16_t>(function, x, grid, st)
+    : dtype == FRNN_F16 ? exchange_launch<half_t>(function, x, grid, st) : exchange_launch<float>(function, x, grid, st);
+  prof_end(st);
+  return e ? hip_fail(e, "decode exchange launch") : 0;
+}
+
+int frnn_fused_decode_close(void* mailbox, void* stream, void* kernel_stream) {
+  g_err[0] = 0;
+  CHECK_PTR(mailbox)
+  hipStream_t st = (hipStream_t)stream, ks = (hipStream_t)kernel_stream;
+  if (st == ks) return fail(FRNN_E_ARG, "kernel_stream must differ from stream");
+  hipLaunchKernelGGL(decode_ctrl_store_kernel, dim3(1), dim3(64), 0, st, (int*)mailbox + MB_STOP, 1);
+  int e = (int)hipGetLastError();
+  if (e) return hip_fail(e, "stop word");
+  e = order_streams(ks, st);  // what follows on the caller's stream sees the carry and the control block
+  return e ? hip_fail(e, "ordering the caller's stream behind the resident kernel") : 0;
 }
 
 // ---- alternating --------------------------------------------------------------------------------------
@@ -826,8 +1035,8 @@ int frnn_fused_step(int function, int dtype, int B, int N, int D,
   void* ws = nullptr;
   int e = static_scratch(&ws);
   if (e) return e;
-  return fused_forward_impl(function, dtype, 0, B, 1, N, D, Wx_t, R, b, s_in, s_out, nullptr, ws, kStaticScratchBytes,
-                            stream, opt, 1, carry);
+  return fused_forward_impl(function, dtype, 0, B, 1, N, D, Wx_t, R, b, s_in, s_out, nullptr,
+                            static_cast<unsigned char*>(ws) + kStaticForwardBytes, kStaticStepBytes, stream, opt, 1, carry);
 }
 
 int frnn_alt_step(int function, int dtype, int B, int N, int D,

@@ -19,6 +19,7 @@
 // first MFMA of each gate.
 #pragma once
 #include "frnn_exchange.h"
+#include "frnn_mailbox.h"
 #include "frnn_plan.h"
 #include "frnn_pointwise.h"
 
@@ -40,6 +41,10 @@ struct FwdArgs {
   // step != 0: all groups send their (unread) exchange words to one area
   float* carry; int step;
   float h_clip;      // > 0: new h clamped to [-h_clip, h_clip] (forward_clipval)
+  // resident decode kernel (the MB instantiations): T = the most tokens the launch serves; the Wx of token t is taken
+  // from the inbox of `mailbox` and the new states go to its outbox (frnn_mailbox.h); a wait for a token gives up after
+  // idle_limit probes or when the stop word of the control block is set, and the kernel then ends normally
+  void* mailbox; size_t inbox_off, outbox_off, in_slot, out_slot; int slots, idle_limit;
   long long* trace;  // phase cycle sums per workgroup; only written by -DFRNN_TRACE builds
 };
 
@@ -60,9 +65,10 @@ template <> __device__ __forceinline__ float load_frag<float>(const float* row, 
   return row[ks * 4 + kq];
 }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR>
-__global__ void __launch_bounds__((WAVES + (fwd_producer_wave(Cell<F>::GR, D, WAVES, UTW, KW, TR, (int)sizeof(T)) ? 1 : 0)) * 64)
+template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool MB = false>
+__global__ void __launch_bounds__((WAVES + (!MB && fwd_producer_wave(Cell<F>::GR, D, WAVES, UTW, KW, TR, (int)sizeof(T)) ? 1 : 0)) * 64)
 fused_fwd_kernel(const FwdArgs a) {
+  static_assert(!MB || TR == 4, "the resident decode kernel runs on 4-row batch tiles");
   typedef Cell<F> C;
   typedef ST<T> X;
   typedef CellMath<F, X::FAST> CM;
@@ -103,9 +109,9 @@ fused_fwd_kernel(const FwdArgs a) {
 #endif
   constexpr int KSO = OWN_FIRST ? (D / KW) / X::KM : 0;
   __shared__ __attribute__((aligned(16))) T hbuf[2][16 * D];
-  __shared__ int dead_flag, near_word;
+  __shared__ int dead_flag, near_word, stop_flag, stop_reason;
   // Wx of one step for the whole workgroup, two buffers by step parity: [tile][gate][batch row][16 units]
-  constexpr bool PW = fwd_producer_wave(GR, D, WAVES, UTW, KW, TR, (int)sizeof(T));
+  constexpr bool PW = !MB && fwd_producer_wave(GR, D, WAVES, UTW, KW, TR, (int)sizeof(T));  // (a token's Wx cannot be fetched ahead)
   constexpr int WBUF = UT_WG * GW * TR * 16;
   __shared__ __attribute__((aligned(16))) T wbuf[PW ? 2 * WBUF + 8 : 1];  // (+ 16 bytes that swallow the writes of lanes without a piece)
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
@@ -127,7 +133,7 @@ fused_fwd_kernel(const FwdArgs a) {
   const T* __restrict__ bias_g = static_cast<const T*>(a.b);
   const T* __restrict__ s0 = static_cast<const T*>(a.s0);
   const unsigned ND = (unsigned)N * D;
-  if (tid == 0) dead_flag = 0;
+  if (tid == 0) { dead_flag = 0; stop_flag = 0; stop_reason = MB_END_NONE; }
   // (a head of one workgroup never waits, so nothing else writes its call's status word: the host launches no clearing
   // kernel for such a call and the word is set here)
   if constexpr (KW == 1) { if (blockIdx.x == 0 && tid == 0) *a.status = 0; }
@@ -194,12 +200,23 @@ fused_fwd_kernel(const FwdArgs a) {
     }
   }
 
+  // mailbox records of this lane's elements (resident decode kernel): one inbox and one outbox record per tile
+  typedef MbRec<T, GW> RI;
+  typedef MbRec<T, S> RO;
+  int* const mb_ctrl = static_cast<int*>(a.mailbox);
+  const rsrc_t rIn = make_rsrc(MB ? static_cast<char*>(a.mailbox) + a.inbox_off : nullptr, MB ? (size_t)a.slots * a.in_slot : 0);
+  const rsrc_t rOut = make_rsrc(MB ? static_cast<char*>(a.mailbox) + a.outbox_off : nullptr, MB ? (size_t)a.slots * a.out_slot : 0);
+  unsigned mi_v[MB ? UTW : 1], mo_v[MB ? UTW : 1];
   int ub[UTW];
   unsigned wx_v[UTW], st_v[UTW], ca_v[UTW];  // per-lane byte offsets; out of range for padded rows
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
     ub[u] = (slice * UT_WG + w * UTW + u) * 16;
     const unsigned d0 = n * D + ub[u] + esub;
+    if constexpr (MB) {
+      mi_v[u] = bvalid ? ((unsigned)bg * ND + d0) * RI::BYTES : kInvalidOff;
+      mo_v[u] = bvalid ? ((unsigned)bg * ND + d0) * RO::BYTES : kInvalidOff;
+    }
     wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
     st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
     ca_v[u] = (bvalid && a.training) ? ((((unsigned)(ub[u] >> 4) * Bpad + bg) * 16 + (esub & 15)) * NCP) * ES : kInvalidOff;
@@ -331,7 +348,7 @@ fused_fwd_kernel(const FwdArgs a) {
   constexpr bool WX_LATE = KW == 1;
   Dw<ND_> wx[PD + 1][UTW][GW];
   auto load_wx = [&](Dw<ND_> (&dst)[UTW][GW], int t) __attribute__((always_inline)) {
-    if constexpr (PW) return;  // (the producer wave's job)
+    if constexpr (PW || MB) return;  // (the producer wave's job; the mailbox's)
 #pragma unroll
     for (int u = 0; u < UTW; ++u)
 #pragma unroll
@@ -355,6 +372,7 @@ fused_fwd_kernel(const FwdArgs a) {
   const long long tr_begin = clock64();
 #endif
   bool dead = near_i < 0;
+  bool stopped = false;  // resident decode kernel: a wait for a token gave up (idle bound or stop word)
   // one time step: consumes `wc` (Wx of step t), prefetches Wx of step t+PD into `wn`
   auto step = [&](const int t, Dw<ND_> (&wc)[UTW][GW], Dw<ND_> (&wn)[UTW][GW]) __attribute__((always_inline)) {
     const int cur = t & 1;
@@ -395,6 +413,15 @@ fused_fwd_kernel(const FwdArgs a) {
     }
     FRNN_STAMP(c1);
     if constexpr (!WX_LATE) load_wx(wn, min(t + PD, Tn - 1));
+    // resident decode kernel: the first probe for this token's Wx goes out here and comes back behind the MFMAs;
+    // R h_(t-1) does not need it, so a token that arrives while the product runs costs its gate math only
+    Dw<RI::DW> mrec[MB ? UTW : 1];
+    const unsigned mslot = MB ? (unsigned)(t & (a.slots - 1)) : 0u;
+    auto mb_probe = [&]() __attribute__((always_inline)) {
+#pragma unroll
+      for (int u = 0; u < (MB ? UTW : 0); ++u) mrec[u] = mb_load<RI::DW>(rIn, mi_v[u], mslot * (unsigned)a.in_slot);
+    };
+    if constexpr (MB) mb_probe();
     Dw<ND_> wcl[PW ? UTW : 1][PW ? GW : 1];  // this step's Wx from the producer wave's buffer
     if constexpr (PW) {
       // (the lane's E consecutive units of a gate: 2, 4 or 8 bytes)
@@ -501,6 +528,25 @@ fused_fwd_kernel(const FwdArgs a) {
       load_wx(wn, min(t + PD, Tn - 1));
       __builtin_amdgcn_sched_barrier(0);
     }
+    if constexpr (MB) {
+      // wait for the token: every record of this wave's valid lanes carries the tags of token t.  Bounded: after
+      // idle_limit probes, or when the stop word is set, the workgroup leaves the loop (all waves together, behind
+      // one barrier) and the kernel ends normally
+      int give_up = a.spin_limit < -1 ? MB_END_IDLE : MB_END_NONE;  // (host-side test hook: give up at once)
+      for (int spins = 0; give_up == MB_END_NONE; ++spins) {
+        bool ok = true;
+#pragma unroll
+        for (int u = 0; u < UTW; ++u) ok = ok & (!bvalid | mb_ok<T, GW>(mrec[u], t));
+        if (__all(ok)) break;
+        if (spins > a.idle_limit) { give_up = MB_END_IDLE; break; }
+        if ((spins & 15) == 15 && __any(__hip_atomic_load(mb_ctrl + MB_STOP, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) != 0)) {
+          give_up = MB_END_STOP; break;
+        }
+        mb_probe();
+      }
+      if (give_up != MB_END_NONE && lane == 0) stop_reason = give_up;
+      if (barrier_or(give_up != MB_END_NONE, &stop_flag)) { stopped = true; return; }
+    }
 #ifdef FRNN_TRACE
     { float sink = 0.f;
 #pragma unroll
@@ -523,7 +569,10 @@ fused_fwd_kernel(const FwdArgs a) {
         }
       }
 #pragma unroll
-      for (int g = 0; g < GW; ++g) unpack<E>(PW ? wcl[PW ? u : 0][PW ? g : 0] : wc[u][g], wxv[g], (T*)0);
+      for (int g = 0; g < GW; ++g) {
+        if constexpr (MB) wxv[g][0] = mb_value<T, GW>(mrec[u], g);
+        else unpack<E>(PW ? wcl[PW ? u : 0][PW ? g : 0] : wc[u][g], wxv[g], (T*)0);
+      }
       float cv[NCA][E];
       float so[S][E];
 #pragma unroll
@@ -545,12 +594,19 @@ fused_fwd_kernel(const FwdArgs a) {
       if (KW > 1) ll_write<E>((T*)0, llbase, (unsigned)(bvalid ? (t & 1) : 2) * (unsigned)(LLW * 8), brow, ub[u] + esub, so[0], t, near_m);
       if constexpr (M44) reinterpret_cast<float*>(hbuf[cur ^ 1])[lds_index4(brow, ub[u] + esub)] = so[0][0];
       else lds_write<E>(hbuf[cur ^ 1], brow, ub[u] - rot_u + esub, so[0]);
+      if constexpr (MB) {  // the new states of the element as one tagged record of the outbox
+        unsigned sbits[S];
+#pragma unroll
+        for (int k = 0; k < S; ++k) sbits[k] = mb_bits<T>(so[k][0]);
+        mb_store<RO::DW>(mb_pack<T, S>(sbits, t), rOut, mo_v[u], mslot * (unsigned)a.out_slot);
+      } else {
 #pragma unroll
       for (int k = 0; k < S; ++k)
         buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
       // private cache layout [t][head][unit tile][batch row][16 units][value]: one store per tile
       if constexpr (NC > 0)
         buf_store_wide<NWC>(cache_pack<T, NCA, E>(cv), rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
+      }
     }
 #ifdef FRNN_TRACE
     FRNN_STAMP(c3);
@@ -561,7 +617,16 @@ fused_fwd_kernel(const FwdArgs a) {
   // the time loop, unrolled over the ring: step t + j consumes set j and refills the set that the
   // step before it consumed
   int t = 0;
-  if constexpr (PD == 1) {
+  int served = 0;  // resident decode kernel: tokens whose states were posted
+  if constexpr (MB) {
+    for (; t < Tn && !dead; ++t) {
+      step(t, wx[0], wx[0]);
+      if (dead || stopped) break;
+      served = t + 1;
+    }
+    t = Tn;
+  }
+  if constexpr (!MB && PD == 1) {
     // (written out: the general form below changes the register allocation of kernels that sit
     // at the register limit)
     for (; t + 1 < Tn && !dead; t += 2) {
@@ -572,7 +637,7 @@ fused_fwd_kernel(const FwdArgs a) {
     if (!dead && t < Tn) step(t, wx[0], wx[1]);
     t = Tn;
   }
-  for (; t + PD < Tn && !dead; t += PD + 1) {
+  for (; !MB && t + PD < Tn && !dead; t += PD + 1) {
 #pragma unroll
     for (int j = 0; j <= PD; ++j) {
       step(t + j, wx[j], wx[(j + PD) % (PD + 1)]);
@@ -581,7 +646,7 @@ fused_fwd_kernel(const FwdArgs a) {
   }
 #pragma unroll
   for (int j = 0; j < PD; ++j)
-    if (!dead && t + j < Tn) step(t + j, wx[j], wx[(j + PD) % (PD + 1)]);
+    if (!MB && !dead && t + j < Tn) step(t + j, wx[j], wx[(j + PD) % (PD + 1)]);
 
 #ifdef FRNN_TRACE
   if (lane == 0 && a.trace) {
@@ -596,6 +661,17 @@ fused_fwd_kernel(const FwdArgs a) {
       for (int e = 0; e < E; ++e)
 #pragma unroll
         for (int k = 0; k < S; ++k) a.carry[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e] = s[u][e][k];
+  }
+  if constexpr (MB) {
+    // (a resident kernel reports through the control block of its mailbox; the caller's collecting kernel marks what it
+    // did not get)
+    if (tid == 0 && dead) __hip_atomic_store(a.status, (int)STATUS_WAIT_EXPIRED, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    if (tid == 0 && grp == 0 && slice == 0) {
+      __hip_atomic_store(mb_ctrl + MB_DONE, served, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(mb_ctrl + MB_REASON, dead ? (int)MB_END_WAIT : stopped ? stop_reason : (int)MB_END_TOKENS,
+                         __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    return;
   }
   if (dead) {
     // bounded wait ran out: report, and make the damage visible (NaN in every h of this

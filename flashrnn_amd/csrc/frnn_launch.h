@@ -13,6 +13,8 @@ struct BwdArgs;
 // plan is not compiled in.
 template <int F, int DT> int fused_fwd_launch(const Plan& p, const FwdArgs& a, hipStream_t st);
 template <int F, int DT> int fused_bwd_launch(const Plan& p, const BwdArgs& a, hipStream_t st);
+// the forward kernel as a resident decode kernel (mailbox mode, 4-row tiles): fused_dec_tu.hip, functions 0..3
+template <int F, int DT> int fused_dec_launch(const Plan& p, const FwdArgs& a, hipStream_t st);
 
 // plan table lookup: function, dtype, D, variant -> plan; false if none.
 // backward: 0 forward, 1 reverse scan with gate cache, 2 reverse scan in recompute mode

@@ -301,6 +301,8 @@ def _teardown() -> None:
     try:
         if not torch.cuda.is_available() or not torch.cuda.is_initialized():
             return
+        for dec in list(_open_decoders):  # (a resident kernel that nobody stops holds the device until it idles out)
+            dec.close(check=False)
         devices = sorted(_backward_devices)
         _backward_devices.clear()
         for index in sorted(_used_devices):
@@ -691,6 +693,173 @@ def flashrnn_step(
 def make_carry(states: torch.Tensor) -> torch.Tensor:
     """The fp32 carry of ``flashrnn_step`` for a chain that starts at ``states`` [S,B,1,N,D]."""
     return states[:, :, 0].to(torch.float32).contiguous()
+
+class FlashRNNDecoder:
+    """A decode session: the fused forward kernel of the head dimension stays on the device, R in its registers and the
+    state in fp32 registers, and serves one token after the other (the reference decodes with one launch per token that
+    reloads R, flashrnn.py:957-985).  A chain of tokens gives bit for bit what ``flashrnn()`` gives over the sequence.
+
+        dec = FlashRNNDecoder(R, b, states, function="lstm")       # launches the resident kernel on a stream of its own
+        for t in ...:  new_states = dec.step(Wx_t)                 # [B,C,G_w,N,D] -> [S,B,C,N,D], C <= dec.slots tokens
+        dec.close()                                                # stops the kernel; dec.states / dec.carry hold the end
+
+    ``step`` is one small launch on the current stream that posts the tokens into the session's mailbox and collects
+    the new states; it allocates its output only (pass ``out=`` to allocate nothing) and can be captured into a HIP
+    graph.  While the session is open: its workgroups keep their compute units, so do not call
+    ``torch.cuda.synchronize()`` (it would wait until the kernel has idled out; synchronise streams or events
+    instead), and run every ``step`` on one stream, not on ``dec.kernel_stream``.  Every wait is bounded: the kernel
+    ends by itself after ``idle_polls`` probes without a token (about 0.4 us each) or ``max_tokens`` tokens; the
+    session can then be continued with a new ``FlashRNNDecoder(..., states=dec.states, carry=dec.carry)``.  Tensors
+    must be in the kernel dtype and the default layouts (nothing is cast or copied on this path); not differentiable."""
+
+    def __init__(self, R, b, states, function: str = "lstm", dtype: str = "bfloat16", config: Optional[FlashRNNConfig] = None,
+                 carry: Optional[torch.Tensor] = None, slots: int = 4, max_tokens: int = 1 << 30, idle_polls: int = 1 << 22,
+                 kernel_stream: Optional["torch.cuda.Stream"] = None):
+        Gr, Gw, _, Gt, S = rnn_function_registry[function]["gates_states"]
+        if states.dim() != 5 or states.shape[0] != S or states.shape[2] != 1:
+            raise ValueError(f"states must be [{S},B,1,N,D], got {tuple(states.shape)}")
+        _, B, _, N, D = states.shape
+        if config is None:
+            config = FlashRNNConfig(head_dim=D, num_heads=N, batch_size=B, function=function, backend="hip_fused", dtype=dtype)
+        if config.backend != "hip_fused":
+            raise ValueError("the resident decode kernel is the hip_fused backend's")
+        kdt = DTYPE_DICT[config.dtype]
+        if tuple(R.shape) != (Gr, N, D, D) or tuple(b.shape) != (Gt, N, D):
+            raise ValueError(f"R, b must be [{Gr},{N},{D},{D}], [{Gt},{N},{D}]; got {tuple(R.shape)}, {tuple(b.shape)}")
+        for name, x in (("R", R), ("b", b), ("states", states)):
+            if not x.is_cuda:
+                raise RuntimeError("flashrnn_amd runs on a GPU only (got a CPU tensor); there is no CPU fallback")
+            if x.dtype != kdt or not x.is_contiguous():
+                raise TypeError(f"{name} must be a contiguous {kdt} tensor (the decode path casts and copies nothing)")
+        self.config, self.function, self.kdt = config, function, kdt
+        self.B, self.N, self.D, self.S, self.Gw, self.slots = B, N, D, S, Gw, slots
+        self.device = states.device
+        self._ids = (_lib.FUNCTION_IDS[function], _lib.DTYPE_IDS[config.dtype], B, N, D)
+        lib = _lib.load_library()
+        with _on_device(self.device):
+            rc = lib.frnn_fused_decode_mailbox_layout(*self._ids, slots, None, None, None, None)
+            if rc != 0:
+                _raise(rc, "decode session")
+            nbytes = lib.frnn_fused_decode_mailbox_bytes(*self._ids, slots)
+            self.mailbox = torch.empty(nbytes, dtype=torch.uint8, device=self.device)
+            self.carry = carry if carry is not None else make_carry(states)
+            if (self.carry.dtype != torch.float32 or tuple(self.carry.shape) != (S, B, N, D)
+                    or not self.carry.is_contiguous() or self.carry.device != self.device):
+                raise TypeError(f"carry must be a contiguous float32 tensor [{S},{B},{N},{D}] on the device of the states")
+            self.states = states  # the states behind the last collected token, [S,B,1,N,D]
+            self._keep = (R, b, states)  # the kernel reads them when it starts
+            self.kernel_stream = kernel_stream if kernel_stream is not None else _kernel_stream_for(self.device)
+            _used_devices.add(self.device.index if self.device.index is not None else torch.cuda.current_device())
+            rc = lib.frnn_fused_decode_open(*self._ids, R.data_ptr(), b.data_ptr(), states.data_ptr(), self.carry.data_ptr(),
+                                            self.mailbox.data_ptr(), nbytes, slots, int(max_tokens), int(idle_polls),
+                                            _raw_stream(self.device), self.kernel_stream.cuda_stream, _options(config))
+            if rc != 0:
+                _raise(rc, "decode session")
+        self.open = True
+        _open_decoders.add(self)
+
+    def step(self, Wx: torch.Tensor, out: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Wx [B,C,G_w,N,D] (C <= slots tokens) -> their new states [S,B,C,N,D]."""
+        if not self.open:
+            raise RuntimeError("the decode session is closed")
+        if Wx.dim() != 5 or (Wx.shape[0], Wx.shape[2], Wx.shape[3], Wx.shape[4]) != (self.B, self.Gw, self.N, self.D):
+            raise ValueError(f"Wx must be [{self.B},C,{self.Gw},{self.N},{self.D}], got {tuple(Wx.shape)}")
+        C = Wx.shape[1]
+        if Wx.dtype != self.kdt or not Wx.is_contiguous() or Wx.device != self.device:
+            raise TypeError(f"Wx must be a contiguous {self.kdt} tensor on {self.device}")
+        with _on_device(self.device):
+            if out is None:
+                out = torch.empty((self.S, self.B, C, self.N, self.D), dtype=self.kdt, device=self.device)
+            elif tuple(out.shape) != (self.S, self.B, C, self.N, self.D) or out.dtype != self.kdt or not out.is_contiguous():
+                raise TypeError(f"out must be a contiguous {self.kdt} tensor [{self.S},{self.B},{C},{self.N},{self.D}]")
+            rc = _lib.load_library().frnn_fused_decode_step(*self._ids, C, Wx.data_ptr(), out.data_ptr(), self.mailbox.data_ptr(),
+                                                            self.mailbox.numel(), self.slots, _raw_stream(self.device))
+            if rc != 0:
+                _raise(rc, "decode step")
+        self.states = out[:, :, -1:]
+        return out
+
+    def control(self) -> dict:
+        """The session's control block (synchronises the current stream): status, end reason, tokens served."""
+        c = self.mailbox[:64 * 4].view(torch.int32).cpu()
+        reasons = {0: "running", 1: "a wait between workgroups ran out", 2: "idle bound reached", 3: "stopped", 4: "max_tokens served"}
+        return {"wait_expired": int(c[0]) != 0, "ended": reasons.get(int(c[2]), str(int(c[2]))), "tokens_served": int(c[3]),
+                "collect_gave_up": int(c[4]) != 0, "tokens_posted": int(c[9])}
+
+    def close(self, check: bool = True) -> None:
+        """Sets the stop word and orders the current stream behind the end of the resident kernel.  check: read the
+        control block (a synchronisation of the current stream) and raise RuntimeError if a wait ran out."""
+        if not self.open:
+            return
+        self.open = False
+        _open_decoders.discard(self)
+        with _on_device(self.device):
+            rc = _lib.load_library().frnn_fused_decode_close(self.mailbox.data_ptr(), _raw_stream(self.device),
+                                                             self.kernel_stream.cuda_stream)
+            if rc != 0:
+                _raise(rc, "decode close")
+        self._keep = None
+        if check:
+            c = self.control()
+            if c["wait_expired"] or c["collect_gave_up"]:
+                raise RuntimeError(f"flashrnn_amd decode session: a bounded wait ran out ({c}); states collected after that are NaN")
+
+    def __enter__(self):
+        return self
+
+    def __exit__(self, *exc):
+        self.close(check=exc[0] is None)
+        return False
+
+
+_open_decoders = set()
+_kernel_streams = {}
+
+
+def _kernel_stream_for(device: torch.device):
+    """A stream on which a resident kernel can run while the current stream of `device` keeps launching: the runtime
+    maps streams onto a few hardware queues, and two streams of one queue run one after the other, so candidates are
+    tried (frnn_streams_overlap measures it) and the first that works is kept for this pair."""
+    cur = _raw_stream(device)
+    key = (device.index if device.index is not None else torch.cuda.current_device(), cur)
+    known = _kernel_streams.setdefault(key, [])
+    busy = {d.kernel_stream.cuda_stream for d in _open_decoders}  # (a stream serves one resident kernel at a time)
+    for cand in known:
+        if cand.cuda_stream not in busy:
+            return cand
+    lib = _lib.load_library()
+    for _ in range(24):
+        cand = torch.cuda.Stream(device=device)
+        if cand.cuda_stream in busy or any(cand.cuda_stream == k.cuda_stream for k in known):
+            continue
+        rc = lib.frnn_streams_overlap(cur, cand.cuda_stream)
+        if rc < 0:
+            _raise(rc, "stream probe")
+        if rc == 1:
+            known.append(cand)
+            return cand
+    raise RuntimeError("flashrnn_amd: found no free stream whose kernels run beside those of the current stream "
+                       "(every candidate shares its hardware queue or serves another open session)")
+
+
+def flashrnn_decode(Wx, R, b, states=None, function: str = "lstm", dtype: str = "bfloat16", chunk: int = 1,
+                    idle_polls: int = 1 << 22):
+    """``flashrnn()`` for inference, token by token through one decode session (``chunk`` tokens per post): returns
+    ``(all_states [S,B,T,N,D], last_states [S,B,1,N,D])``, bit for bit what ``flashrnn(..., backend="hip_fused")``
+    returns.  Meant for tests and for callers that have the whole Wx; a serving loop uses FlashRNNDecoder itself."""
+    B, T, Gw, N, D = Wx.shape
+    if states is None:
+        cfg = FlashRNNConfig(head_dim=D, num_heads=N, batch_size=B, function=function, backend="hip_fused", dtype=dtype)
+        states = _zero_state(cfg, Wx)
+    S = states.shape[0]
+    out = torch.empty((S, B, T, N, D), dtype=Wx.dtype, device=Wx.device)
+    with FlashRNNDecoder(R, b, states, function=function, dtype=dtype, slots=max(2, 1 << (chunk - 1).bit_length()),
+                         idle_polls=idle_polls) as dec:
+        for t0 in range(0, T, chunk):
+            t1 = min(T, t0 + chunk)
+            out[:, :, t0:t1] = dec.step(Wx[:, t0:t1].contiguous())
+    return out, out[:, :, -1:]
+
 
 
 def _paired_heads(Wx, R, b, states, config, training):

@@ -165,6 +165,8 @@ int frnn_alt_backward(int function, int dtype, int B, int T, int N, int D,
  * Unlike the reference (which feeds gradient_recurrent_clipval into both clip defines) each
  * option acts on its own. */
 typedef struct frnn_options {
+  unsigned struct_size;  /* sizeof(frnn_options) of the caller's build: fields are only ever appended, and the library reads
+                          * no further than this (a smaller value than the first four fields need is FRNN_E_ARG) */
   float forward_clipval;
   float gradient_recurrent_clipval;
   int gradient_recurrent_cut;
@@ -247,6 +249,52 @@ size_t frnn_fused_forward_static_max_bytes(void);
 int frnn_fused_forward_static(int function, int dtype, int training, int B, int T, int N, int D,
                               const void* Wx, const void* R, const void* b, const void* s0,
                               void* states, void* cache, void* stream, const frnn_options* opt);
+
+/* ---- resident decode: the forward kernel stays on the device between tokens ---------------------------------
+ * The second half of the reference's step path (flashrnn.py:957-985, alternating/flashrnn.h:97-101), which pays a
+ * launch and a reload of R for every token: frnn_fused_decode_open launches the fused forward kernel of the head dim
+ * ONCE, on `kernel_stream`; it keeps R in its registers and the state in fp32 registers (as inside a sequence call, so
+ * a chain of tokens gives the bits of frnn_fused_forward over the same sequence) and serves one token after the other
+ * from a mailbox, a buffer of the caller (frnn_fused_decode_mailbox_bytes, 256-byte aligned, the library clears it
+ * in open): a ring of `slots` (2, 4, 8 or 16) inbox and outbox slots of tagged records, one record per element
+ * (batch row, head, unit):
+ *     inbox  record = the G_w values Wx_t[b, g, n, d] of the element, gate innermost, padded to 1, 2 or 4 values;
+ *     outbox record = its S new states; a value of a 16-bit type travels as the dword (tag16 << 16 | bits) with
+ *     tag16 = token % 65535 + 1, an fp32 value as two dwords (bits, token + 1).
+ *   Offsets inside the buffer: frnn_fused_decode_mailbox_layout.  Any kernel of the caller may write inbox records
+ *   (agent-scope stores; a GEMM epilogue, say) and read outbox records; frnn_fused_decode_step is the library's own:
+ *   one small launch on `stream` that posts Wx [B, count, G_w, N, D] (count <= slots tokens) and collects s_out
+ *   [S, B, count, N, D], taking the token numbers from the mailbox itself, so it can be captured and replayed.
+ *   Token t uses slot t % slots; token t + slots may be posted only when token t has been collected.
+ * Every wait is bounded: the kernel gives up waiting for a token after `idle_polls` probes (about 0.4 us each) or
+ * when frnn_fused_decode_close has set the stop word, or after `max_tokens`, and then ends normally, writing the
+ * unrounded state to `carry` ([S,B,N,D] fp32, optional; on entry, if given, it is the unrounded initial state as for
+ * frnn_fused_step) and the reason to the control block; the collecting side gives up after FRNN_SPIN_LIMIT probes
+ * and writes NaN.  Nothing is allocated.  While a session is open its workgroups occupy their compute units
+ * (N * ceil(B / 4) * workgroups-per-head of them; FRNN_E_UNSUPPORTED if they do not fit at once), a device-wide
+ * synchronisation waits for the session to end, and `kernel_stream` must not share a hardware queue with `stream`
+ * (a runtime maps streams onto a few queues; a post that queues behind the resident kernel is only served when the
+ * kernel has idled out).  close orders `stream` behind the end of the resident kernel. */
+/* 1 if a kernel launched on `stream` runs while a kernel on `kernel_stream` is still running, 0 if it queues behind it
+ * (the runtime maps streams onto a few hardware queues, GPU_MAX_HW_QUEUES, and two streams of one queue run one after
+ * the other), negative on error.  Measured, not guessed: a kernel on `kernel_stream` waits up to ~3 ms for a word that a
+ * kernel on `stream` sets.  Synchronises both streams; allocates nothing.  frnn_fused_decode_open runs it and refuses
+ * a pair that returns 0 (FRNN_E_DEVICE). */
+int frnn_streams_overlap(void* stream, void* kernel_stream);
+size_t frnn_fused_decode_mailbox_bytes(int function, int dtype, int B, int N, int D, int slots);
+/* byte offsets of the inbox and outbox rings and the sizes of one slot of each; the control block is the first 64 ints:
+ * [0] status (1: a wait between workgroups ran out), [1] stop word, [2] why the kernel ended (1 wait ran out, 2 idle,
+ * 3 stop word, 4 max_tokens), [3] tokens served, [4] 1 if a collecting thread gave up, [9] next token number */
+int frnn_fused_decode_mailbox_layout(int function, int dtype, int B, int N, int D, int slots,
+                                     size_t* inbox_offset, size_t* inbox_slot_bytes,
+                                     size_t* outbox_offset, size_t* outbox_slot_bytes);
+int frnn_fused_decode_open(int function, int dtype, int B, int N, int D,
+                           const void* R, const void* b, const void* s_in, float* carry,
+                           void* mailbox, size_t mailbox_bytes, int slots, int max_tokens, int idle_polls,
+                           void* stream, void* kernel_stream, const frnn_options* opt);
+int frnn_fused_decode_step(int function, int dtype, int B, int N, int D, int count,
+                           const void* Wx, void* s_out, void* mailbox, size_t mailbox_bytes, int slots, void* stream);
+int frnn_fused_decode_close(void* mailbox, void* stream, void* kernel_stream);
 
 #ifdef __cplusplus
 }

@@ -235,3 +235,51 @@ def test_layout_options_and_initial_state():
         FlashRNNConfig(input_shape="BTGH")
     with pytest.raises(ValueError):
         FlashRNNConfig(output_shape="SBTHX")
+
+
+def test_decode_session_arguments_are_checked_before_any_launch(lib):
+    L, G = _lib.FUNCTION_IDS["lstm"], _lib.FUNCTION_IDS["gru"]
+    # mailbox: control block + exchange area (heads of several workgroups) + slots x (inbox + outbox) of tagged records
+    small = lib.frnn_fused_decode_mailbox_bytes(L, 0, 8, 2, 64, 4)     # one workgroup per head: no exchange area
+    assert small == 256 + 4 * (8 * 2 * 64 * 16) + 4 * (8 * 2 * 64 * 8)
+    big = lib.frnn_fused_decode_mailbox_bytes(L, 0, 8, 3, 256, 4)
+    assert big > 256 + 4 * (8 * 3 * 256 * 24)
+    assert lib.frnn_fused_decode_mailbox_bytes(G, 1, 4, 2, 64, 2) == 256 + 2 * (4 * 2 * 64 * 32) + 2 * (4 * 2 * 64 * 8)  # fp32: 8 bytes a value
+    off = [ctypes.c_size_t() for _ in range(4)]
+    assert lib.frnn_fused_decode_mailbox_layout(L, 0, 8, 2, 64, 4, *[ctypes.byref(o) for o in off]) == 0
+    assert [o.value for o in off] == [256, 8 * 2 * 64 * 16, 256 + 4 * 8 * 2 * 64 * 16, 8 * 2 * 64 * 8]
+    assert lib.frnn_fused_decode_mailbox_bytes(L, 0, 8, 2, 64, 3) == 0 and b"slots" in lib.frnn_last_error()
+    assert lib.frnn_fused_decode_mailbox_layout(L, 0, 8, 2, 80, 4, None, None, None, None) == _lib.E_UNSUPPORTED
+    # more groups than can stay on the device at once: 2000 heads x 1 batch tile
+    assert lib.frnn_fused_decode_mailbox_layout(L, 0, 4, 2000, 64, 4, None, None, None, None) == _lib.E_UNSUPPORTED
+    assert b"fit" in lib.frnn_last_error()
+    mb = ctypes.c_void_p(0x10000)
+    s1, s2 = ctypes.c_void_p(0x100), ctypes.c_void_p(0x200)
+    args = lambda **kw: [L, 0, 8, 2, 64, kw.get("R", FAKE), FAKE, FAKE, None, kw.get("mb", mb), kw.get("bytes", small),
+                         kw.get("slots", 4), kw.get("max_tokens", 100), kw.get("idle", 1000), s1, kw.get("ks", s2), None]
+    assert lib.frnn_fused_decode_open(*args(R=None)) == _lib.E_NULL
+    assert lib.frnn_fused_decode_open(*args(mb=ctypes.c_void_p(0x10010))) == _lib.E_ALIGN
+    assert lib.frnn_fused_decode_open(*args(bytes=small - 1)) == _lib.E_WORKSPACE
+    assert lib.frnn_fused_decode_open(*args(max_tokens=0)) == _lib.E_ARG
+    assert lib.frnn_fused_decode_open(*args(idle=0)) == _lib.E_ARG
+    assert lib.frnn_fused_decode_open(*args(ks=s1)) == _lib.E_ARG and b"stream of its own" in lib.frnn_last_error()
+    step = lambda count, wx=FAKE: lib.frnn_fused_decode_step(L, 0, 8, 2, 64, count, wx, FAKE, mb, small, 4, s1)
+    assert step(0) == _lib.E_ARG and step(5) == _lib.E_ARG and step(1, None) == _lib.E_NULL
+    assert lib.frnn_fused_decode_close(None, s1, s2) == _lib.E_NULL
+    assert lib.frnn_fused_decode_close(mb, s1, s1) == _lib.E_ARG
+    assert lib.frnn_streams_overlap(s1, s1) == 0
+
+
+def test_options_carry_their_size(lib):
+    """frnn_options starts with struct_size, so that fields can be appended: a caller that knows fewer fields is served
+    with the later ones off, one that does not set the size is refused."""
+    L = _lib.FUNCTION_IDS["lstm"]
+    o = _lib.Options(0.5, 0.0, 0, 0)
+    assert o.struct_size == ctypes.sizeof(_lib.Options) == 20
+    assert lib.frnn_fused_cache_bytes_opt(L, 0, 4, 8, 2, 64, ctypes.byref(o)) > 0
+    o.struct_size = 0
+    assert lib.frnn_fused_cache_bytes_opt(L, 0, 4, 8, 2, 64, ctypes.byref(o)) == 0 and b"struct_size" in lib.frnn_last_error()
+    o = _lib.Options(0.0, 0.0, 0, 1)            # recompute on ...
+    assert lib.frnn_fused_cache_bytes_opt(L, 0, 4, 8, 2, 64, ctypes.byref(o)) == 0
+    o.struct_size = 16                          # ... but the caller's build ends before that field: it is not read
+    assert lib.frnn_fused_cache_bytes_opt(L, 0, 4, 8, 2, 64, ctypes.byref(o)) > 0
