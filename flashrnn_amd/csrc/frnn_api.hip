@@ -621,6 +621,9 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(fx, dtype, p, tr));
   a.h_clip = o.h_clip;
   a.mailbox = nullptr; a.inbox_off = a.outbox_off = a.in_slot = a.out_slot = 0; a.slots = 1; a.idle_limit = 0;
+  // producer-wave stores: for launches that fill the device (more workgroups than compute units), where the kernel is
+  // bound by its memory traffic; FRNN_PRODUCER_STORES=0/1 overrides
+  a.pst = step ? 0 : env_int("FRNN_PRODUCER_STORES", tr == 4 && p.kw == 1 && groups > device_cus() ? 1 : 0);
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);
@@ -894,7 +897,7 @@ int frnn_fused_decode_open(int function, int dtype, int B, int N, int D,
   a.training = 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(function, dtype, p, 4));
-  a.h_clip = o.h_clip;
+  a.h_clip = o.h_clip; a.pst = 0;
   a.mailbox = mailbox; a.inbox_off = dp.l.inbox_off; a.outbox_off = dp.l.outbox_off;
   a.in_slot = dp.l.in_slot; a.out_slot = dp.l.out_slot; a.slots = slots; a.idle_limit = idle_polls;
   a.trace = nullptr;

@@ -128,6 +128,7 @@ typedef __bf16 bf16x2 __attribute__((ext_vector_type(2)));
 typedef float f32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x2 __attribute__((ext_vector_type(2)));
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef unsigned u32x3 __attribute__((ext_vector_type(3)));
 
 // 16-bit storage types: the two elements of a dword <-> float, round to nearest even
 template <typename T> struct H16;
@@ -205,16 +206,39 @@ template <int N, bool SUB = false> __device__ __forceinline__ Dw<N> buf_load(rsr
   else { static_assert(N == 4, "1, 2 or 4 dwords"); const u32x4 t = __builtin_amdgcn_raw_buffer_load_b128(r, voff, soff, 0); d.v[0] = t.x; d.v[1] = t.y; d.v[2] = t.z; d.v[3] = t.w; }
   return d;
 }
+// A buffer store of more than 8 bytes reads its data registers a cycle after it issues.  When the store takes its
+// offset from an SGPR the compiler assumes that this cannot hurt and lets a vector instruction overwrite a data
+// register in the very next slot; on gfx950 that instruction's result was what reached memory (seen as the LDS address
+// of the next piece in the first dword of every 16-byte piece that a wave stored in a loop).  One independent
+// instruction in between is enough: the s_nop below names the data registers as its inputs, so nothing can overwrite
+// them before it, and it cannot move in front of the store.  Every store of 12 or 16 bytes in this library goes
+// through these helpers; a test scans the generated code of every kernel for the pattern.
+// (The data first pass through an empty asm that makes them opaque: a constant would otherwise be re-materialised
+// into other registers for the s_nop, which then would not hold the store's own registers.)
+template <int AUX = 0> __device__ __forceinline__ void store_b128_safe(unsigned a, unsigned b, unsigned c, unsigned d, rsrc_t r, unsigned voff, unsigned soff) {
+  u32x4 v = {a, b, c, d};
+  asm volatile("" : "+v"(v));  // (the register tuple itself, not the four values, is what the s_nop has to name)
+  __builtin_amdgcn_raw_buffer_store_b128(v, r, voff, soff, AUX);
+  asm volatile("s_nop 0" ::"v"(v));
+}
+__device__ __forceinline__ void store_b96_safe(unsigned a, unsigned b, unsigned c, rsrc_t r, unsigned voff, unsigned soff) {
+  u32x3 v = {a, b, c};
+  asm volatile("" : "+v"(v));
+  __builtin_amdgcn_raw_buffer_store_b96(v, r, voff, soff, 0);
+  asm volatile("s_nop 0" ::"v"(v));
+}
 template <int N, bool SUB = false> __device__ __forceinline__ void buf_store(const Dw<N>& d, rsrc_t r, unsigned voff, unsigned soff) {
   if constexpr (SUB) { static_assert(N == 1, "one 16-bit element"); __builtin_amdgcn_raw_buffer_store_b16((unsigned short)d.v[0], r, voff, soff, 0); }
   else if constexpr (N == 1) { __builtin_amdgcn_raw_buffer_store_b32(d.v[0], r, voff, soff, 0); }
   else if constexpr (N == 2) { __builtin_amdgcn_raw_buffer_store_b64(u32x2{d.v[0], d.v[1]}, r, voff, soff, 0); }
-  else { static_assert(N == 4, "1, 2 or 4 dwords"); __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[0], d.v[1], d.v[2], d.v[3]}, r, voff, soff, 0); }
+  else {
+    static_assert(N == 4, "1, 2 or 4 dwords");
+    store_b128_safe(d.v[0], d.v[1], d.v[2], d.v[3], r, voff, soff);
+  }
 }
 
 // N dwords per lane with as few instructions as possible (pieces of 4, then 3, 2 or 1 dwords):
 // every vector memory instruction costs a wave some 30 cycles of issue time, whatever its width
-typedef unsigned u32x3 __attribute__((ext_vector_type(3)));
 template <int N> __device__ __forceinline__ Dw<N> buf_load_wide(rsrc_t r, unsigned voff, unsigned soff) {
   Dw<N> d;
   constexpr int Q = N / 4 * 4, R = N % 4;
@@ -231,9 +255,12 @@ template <int N> __device__ __forceinline__ Dw<N> buf_load_wide(rsrc_t r, unsign
 template <int N> __device__ __forceinline__ void buf_store_wide(const Dw<N>& d, rsrc_t r, unsigned voff, unsigned soff) {
   constexpr int Q = N / 4 * 4, R = N % 4;
 #pragma unroll
-  for (int i = 0; i < Q; i += 4)
-    __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[i], d.v[i + 1], d.v[i + 2], d.v[i + 3]}, r, voff + i * 4, soff, 0);
-  if constexpr (R == 3) __builtin_amdgcn_raw_buffer_store_b96(u32x3{d.v[Q], d.v[Q + 1], d.v[Q + 2]}, r, voff + Q * 4, soff, 0);
+  for (int i = 0; i < Q; i += 4) {
+    store_b128_safe(d.v[i], d.v[i + 1], d.v[i + 2], d.v[i + 3], r, voff + i * 4, soff);
+  }
+  if constexpr (R == 3) {
+    store_b96_safe(d.v[Q], d.v[Q + 1], d.v[Q + 2], r, voff + Q * 4, soff);
+  }
   else if constexpr (R == 2) __builtin_amdgcn_raw_buffer_store_b64(u32x2{d.v[Q], d.v[Q + 1]}, r, voff + Q * 4, soff, 0);
   else if constexpr (R == 1) __builtin_amdgcn_raw_buffer_store_b32(d.v[Q], r, voff + Q * 4, soff, 0);
 }

@@ -41,6 +41,7 @@ struct FwdArgs {
   // step != 0: all groups send their (unread) exchange words to one area
   float* carry; int step;
   float h_clip;      // > 0: new h clamped to [-h_clip, h_clip] (forward_clipval)
+  int pst;           // host side only: launch the instantiation whose producer wave stores the outputs (fwd_producer_stores)
   // resident decode kernel (the MB instantiations): T = the most tokens the launch serves; the Wx of token t is taken
   // from the inbox of `mailbox` and the new states go to its outbox (frnn_mailbox.h); a wait for a token gives up after
   // idle_limit probes or when the stop word of the control block is set, and the kernel then ends normally
@@ -65,7 +66,7 @@ template <> __device__ __forceinline__ float load_frag<float>(const float* row, 
   return row[ks * 4 + kq];
 }
 
-template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool MB = false>
+template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool MB = false, bool PSTV = false>
 __global__ void __launch_bounds__((WAVES + (!MB && fwd_producer_wave(Cell<F>::GR, D, WAVES, UTW, KW, TR, (int)sizeof(T)) ? 1 : 0)) * 64)
 fused_fwd_kernel(const FwdArgs a) {
   static_assert(!MB || TR == 4, "the resident decode kernel runs on 4-row batch tiles");
@@ -114,6 +115,15 @@ fused_fwd_kernel(const FwdArgs a) {
   constexpr bool PW = !MB && fwd_producer_wave(GR, D, WAVES, UTW, KW, TR, (int)sizeof(T));  // (a token's Wx cannot be fetched ahead)
   constexpr int WBUF = UT_WG * GW * TR * 16;
   __shared__ __attribute__((aligned(16))) T wbuf[PW ? 2 * WBUF + 8 : 1];  // (+ 16 bytes that swallow the writes of lanes without a piece)
+  // Producer-wave stores (PSTV instantiations of the heads that run as one workgroup with a producer wave; chosen on the
+  // host for launches that fill the device, where the kernel is bound by memory traffic): at 4-row tiles a compute
+  // lane owns one element and stores 2 bytes per state and step, 9.4 M store instructions per launch at B = 256; here
+  // the compute waves leave the step's states and cache values in LDS as they lie in memory, two buffers by step
+  // parity, and the producer wave stores them one step later in 16-byte pieces.
+  constexpr bool PST = PSTV && PW && KW == 1;
+  constexpr int NCP_O = CacheBlk<T, (NC > 0 ? NC : 1)>::NCP;
+  constexpr int OB_ST = S * TR * D, OB_CA = NC > 0 ? UT_WG * TR * 16 * NCP_O : 0, OB = OB_ST + OB_CA;  // [state][row][unit] [tile][row][unit][value]
+  __shared__ __attribute__((aligned(16))) T obuf[PST ? 2 * OB : 1];
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
 
@@ -171,6 +181,38 @@ fused_fwd_kernel(const FwdArgs a) {
         for (int i = 0; i < NCH; ++i)
           *reinterpret_cast<uint4*>(wbuf + (pl[i] >= 0 ? (s_ & 1) * WBUF + pl[i] : 2 * WBUF)) = make_uint4(src[i].v[0], src[i].v[1], src[i].v[2], src[i].v[3]);
       };
+      // producer-wave stores: the 16-byte pieces of a step's outputs that this lane stores (states, then gate cache)
+      constexpr int SP_TOT = PST ? S * TR * (D / 8) : 0, NSP = (SP_TOT + 63) / 64;
+      constexpr int CPR = NCP_O * 2;  // pieces per (tile, batch row) of the cache
+      constexpr int CP_TOT = PST && NC > 0 ? UT_WG * TR * CPR : 0, NCQ = (CP_TOT + 63) / 64;
+      unsigned svo[NSP > 0 ? NSP : 1], cvo[NCQ > 0 ? NCQ : 1]; int sl[NSP > 0 ? NSP : 1], cl[NCQ > 0 ? NCQ : 1];
+#pragma unroll
+      for (int i = 0; i < NSP; ++i) {
+        const int c = lane + 64 * i, ch = c % (D / 8), pr = (c / (D / 8)) % TR, pk = c / ((D / 8) * TR);
+        const bool ok = c < SP_TOT && bt * TR + pr < B;
+        svo[i] = ok ? ((((unsigned)(pk * B + bt * TR + pr) * Tn) * ND + n * D + ch * 8) * ES) : kInvalidOff;
+        sl[i] = c < SP_TOT ? (pk * TR + pr) * D + ch * 8 : 0;
+      }
+#pragma unroll
+      for (int i = 0; i < NCQ; ++i) {
+        const int c = lane + 64 * i, q = c % CPR, pr = (c / CPR) % TR, ptile = c / (CPR * TR);
+        const bool ok = c < CP_TOT && bt * TR + pr < B && a.training;
+        cvo[i] = ok ? ((((unsigned)ptile * Bpad + bt * TR + pr) * 16) * NCP_O * ES + q * 16) : kInvalidOff;
+        cl[i] = c < CP_TOT ? OB_ST + ((ptile * TR + pr) * 16) * NCP_O + q * 8 : 0;
+      }
+      auto drain = [&](int s_) __attribute__((always_inline)) {  // the outputs of step s_, complete in obuf[s_ & 1]
+        const T* const ob = obuf + (s_ & 1) * OB;
+#pragma unroll
+        for (int i = 0; i < NSP; ++i) {
+          const uint4 v = *reinterpret_cast<const uint4*>(ob + sl[i]);
+          buf_store<4>(Dw<4>{{v.x, v.y, v.z, v.w}}, rSt, svo[i], (unsigned)s_ * ND * ES);
+        }
+#pragma unroll
+        for (int i = 0; i < NCQ; ++i) {
+          const uint4 v = *reinterpret_cast<const uint4*>(ob + cl[i]);
+          buf_store<4>(Dw<4>{{v.x, v.y, v.z, v.w}}, rCa, cvo[i], (((unsigned)s_ * N + n) * (D / 16)) * Bpad * 16 * NCP_O * ES);
+        }
+      };
       fetch(set[0], 0); fetch(set[1], 1); fetch(set[2], 2);
       put(set[0], 0);
       __syncthreads();  // (the one of the prologue below)
@@ -182,6 +224,7 @@ fused_fwd_kernel(const FwdArgs a) {
           else lds_barrier();
         }
         put(next, t + 1);
+        if constexpr (PST) { if (t > 0) drain(t - 1); }
         fetch(refill, t + 3);
       };
       int t = 0;
@@ -195,6 +238,10 @@ fused_fwd_kernel(const FwdArgs a) {
       if (!pdead && t < Tn) {
         iter(t, set[1], set[0]);
         if (!pdead && t + 1 < Tn) iter(t + 1, set[2], set[1]);
+      }
+      if constexpr (PST) {  // the last step's outputs, behind the barrier that follows the time loop
+        lds_barrier();
+        drain(Tn - 1);
       }
       return;
     }
@@ -599,6 +646,21 @@ fused_fwd_kernel(const FwdArgs a) {
 #pragma unroll
         for (int k = 0; k < S; ++k) sbits[k] = mb_bits<T>(so[k][0]);
         mb_store<RO::DW>(mb_pack<T, S>(sbits, t), rOut, mo_v[u], mslot * (unsigned)a.out_slot);
+      } else if constexpr (PST) {  // outputs to LDS as they lie in memory; the producer wave stores them one step later
+        static_assert(!PST || E == 1, "producer-wave stores: 4-row tiles");
+        T* const ob = obuf + cur * OB;
+#pragma unroll
+        for (int k = 0; k < S; ++k)
+          *reinterpret_cast<unsigned short*>(ob + (k * TR + brow) * D + ub[u] + esub) = (unsigned short)pack<E>(so[k], (T*)0).v[0];
+        if constexpr (NC > 0) {
+          const Dw<NWC> cw = cache_pack<T, NCA, E>(cv);
+          unsigned* const dst = reinterpret_cast<unsigned*>(ob + OB_ST + (((w * UTW + u) * TR + brow) * 16 + (esub & 15)) * NCP);
+          if constexpr (NWC == 2) *reinterpret_cast<uint2*>(dst) = make_uint2(cw.v[0], cw.v[1]);
+          else {
+#pragma unroll
+            for (int i = 0; i < NWC; ++i) dst[i] = cw.v[i];
+          }
+        }
       } else {
 #pragma unroll
       for (int k = 0; k < S; ++k)
@@ -648,6 +710,7 @@ fused_fwd_kernel(const FwdArgs a) {
   for (int j = 0; j < PD; ++j)
     if (!MB && !dead && t + j < Tn) step(t + j, wx[j], wx[(j + PD) % (PD + 1)]);
 
+  if constexpr (PST) lds_barrier();  // (the last step's outputs are in LDS: the producer wave stores them behind this barrier)
 #ifdef FRNN_TRACE
   if (lane == 0 && a.trace) {
     long long* o = a.trace + ((size_t)blockIdx.x * WAVES + w) * 4;

@@ -56,8 +56,9 @@ template <int N> __device__ __forceinline__ void mb_store(const Dw<N>& d, rsrc_t
   else {
     static_assert(N == 4 || N == 8, "1, 2, 4 or 8 dwords");
 #pragma unroll
-    for (int i = 0; i < N; i += 4)
-      __builtin_amdgcn_raw_buffer_store_b128(u32x4{d.v[i], d.v[i + 1], d.v[i + 2], d.v[i + 3]}, r, voff + i * 4, soff, 16);
+    for (int i = 0; i < N; i += 4) {
+      store_b128_safe<16>(d.v[i], d.v[i + 1], d.v[i + 2], d.v[i + 3], r, voff + i * 4, soff);
+    }
   }
 }
 

@@ -57,6 +57,13 @@ constexpr bool fwd_producer_wave(int GR, int D, int WAVES, int UTW, int KW, int 
   if (KW == 1) return esize == 2 && GR >= 3 && TR == 4 && WAVES <= 8 && UTW == 1;
   return esize == 2 && GR == 4 && KW > 1 && TR <= 8 && WAVES == 4 && UTW * GR * (D / 32) * 4 <= (TR == 4 ? 160 : 128);
 }
+// Forward kernel: may the producer wave also store the outputs of a step (16-byte pieces, one step late) instead of the
+// compute lanes (2 bytes per state and lane at 4-row tiles)?  Exists for the heads that run as one workgroup with a
+// producer wave; the host picks these instantiations for launches that fill the device (measured: LSTM B256 N12 D64
+// forward -20 %, but +5-9 % at B = 16, where the stores of the compute lanes are hidden anyway).
+constexpr bool fwd_producer_stores(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize) {
+  return KW == 1 && fwd_producer_wave(GR, D, WAVES, UTW, KW, TR, esize);
+}
 // Backward kernel: the same producer wave for the operands of a step (gate cache, s_(t-1), the cotangent of the
 // states), for the heads that run as one workgroup: there every load of the compute waves is on the chain of dependent
 // steps, and a step (~1600 cycles) is shorter than a fetch from HBM, which their one-step prefetch therefore waits for
