@@ -54,6 +54,7 @@ struct BwdArgs {
   // recompute mode (kernels instantiated with RC = true): no gate cache; the gates of step t are rebuilt from
   // Wx_t, b and R h_(t-1), with h_(t-1) read back from the stored states
   const void* Wx; const void* R; const void* b;
+  int pst;  // host side only: launch the instantiation whose producer wave stores dWx (bwd_producer_stores)
 };
 
 // words (64-bit for fp32 storage, 32-bit otherwise) of one inbox area of one group:
@@ -97,7 +98,7 @@ template <> __device__ __forceinline__ float load_frag_at<float>(const float* p)
 // the cache would have held.  For the sLSTM the stabilised gates exp(i - m') and exp(logsig(f) + m - m')
 // are rebuilt from the stored (rounded) m_(t-2); the larger of the two is still exactly 1, the other carries
 // the rounding error of m_(t-2) as a relative error (2^-9 |m| for bf16).
-template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool RC = false>
+template <int F, typename T, int D, int WAVES, int UTW, int KW, int TR, bool RC = false, bool PSTV = false>
 __global__ void __launch_bounds__((WAVES + (bwd_producer_wave(Cell<F>::GR, Cell<F>::NC, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC) ? 1 : 0)) * 64)
 fused_bwd_kernel(const BwdArgs a) {
   typedef Cell<F> C;
@@ -185,6 +186,14 @@ fused_bwd_kernel(const BwdArgs a) {
   constexpr int PB_CA = NC > 0 ? UT_WG * TR * 16 * NCP : 0, PB_ST = S * UT_WG * TR * 16, PB = PB_CA + 2 * PB_ST;
   static_assert(!PW || 2 * PB * (int)sizeof(T) + 16 == bwd_producer_bytes(NC, S, UT_WG, TR, (int)sizeof(T)), "hand-over buffer size");
   T* const pbuf = reinterpret_cast<T*>(smem_raw + bwd_lds_bytes(GR, D, WAVES, UTW, KW, (int)sizeof(T)));
+  // Producer-wave stores (PSTV instantiations, chosen on the host for launches that fill the device; see the forward
+  // kernel): the compute waves leave dWx_t (and the GRU's g-gate cotangent) in LDS as they lie in memory, two buffers by
+  // iteration parity behind the hand-over buffers, and the producer wave stores them in 16-byte pieces behind the
+  // barrier of the step.
+  constexpr bool PST = PSTV && bwd_producer_stores(GR, NC, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC);
+  constexpr int DB_W = GW * TR * D, DB_X = F == FRNN_GRU ? TR * D : 0, DB = DB_W + DB_X;  // [gate][row][unit] [row][unit]
+  static_assert(!PST || DB * 2 * (int)sizeof(T) == bwd_producer_store_bytes(GW, F == FRNN_GRU, D, TR, (int)sizeof(T)), "dWx hand-over size");
+  T* const dbuf = pbuf + 2 * PB + 8;
   if constexpr (PW) {
     if (w == WAVES) {
       constexpr int CPR = NCP * 2;  // 16-byte pieces per (tile, batch row) of the cache
@@ -235,6 +244,38 @@ fused_bwd_kernel(const BwdArgs a) {
           *reinterpret_cast<uint4*>(sl[i] >= 0 ? pb + PB_CA + PB_ST + sl[i] : spare) = make_uint4(o.dso[i].v[0], o.dso[i].v[1], o.dso[i].v[2], o.dso[i].v[3]);
         }
       };
+      // producer-wave stores: the 16-byte pieces of a step's dWx (and dgx) that this lane stores
+      constexpr int WP_TOT = PST ? GW * TR * (D / 8) : 0, NWP = (WP_TOT + 63) / 64;
+      constexpr int XP_TOT = PST && F == FRNN_GRU ? TR * (D / 8) : 0, NXP = (XP_TOT + 63) / 64;
+      unsigned wvo[NWP > 0 ? NWP : 1], xvo[NXP > 0 ? NXP : 1]; int wl[NWP > 0 ? NWP : 1], xl[NXP > 0 ? NXP : 1];
+#pragma unroll
+      for (int i = 0; i < NWP; ++i) {
+        const int c = lane + 64 * i, ch = c % (D / 8), pr = (c / (D / 8)) % TR, pg = c / ((D / 8) * TR);
+        const bool ok = c < WP_TOT && bt * TR + pr < B;
+        wvo[i] = ok ? ((((unsigned)(bt * TR + pr) * Tn * GW + pg) * ND + n * D + ch * 8) * ES) : kInvalidOff;  // + t * GW * ND * ES
+        wl[i] = c < WP_TOT ? (pg * TR + pr) * D + ch * 8 : 0;
+      }
+#pragma unroll
+      for (int i = 0; i < NXP; ++i) {
+        const int c = lane + 64 * i, ch = c % (D / 8), pr = c / (D / 8);
+        const bool ok = c < XP_TOT && bt * TR + pr < B;
+        xvo[i] = ok ? (((unsigned)(bt * TR + pr) * Tn * ND + n * D + ch * 8) * ES) : kInvalidOff;  // + t * ND * ES
+        xl[i] = c < XP_TOT ? DB_W + pr * D + ch * 8 : 0;
+      }
+      auto drain = [&](int i_) __attribute__((always_inline)) {  // dWx of iteration i_ (step T-1-i_), complete in dbuf[i_ & 1]
+        const T* const db = dbuf + (i_ & 1) * DB;
+        const unsigned t = (unsigned)(Tn - 1 - i_);
+#pragma unroll
+        for (int i = 0; i < NWP; ++i) {
+          const uint4 v = *reinterpret_cast<const uint4*>(db + wl[i]);
+          buf_store<4>(Dw<4>{{v.x, v.y, v.z, v.w}}, rDw, wvo[i], t * GW * ND * ES);
+        }
+#pragma unroll
+        for (int i = 0; i < NXP; ++i) {
+          const uint4 v = *reinterpret_cast<const uint4*>(db + xl[i]);
+          buf_store<4>(Dw<4>{{v.x, v.y, v.z, v.w}}, rDx, xvo[i], t * ND * ES);
+        }
+      };
       fetch(set[1], 1); fetch(set[2], 2); fetch(set[0], 3);
       put(set[1], 1);
       __syncthreads();  // (the one of the prologue below)
@@ -243,6 +284,7 @@ fused_bwd_kernel(const BwdArgs a) {
         auto iter = [&](int i, const Ops& next, Ops& refill) __attribute__((always_inline)) {
           if (barrier_or(false, dead_flag)) { pdead = true; return; }
           put(next, i + 2);
+          if constexpr (PST) drain(i);
           fetch(refill, i + 4);
         };
         int i = 0;
@@ -641,6 +683,13 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
         for (int g = 0; g < GW; ++g) dwp[u][g] = pack<E>(dgw[g], (T*)0);
         if (F == FRNN_GRU) dxp[u] = pack<E>(dgr[0], (T*)0);
+      } else if constexpr (PST && !cut) {  // to LDS as they lie in memory; the producer wave stores them behind this step's barrier
+        T* const db = dbuf + ((Tn - 1 - t) & 1) * DB;
+#pragma unroll
+        for (int g = 0; g < GW; ++g)
+          *reinterpret_cast<unsigned short*>(db + (g * TR + brow) * D + ub[u] + esub) = (unsigned short)pack<E>(dgw[g], (T*)0).v[0];
+        if (F == FRNN_GRU)
+          *reinterpret_cast<unsigned short*>(db + DB_W + brow * D + ub[u] + esub) = (unsigned short)pack<E>(dgr[0], (T*)0).v[0];
       } else {
 #pragma unroll
         for (int g = 0; g < GW; ++g)

@@ -81,6 +81,16 @@ constexpr bool bwd_producer_wave(int GR, int nc, int D, int WAVES, int UTW, int 
 constexpr int bwd_producer_bytes(int nc, int s, int ut_wg, int TR, int esize) {
   return 2 * ut_wg * TR * 16 * ((nc + 1) / 2 * 2 + 2 * s) * esize + 16;
 }
+// Backward kernel: may the producer wave also store dWx (see fwd_producer_stores)?  Not the 8-wave kernels: nine waves
+// have 170 registers each and the fp16 LSTM kernel spills with the extra addresses.
+constexpr bool bwd_producer_stores(int GR, int nc, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
+  return bwd_producer_wave(GR, nc, D, WAVES, UTW, KW, TR, esize, rc) && WAVES <= 6;
+}
+// Backward kernel: LDS bytes of the two dWx hand-over buffers of the producer-store instantiations
+// ([gate][row][unit], and [row][unit] for the GRU's g-gate cotangent), behind the operand hand-over buffers
+constexpr int bwd_producer_store_bytes(int gw, bool gru, int D, int TR, int esize) {
+  return 2 * (gw * TR * D + (gru ? TR * D : 0)) * esize;
+}
 // Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
 // 2..16 workgroups (up to 12 where part of the operand lives in LDS) whose slice is a whole number of k-steps; not the fp32
 // kernels whose operand alone takes 256 registers, at the tile heights where they keep 2 or 4 elements per lane

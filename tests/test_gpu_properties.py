@@ -332,3 +332,30 @@ def test_slstm_backward_through_the_carried_state_of_two_calls(gpu, backend):
         assert_close(f"state {k}", out[k].detach().cpu(), ref_out[k], "float32", "state")
     for name, g, r in zip(("dWx", "dR", "db", "ds0"), grads, ref_g):
         assert_close(name, g.cpu(), r, "float32", "token")
+
+
+@pytest.mark.parametrize("function,B,T,N,D,dtype", [
+    ("lstm", 9, 11, 3, 64, "bfloat16"), ("lstm", 6, 7, 5, 32, "bfloat16"), ("lstm", 5, 6, 2, 128, "bfloat16"),
+    ("slstm", 7, 9, 2, 64, "bfloat16"), ("slstm", 4, 5, 3, 32, "float16"), ("gru", 10, 8, 2, 64, "bfloat16"),
+    ("gru", 3, 6, 4, 32, "bfloat16"), ("gru", 6, 5, 1, 96, "float16"), ("lstm", 4, 1, 2, 64, "bfloat16")])
+def test_producer_wave_stores_give_the_same_bits(gpu, monkeypatch, function, B, T, N, D, dtype):
+    """The instantiations whose producer wave stores the outputs (forward: states and gate cache; backward: dWx), which
+    the host picks for launches that fill the device, only move data differently: every output and gradient must come
+    out bit for bit as with the compute lanes' own stores."""
+    from flashrnn_amd import flashrnn
+
+    print(f"case producer stores {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
+    kdt = {"bfloat16": torch.bfloat16, "float16": torch.float16}[dtype]
+    inp = make_inputs(function, B, T, N, D, 41, init="randn", round_to=kdt)
+    res = {}
+    for flag in ("0", "1"):
+        monkeypatch.setenv("FRNN_PRODUCER_STORES", flag)
+        leaves = [inp[k].to(gpu, kdt).requires_grad_() for k in ("Wx", "R", "b", "states")]
+        out, last = flashrnn(*leaves, function=function, backend="hip_fused", dtype=dtype)
+        grads = torch.autograd.grad(out, leaves, grad_outputs=inp["dstates"].to(gpu, kdt))
+        with torch.no_grad():  # the inference forward (no gate cache) as well
+            out2, _ = flashrnn(*[x.detach() for x in leaves], function=function, backend="hip_fused", dtype=dtype)
+        torch.cuda.synchronize()
+        res[flag] = [out.detach(), out2] + [g.detach() for g in grads]
+    for a, b in zip(res["0"], res["1"]):
+        assert torch.equal(a, b), f"max diff {(a.float() - b.float()).abs().max().item():.3e}"
