@@ -29,11 +29,12 @@ WORKLOADS = {
 }
 GATES_R = {"lstm": 4, "slstm": 4, "gru": 3, "elman": 1}
 PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, published
-# roofline.traffic comes from the committed counter profile of the same command, never from a constant in this file:
-# the profile holds one "traffic:" line per kernel template it measured (FETCH_SIZE and WRITE_SIZE in KiB per
-# dispatch and the factors a plain 256 MiB copy gave in the same run).  If the kernel that ran here is not the
-# template that was profiled (another tiling, tile height or mode), traffic is null and the reason is given.
-TRAFFIC_PROFILE = os.path.join(ROOT, "profiles", "fused_kernels_lstm_bf16_B8_T1024_N3_D256_hbm_traffic.txt")
+# roofline.traffic comes from the committed counter profiles of the same commands, never from a constant in this file:
+# a profile holds one "traffic:" line per kernel template it measured (FETCH_SIZE and WRITE_SIZE in KiB per dispatch
+# and the factors a plain 256 MiB copy gave in the same run; for the alternating backend per call, all step launches
+# together).  Every profiles/*_counters*.txt is searched.  If the kernel that ran here is not a template that was
+# profiled (another tiling, tile height or mode), traffic is null and the reason is given.
+PROFILES = os.path.join(ROOT, "profiles")
 CELL_NAMES = {"lstm": "LSTM", "slstm": "sLSTM", "gru": "GRU", "elman": "Elman"}
 
 
@@ -52,22 +53,34 @@ def kernel_template(w, kernel, recompute):
 
 def profiled_traffic(w, kernel, recompute):
     """(bytes per launch or None, note)."""
-    try:
-        name = kernel_template(w, kernel, recompute)
-    except Exception as e:  # no fused plan (alternating backend)
-        return None, f"no fused kernel template for this run ({e})"
+    import glob
+
+    if kernel in ("alt_forward_steps", "alt_backward_steps"):
+        name = kernel  # (the benchmark's launch is the whole scan: every step kernel of one call)
+        wanted = f"{w['function']}_{ {'bfloat16': 'bf16', 'float32': 'f32', 'float16': 'f16'}[w['dtype']] }_B{w['B']}_T{w['T']}_N{w['N']}_D{w['D']}".replace(" ", "")
+    else:
+        wanted = None
+        try:
+            name = kernel_template(w, kernel, recompute)
+        except Exception as e:
+            return None, f"no fused kernel template for this run ({e})"
     mode = "recomputed" if recompute else "stored"
-    try:
-        lines = [l for l in open(TRAFFIC_PROFILE) if l.startswith("traffic:")]
-    except OSError:
-        return None, f"{os.path.relpath(TRAFFIC_PROFILE, ROOT)} is missing"
-    for l in lines:
-        f = dict(x.split("=", 1) for x in l.split()[1:])
-        if f["kernel"] == name and f["mode"] == mode:
-            b = float(f["fetch_kib"]) * 1024 / float(f["fetch_factor"]) + float(f["write_kib"]) * 1024 / float(f["write_factor"])
-            return b, (f"{os.path.relpath(TRAFFIC_PROFILE, ROOT)}: FETCH_SIZE {f['fetch_kib']} KiB / {f['fetch_factor']} + "
-                       f"WRITE_SIZE {f['write_kib']} KiB / {f['write_factor']} (factors of a plain 256 MiB copy in the same run)")
-    return None, f"the committed profile has no entry for {name} (gate cache {mode}): not measured"
+    files = sorted(glob.glob(os.path.join(PROFILES, "*counters*.txt")))
+    if not files:
+        return None, "no counter profiles under profiles/"
+    for path in files:
+        if wanted is not None and wanted not in os.path.basename(path):
+            continue  # (an aggregate of step kernels only means something for the workload it was measured on)
+        for l in open(path):
+            if not l.startswith("traffic:"):
+                continue
+            f = dict(x.split("=", 1) for x in l.split()[1:])
+            if f["kernel"] == name and f["mode"] == mode:
+                b = float(f["fetch_kib"]) * 1024 / float(f["fetch_factor"]) + float(f["write_kib"]) * 1024 / float(f["write_factor"])
+                rel = os.path.relpath(path, ROOT)
+                return b, (f"{rel}: FETCH_SIZE {f['fetch_kib']} KiB / {f['fetch_factor']} + WRITE_SIZE {f['write_kib']} KiB / "
+                           f"{f['write_factor']} (factors of a plain 256 MiB copy in the same run)")
+    return None, f"no committed profile has an entry for {name} (gate cache {mode}): not measured"
 
 
 def describe(w):
