@@ -191,7 +191,8 @@ fused_bwd_kernel(const BwdArgs a) {
   // iteration parity behind the hand-over buffers, and the producer wave stores them in 16-byte pieces behind the
   // barrier of the step.
   constexpr bool PST = PSTV && bwd_producer_stores(GR, NC, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC);
-  constexpr int DB_W = GW * TR * D, DB_X = F == FRNN_GRU ? TR * D : 0, DB = DB_W + DB_X;  // [gate][row][unit] [row][unit]
+  constexpr int DBR = D + 8;  // (row stride: see the forward kernel)
+  constexpr int DB_W = GW * TR * DBR, DB_X = F == FRNN_GRU ? TR * DBR : 0, DB = DB_W + DB_X;  // [gate][row][unit] [row][unit]
   static_assert(!PST || DB * 2 * (int)sizeof(T) == bwd_producer_store_bytes(GW, F == FRNN_GRU, D, TR, (int)sizeof(T)), "dWx hand-over size");
   T* const dbuf = pbuf + 2 * PB + 8;
   if constexpr (PW) {
@@ -253,14 +254,14 @@ fused_bwd_kernel(const BwdArgs a) {
         const int c = lane + 64 * i, ch = c % (D / 8), pr = (c / (D / 8)) % TR, pg = c / ((D / 8) * TR);
         const bool ok = c < WP_TOT && bt * TR + pr < B;
         wvo[i] = ok ? ((((unsigned)(bt * TR + pr) * Tn * GW + pg) * ND + n * D + ch * 8) * ES) : kInvalidOff;  // + t * GW * ND * ES
-        wl[i] = c < WP_TOT ? (pg * TR + pr) * D + ch * 8 : 0;
+        wl[i] = c < WP_TOT ? (pg * TR + pr) * DBR + ch * 8 : 0;
       }
 #pragma unroll
       for (int i = 0; i < NXP; ++i) {
         const int c = lane + 64 * i, ch = c % (D / 8), pr = c / (D / 8);
         const bool ok = c < XP_TOT && bt * TR + pr < B;
         xvo[i] = ok ? (((unsigned)(bt * TR + pr) * Tn * ND + n * D + ch * 8) * ES) : kInvalidOff;  // + t * ND * ES
-        xl[i] = c < XP_TOT ? DB_W + pr * D + ch * 8 : 0;
+        xl[i] = c < XP_TOT ? DB_W + pr * DBR + ch * 8 : 0;
       }
       auto drain = [&](int i_) __attribute__((always_inline)) {  // dWx of iteration i_ (step T-1-i_), complete in dbuf[i_ & 1]
         const T* const db = dbuf + (i_ & 1) * DB;
@@ -687,9 +688,9 @@ fused_bwd_kernel(const BwdArgs a) {
         T* const db = dbuf + ((Tn - 1 - t) & 1) * DB;
 #pragma unroll
         for (int g = 0; g < GW; ++g)
-          *reinterpret_cast<unsigned short*>(db + (g * TR + brow) * D + ub[u] + esub) = (unsigned short)pack<E>(dgw[g], (T*)0).v[0];
+          *reinterpret_cast<unsigned short*>(db + (g * TR + brow) * DBR + ub[u] + esub) = (unsigned short)pack<E>(dgw[g], (T*)0).v[0];
         if (F == FRNN_GRU)
-          *reinterpret_cast<unsigned short*>(db + DB_W + brow * D + ub[u] + esub) = (unsigned short)pack<E>(dgr[0], (T*)0).v[0];
+          *reinterpret_cast<unsigned short*>(db + DB_W + brow * DBR + ub[u] + esub) = (unsigned short)pack<E>(dgr[0], (T*)0).v[0];
       } else {
 #pragma unroll
         for (int g = 0; g < GW; ++g)

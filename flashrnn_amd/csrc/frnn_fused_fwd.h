@@ -122,7 +122,10 @@ fused_fwd_kernel(const FwdArgs a) {
   // parity, and the producer wave stores them one step later in 16-byte pieces.
   constexpr bool PST = PSTV && PW && KW == 1;
   constexpr int NCP_O = CacheBlk<T, (NC > 0 ? NC : 1)>::NCP;
-  constexpr int OB_ST = S * TR * D, OB_CA = NC > 0 ? UT_WG * TR * 16 * NCP_O : 0, OB = OB_ST + OB_CA;  // [state][row][unit] [tile][row][unit][value]
+  // (rows of the state part are D + 8 elements apart: at a stride of 128 bytes, D = 64, rows 0 and 2 of a tile would meet
+  // in the same banks under the lanes' 2-byte writes)
+  constexpr int OBR = D + 8;
+  constexpr int OB_ST = S * TR * OBR, OB_CA = NC > 0 ? UT_WG * TR * 16 * NCP_O : 0, OB = OB_ST + OB_CA;  // [state][row][unit] [tile][row][unit][value]
   __shared__ __attribute__((aligned(16))) T obuf[PST ? 2 * OB : 1];
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
@@ -191,7 +194,7 @@ fused_fwd_kernel(const FwdArgs a) {
         const int c = lane + 64 * i, ch = c % (D / 8), pr = (c / (D / 8)) % TR, pk = c / ((D / 8) * TR);
         const bool ok = c < SP_TOT && bt * TR + pr < B;
         svo[i] = ok ? ((((unsigned)(pk * B + bt * TR + pr) * Tn) * ND + n * D + ch * 8) * ES) : kInvalidOff;
-        sl[i] = c < SP_TOT ? (pk * TR + pr) * D + ch * 8 : 0;
+        sl[i] = c < SP_TOT ? (pk * TR + pr) * OBR + ch * 8 : 0;
       }
 #pragma unroll
       for (int i = 0; i < NCQ; ++i) {
@@ -651,7 +654,7 @@ fused_fwd_kernel(const FwdArgs a) {
         T* const ob = obuf + cur * OB;
 #pragma unroll
         for (int k = 0; k < S; ++k)
-          *reinterpret_cast<unsigned short*>(ob + (k * TR + brow) * D + ub[u] + esub) = (unsigned short)pack<E>(so[k], (T*)0).v[0];
+          *reinterpret_cast<unsigned short*>(ob + (k * TR + brow) * OBR + ub[u] + esub) = (unsigned short)pack<E>(so[k], (T*)0).v[0];
         if constexpr (NC > 0) {
           const Dw<NWC> cw = cache_pack<T, NCA, E>(cv);
           unsigned* const dst = reinterpret_cast<unsigned*>(ob + OB_ST + (((w * UTW + u) * TR + brow) * 16 + (esub & 15)) * NCP);

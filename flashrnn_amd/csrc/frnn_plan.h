@@ -89,7 +89,7 @@ constexpr bool bwd_producer_stores(int GR, int nc, int D, int WAVES, int UTW, in
 // Backward kernel: LDS bytes of the two dWx hand-over buffers of the producer-store instantiations
 // ([gate][row][unit], and [row][unit] for the GRU's g-gate cotangent), behind the operand hand-over buffers
 constexpr int bwd_producer_store_bytes(int gw, bool gru, int D, int TR, int esize) {
-  return 2 * (gw * TR * D + (gru ? TR * D : 0)) * esize;
+  return 2 * (gw * TR * (D + 8) + (gru ? TR * (D + 8) : 0)) * esize;
 }
 // Forward kernel: do the k-steps over the workgroup's own slice of h run in front of the exchange wait?  Heads of
 // 2..16 workgroups (up to 12 where part of the operand lives in LDS) whose slice is a whole number of k-steps; not the fp32

@@ -7,16 +7,20 @@ of the oracle fed the same bf16-rounded inputs):
   bf16   h (state 0):       max|err| <= 2e-2
          other states:      |err| <= 2e-2 * max(1, |ref|) element-wise (c, n, m are not bounded by
                             1; bf16 storage alone is off by 0.03 at |x| = 8)
-         dWx, dstates0:     |err| <= max(2e-2 * max(1, |ref|), 5e-3 * max|ref|) element-wise: the
+         dWx, dstates0:     |err| <= max(2e-2 * max(1, |ref|), 5e-3 * max|ref|) element-wise (1e-2 * max|ref| for
+                            the cotangents of the sLSTM's initial c and n, whose errors multiply up through
+                            one stored, rounded exponential gate per step): the
                             outputs are stored in bf16, whose own rounding is relative (half an ulp
                             is 0.016 at |x| = 4), and the recurrent cotangent of every unit is a
                             product with R^T, so an element's error follows the size of the whole
                             cotangent vector rather than its own
-         dR, db:            max|err| <= max(2e-2, 1e-2 * max|ref|): they are sums over B*T tokens of
+         dR, db:            max|err| <= max(2e-2, 6e-3 * max|ref|): they are sums over B*T tokens of
                             products of bf16-stored factors (h, dg), each carrying a relative
                             rounding error of 2^-9, so the error of the sum grows like sqrt(B*T)
-                            (measured 0.17 on |dR| <= 56 at B*T = 8192); the kernel accumulates and
-                            returns them in fp32.
+                            (measured at the full-size configurations: 1.6e-3 .. 4.3e-3 of max|ref|);
+                            the kernel accumulates and returns them in fp32.  The full-size
+                            configurations additionally carry absolute bounds of twice the error
+                            measured there (``sum_bounds``).
   fp16   as bf16 with every bound divided by 4 (3 more mantissa bits; the reference states no
          fp16 tolerance).
 On top of the element-wise bounds, for the 16-bit types:
@@ -95,7 +99,7 @@ def assert_not_worse_than(name, got, other, ref):
         f"{name}: Frobenius error {float(e.norm()):.3e} exceeds that of the bf16 vanilla run, {float(eo.norm()):.3e}"
 
 
-REL_F = {"h": 3e-3, "state": 3e-3, "token": 8e-3, "sum": 8e-3}   # bf16; fp16: / 4
+REL_F = {"h": 3e-3, "state": 3e-3, "token": 8e-3, "token_gated": 8e-3, "sum": 8e-3}   # bf16; fp16: / 4
 
 
 def assert_close(name, got, ref, dtype, kind):
@@ -115,17 +119,19 @@ def assert_close(name, got, ref, dtype, kind):
     elif kind == "state":
         bad = err > 2e-2 * q * torch.clamp(ref.abs(), min=1.0)
         assert not bool(bad.any()), f"{name}: max err {float(err.max()):.3e} (|ref| there {float(ref.abs()[err.argmax()]) if err.dim()==1 else float(ref.abs().flatten()[err.argmax()]):.2f})"
-    elif kind == "token":
-        tol = torch.clamp(2e-2 * q * torch.clamp(ref.abs(), min=1.0), min=5e-3 * q * float(ref.abs().max()))
+    elif kind in ("token", "token_gated"):
+        # (token_gated: the cotangents of the sLSTM's initial c and n pass through one stored, rounded exponential gate per
+        # step, so their rounding errors multiply up along the sequence: 1e-2 of the largest element instead of 5e-3)
+        tol = torch.clamp(2e-2 * q * torch.clamp(ref.abs(), min=1.0), min=(1e-2 if kind == "token_gated" else 5e-3) * q * float(ref.abs().max()))
         bad = err > tol
         assert not bool(bad.any()), f"{name}: max err {float(err.max()):.3e}, max ref {float(ref.abs().max()):.2f}"
     else:  # sums over B*T tokens
-        tol = max(2e-2 * q, 1e-2 * q * float(ref.abs().max()))
+        tol = max(2e-2 * q, 6e-3 * q * float(ref.abs().max()))
         assert float(err.max()) <= tol, f"{name}: max err {float(err.max()):.3e} > {tol:.3e}"
 
 
 def check_case(device, function, B, T, N, D, dtype, backend, seed=1, init="randn", backward=True,
-               forget_bias_linspace=False, options=None, grad_on="all", vs_bf16_vanilla=False):
+               forget_bias_linspace=False, options=None, grad_on="all", vs_bf16_vanilla=False, sum_bounds=None):
     inp = make_inputs(function, B, T, N, D, seed, init=init,
                       round_to={"bfloat16": torch.bfloat16, "float16": torch.float16}.get(dtype), grad_on=grad_on,
                       forget_bias_linspace=forget_bias_linspace)
@@ -142,11 +148,16 @@ def check_case(device, function, B, T, N, D, dtype, backend, seed=1, init="randn
         assert_close("dWx", grads[0], ref_g[0], dtype, "token")
         assert_close("dR", grads[1], ref_g[1], dtype, "sum")
         assert_close("db", grads[2], ref_g[2], dtype, "sum")
+        if sum_bounds is not None:  # absolute max-abs bounds of this configuration: twice the error measured on it
+            for name, g, r in (("dR", grads[1], ref_g[1]), ("db", grads[2], ref_g[2])):
+                e = float((g.double() - r.double()).abs().max())
+                print(f"  {name}: max abs err {e:.3e} (max |ref| {float(r.abs().max()):.1f}, bound {sum_bounds[name]:.2e})", flush=True)
+                assert e <= sum_bounds[name], f"{name}: max abs err {e:.3e} > {sum_bounds[name]:.2e}"
         for k in range(S):
             if function == "slstm" and k == 3:
                 assert float(grads[3][k].abs().max()) == 0.0  # the stabiliser is held constant: d/dm0 = 0
                 continue
-            assert_close(f"dstates0[{k}]", grads[3][k], ref_g[3][k], dtype, "token")
+            assert_close(f"dstates0[{k}]", grads[3][k], ref_g[3][k], dtype, "token_gated" if function == "slstm" and k > 0 else "token")
     if vs_bf16_vanilla:
         assert dtype == "bfloat16" and not (set(options or {}) - {"recompute_gates"})
         v_out, v_g = bf16_vanilla_run(function, inp, backward)

@@ -219,31 +219,41 @@ def test_config1_lstm_fp32_forward(gpu):
     check_case(gpu, "lstm", 4, 256, 1, 64, "float32", "hip", seed=1001, init="zeros", backward=False)
 
 
+# Absolute max-abs bounds on the weight gradients of the full-size configurations: twice the larger of the two backends'
+# measured errors (dR, db are sums over B*T tokens of bf16-stored factors; the general bound is relative to max|ref|).
+# Measured (hip_fused / hip): C2 dR 0.179 / 0.167 (max |ref| 56), db 0.50 / 0.62 (224); C3 dR 0.35 / 0.36 (96), db 0.67 / 0.90
+# (408); C4 dR 0.095 / 0.096 (32.5), db 0.71 / 0.70 (254); C5 dR 2.27 / 2.18 (534), db 2.38 / 1.88 (587).
+SUM_BOUNDS = {"C2": {"dR": 0.36, "db": 1.24}, "C3": {"dR": 0.72, "db": 1.8}, "C4": {"dR": 0.19, "db": 1.42}, "C5": {"dR": 4.5, "db": 4.8}}
+
+
 # Full size, both backends; besides the fp32 oracle every bf16 configuration is also held against the
 # oracle run in torch.bfloat16 (the reference's vanilla backend in bf16): the HIP path must be closer.
 @pytest.mark.parametrize("backend", ["hip_fused", "hip"])
 def test_config2_lstm_bf16_full_size(gpu, backend):
     print(f"case C2 full {backend}", flush=True)
-    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", backend, seed=1002, init="randn", vs_bf16_vanilla=True)
+    check_case(gpu, "lstm", 8, 1024, 3, 256, "bfloat16", backend, seed=1002, init="randn", vs_bf16_vanilla=True,
+               sum_bounds=SUM_BOUNDS["C2"])
 
 
 @pytest.mark.parametrize("backend", ["hip_fused", "hip"])
 def test_config3_gru_bf16_full_size(gpu, backend):
     print(f"case C3 full {backend}", flush=True)
-    check_case(gpu, "gru", 16, 2048, 4, 128, "bfloat16", backend, seed=1003, init="zeros", vs_bf16_vanilla=True)
+    check_case(gpu, "gru", 16, 2048, 4, 128, "bfloat16", backend, seed=1003, init="zeros", vs_bf16_vanilla=True,
+               sum_bounds=SUM_BOUNDS["C3"])
 
 
 @pytest.mark.parametrize("backend", ["hip_fused", "hip"])
 def test_config4_slstm_bf16_full_size(gpu, backend):
     print(f"case C4 full {backend}", flush=True)
     check_case(gpu, "slstm", 16, 4096, 4, 192, "bfloat16", backend, seed=1004, init="zeros",
-               forget_bias_linspace=True, grad_on="h", vs_bf16_vanilla=True)
+               forget_bias_linspace=True, grad_on="h", vs_bf16_vanilla=True, sum_bounds=SUM_BOUNDS["C4"])
 
 
 @pytest.mark.parametrize("backend", ["hip", "hip_fused"])
 def test_config5_elman_full_size(gpu, backend):
     print(f"case C5 full {backend}", flush=True)
-    check_case(gpu, "elman", 32, 1024, 1, 1024, "bfloat16", backend, seed=1005, init="zeros", vs_bf16_vanilla=True)
+    check_case(gpu, "elman", 32, 1024, 1, 1024, "bfloat16", backend, seed=1005, init="zeros", vs_bf16_vanilla=True,
+               sum_bounds=SUM_BOUNDS["C5"])
 
 
 @pytest.mark.parametrize("N,D", [(24, 32), (12, 64), (6, 128), (3, 256), (1, 512)])

@@ -359,3 +359,51 @@ def test_producer_wave_stores_give_the_same_bits(gpu, monkeypatch, function, B, 
         res[flag] = [out.detach(), out2] + [g.detach() for g in grads]
     for a, b in zip(res["0"], res["1"]):
         assert torch.equal(a, b), f"max diff {(a.float() - b.float()).abs().max().item():.3e}"
+
+
+def test_a_problem_whose_tensors_pass_2_gib_at_its_real_size(gpu):
+    """LSTM bf16 B = 400, T = 1024, N = 12, D = 64: Wx, dWx and the gate cache are 2.5 GB each, beyond the 32-bit offsets
+    of the fused kernels, so flashrnn() runs the call as batch ranges.  Batch rows are independent: 16 rows (the first 8
+    and the last 8, i.e. both ends of the range split) go through the oracle; dR and db, which sum over all rows, are
+    compared with the alternating backend's on the whole problem (64-bit addressing, one call)."""
+    from flashrnn_amd import flashrnn
+    from oracle import flashrnn_oracle_backward
+    from parity import assert_close
+
+    function, B, T, N, D = "lstm", 400, 1024, 12, 64
+    print(f"case beyond 2 GiB {function} B{B} T{T} N{N} D{D}", flush=True)
+    g = torch.Generator(device=gpu).manual_seed(77)
+    rnd = lambda *shape, scale=1.0: (torch.randn(*shape, generator=g, device=gpu, dtype=torch.float32) * scale).to(torch.bfloat16)
+    Wx = torch.empty((B, T, 4, N, D), dtype=torch.bfloat16, device=gpu)
+    for b0 in range(0, B, 50):  # (drawn in fp32 in slices: the whole tensor in fp32 would be 5 GB more)
+        Wx[b0:b0 + 50] = rnd(50, T, 4, N, D)
+    assert Wx.numel() * 2 >= 2 ** 31
+    R, b, s0 = rnd(4, N, D, D, scale=D ** -0.5), rnd(4, N, D, scale=0.1), rnd(2, B, 1, N, D)
+    ds = torch.empty((2, B, T, N, D), dtype=torch.bfloat16, device=gpu)
+    for b0 in range(0, B, 50):
+        ds[:, b0:b0 + 50] = rnd(2, 50, T, N, D)
+    res = {}
+    for backend in ("hip_fused", "hip"):
+        leaves = [x.clone().requires_grad_() for x in (Wx, R, b, s0)]
+        out, last = flashrnn(*leaves, function=function, backend=backend)
+        grads = torch.autograd.grad(out, leaves, grad_outputs=ds)
+        torch.cuda.synchronize()
+        res[backend] = (out.detach(), [x.detach() for x in grads])
+        del leaves, out, grads
+    rows = list(range(8)) + list(range(B - 8, B))
+    ref_out, ref_g = flashrnn_oracle_backward(Wx[rows].float().cpu(), R.float().cpu(), b.float().cpu(), s0[:, rows].float().cpu(),
+                                              function, ds[:, rows].float().cpu())
+    out, grads = res["hip_fused"]
+    got = out[:, rows].float().cpu()
+    assert_close("h", got[0], ref_out[0], "bfloat16", "h")
+    assert_close("c", got[1], ref_out[1], "bfloat16", "state")
+    assert_close("dWx", grads[0][rows].float().cpu(), ref_g[0], "bfloat16", "token")
+    assert_close("ds0", grads[3][:, rows].float().cpu(), ref_g[3], "bfloat16", "token")
+    # the weight gradients of the two backends: each is within 3e-3 .. 4e-3 of max|ref| of the exact sum
+    for name, i in (("dR", 1), ("db", 2)):
+        a, c = grads[i].float(), res["hip"][1][i].float()
+        e, m = float((a - c).abs().max()), float(c.abs().max())
+        print(f"  {name}: fused (batch ranges) vs alternating: max abs diff {e:.3e}, max |ref| {m:.1f}", flush=True)
+        assert e <= 1e-2 * m, f"{name}: {e:.3e} > 1e-2 * {m:.1f}"
+    assert torch.equal(res["hip_fused"][0][:, rows], res["hip"][0][:, rows]) or \
+        float((res["hip_fused"][0][:, rows].float() - res["hip"][0][:, rows].float()).abs().max()) <= 2e-2

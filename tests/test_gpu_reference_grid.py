@@ -31,8 +31,9 @@ def combos(function):
 def test_reference_size_grid(gpu, function, dtype, backend):
     unsupported = []
     for i, (B, D, T, N) in enumerate(combos(function)):
-        # (every third configuration with gradients, the others forward only: the grid is about shapes)
-        backward = i % 3 == 0
+        # bf16, the type the benchmark configurations use: every shape with all its gradients, as the reference's own
+        # grid (flashrnn/tests/utils.py:257-340); the other two storage types: every third shape, the rest forward only
+        backward = dtype == "bfloat16" or i % 3 == 0
         print(f"case grid {function} {dtype} {backend} B{B} D{D} T{T} N{N} bwd={backward}", flush=True)
         try:
             check_case(gpu, function, B, T, N, D, dtype, backend, seed=100 + i, init="zeros", backward=backward)
