@@ -13,7 +13,7 @@ FUNCTION_IDS = {"lstm": 0, "slstm": 1, "gru": 2, "elman": 3}
 DTYPE_IDS = {"bfloat16": 0, "float32": 1, "float16": 2}
 
 # error codes of include/flashrnn_hip.h
-E_ARG, E_UNSUPPORTED, E_NULL, E_ALIGN, E_WORKSPACE, E_DEVICE = -1, -2, -3, -4, -5, -6
+E_ARG, E_UNSUPPORTED, E_NULL, E_ALIGN, E_WORKSPACE, E_DEVICE, E_TOO_LARGE = -1, -2, -3, -4, -5, -6, -7
 
 
 
@@ -21,11 +21,13 @@ class Options(ctypes.Structure):
     """frnn_options of include/flashrnn_hip.h (0 / False = option off)."""
 
     _fields_ = [("struct_size", ctypes.c_uint), ("forward_clipval", ctypes.c_float),
-                ("gradient_recurrent_clipval", ctypes.c_float), ("gradient_recurrent_cut", c_int), ("recompute", c_int)]
+                ("gradient_recurrent_clipval", ctypes.c_float), ("gradient_recurrent_cut", c_int), ("recompute", c_int),
+                ("batch_stride", c_int)]
 
-    def __init__(self, forward_clipval=0.0, gradient_recurrent_clipval=0.0, gradient_recurrent_cut=0, recompute=0):
+    def __init__(self, forward_clipval=0.0, gradient_recurrent_clipval=0.0, gradient_recurrent_cut=0, recompute=0,
+                 batch_stride=0):
         super().__init__(ctypes.sizeof(Options), forward_clipval, gradient_recurrent_clipval, gradient_recurrent_cut,
-                         recompute)
+                         recompute, batch_stride)
 
 
 _P6 = [c_int] * 6
@@ -58,6 +60,7 @@ _SIGNATURES = {
     "frnn_fused_cache_bytes_opt": (c_size_t, _P6 + [POINTER(Options)]),
     "frnn_alt_cache_bytes_opt": (c_size_t, _P6 + [POINTER(Options)]),
     "frnn_fused_recompute_supported": (c_int, [c_int] * 5),
+    "frnn_fused_max_batch": (c_int, [c_int] * 7 + [POINTER(Options)]),
     "frnn_fused_workspace_bytes_opt": (c_size_t, _P6 + [c_int, POINTER(Options)]),
     "frnn_fused_backward_recompute": (c_int, _P6 + [c_void_p] * 11 + [c_size_t, c_void_p, POINTER(Options)]),
     "frnn_fused_step": (c_int, [c_int] * 5 + [c_void_p] * 7 + [POINTER(Options)]),

@@ -253,9 +253,9 @@ static void gate_leave(LaunchGate* g, hipStream_t st, bool launched_ok = true, b
 // fx is the cell the kernels are instantiated for: the function itself, except that an Elman cell under
 // forward_clipval runs as FRNN_ELMAN_CLIP (one cached value per element: the unclamped h).
 // rc: the gate cache is left out (forward) / rebuilt (backward): only for cells that have one.
-struct Opts { float h_clip, g_clip; int cut; int fx; int rc; };
+struct Opts { float h_clip, g_clip; int cut; int fx; int rc; int bs; };
 static int parse_opts(const frnn_options* o, int function, Opts* out) {
-  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0; out->fx = function; out->rc = 0;
+  out->h_clip = 0.f; out->g_clip = 0.f; out->cut = 0; out->fx = function; out->rc = 0; out->bs = 0;
   if (!o) return 0;
   // (the struct may grow at its end: struct_size says how much of it the caller's build knows)
   if (o->struct_size < offsetof(frnn_options, recompute))
@@ -267,7 +267,9 @@ static int parse_opts(const frnn_options* o, int function, Opts* out) {
                 (double)o->gradient_recurrent_clipval);
   out->h_clip = o->forward_clipval; out->g_clip = o->gradient_recurrent_clipval; out->cut = o->gradient_recurrent_cut != 0;
   if (function == FRNN_ELMAN && out->h_clip > 0.f) out->fx = FRNN_ELMAN_CLIP;
-  out->rc = recompute != 0 && function != FRNN_ELMAN;  // (elman caches nothing, or one value under forward_clipval)
+  out->rc = recompute != 0 && function != FRNN_ELMAN;
+  out->bs = o->struct_size >= offsetof(frnn_options, batch_stride) + sizeof(int) ? o->batch_stride : 0;
+  if (out->bs < 0) return fail(FRNN_E_ARG, "batch_stride must be 0 (= B) or the number of rows of the whole batch (got %d)", out->bs);  // (elman caches nothing, or one value under forward_clipval)
   return 0;
 }
 
@@ -289,13 +291,16 @@ static size_t fused_cache_bytes_of(int function, int dtype, int B, int T, int N,
   return (size_t)T * N * B * D * ncp * dtype_size(dtype);
 }
 // the fused kernels address each tensor with 32-bit byte offsets
-static int check_fused_sizes(int function, int dtype, int B, int T, int N, int D) {
+// bs: rows between the state planes (0: B)
+static int check_fused_sizes(int function, int dtype, int B, int T, int N, int D, int bs = 0, bool with_cache = true) {
   const CellDims c = cell_dims(function);
-  const size_t es = dtype_size(dtype), btnd = (size_t)B * T * N * D;
-  const size_t gmax = (size_t)(c.GW > c.S ? c.GW : c.S);
-  const size_t cache = fused_cache_bytes_of(function, dtype, B, T, N, D);
-  if (btnd * gmax * es >= ((size_t)1 << 31) || cache >= ((size_t)1 << 31))
-    return fail(FRNN_E_ARG, "a tensor of this problem reaches 2 GiB; split the batch (fused kernels use 32-bit offsets)");
+  const size_t es = dtype_size(dtype), tnd = (size_t)T * N * D;
+  if (bs != 0 && bs < B) return fail(FRNN_E_ARG, "batch_stride %d is smaller than the %d rows of the call", bs, B);
+  const size_t planes = ((size_t)(c.S - 1) * (bs ? bs : B) + B) * tnd * es;  // from the first row of plane 0 to the last of plane S-1
+  const size_t cache = with_cache ? fused_cache_bytes_of(function, dtype, B, T, N, D) : 0;
+  if ((size_t)B * tnd * c.GW * es >= ((size_t)1 << 31) || planes >= ((size_t)1 << 31) || cache >= ((size_t)1 << 31))
+    return fail(FRNN_E_TOO_LARGE, "a tensor of this call reaches 2 GiB (the fused kernels use 32-bit offsets): run the batch as ranges "
+                "of at most frnn_fused_max_batch() rows (frnn_options.batch_stride lets them use the full tensors in place)");
   return 0;
 }
 static int check_ptr(const void* p, const char* name) {
@@ -535,6 +540,24 @@ size_t frnn_fused_cache_bytes_opt(int function, int dtype, int B, int T, int N, 
   return o.rc ? 0 : fused_cache_bytes_of(o.fx, dtype, B, T, N, D);
 }
 
+int frnn_fused_max_batch(int function, int dtype, int T, int N, int D, int batch_stride, int training, const frnn_options* opt) {
+  g_err[0] = 0;
+  Opts o;
+  if (check_problem(function, dtype, 1, T, N, D) || parse_opts(opt, function, &o) || batch_stride < 0) return 0;
+  const CellDims c = cell_dims(o.fx);
+  const size_t es = dtype_size(dtype), tnd = (size_t)T * N * D, lim = ((size_t)1 << 31) - 1;
+  size_t rows = lim / (tnd * c.GW * es);
+  const size_t cache_row = (training && !o.rc) ? fused_cache_bytes_of(o.fx, dtype, 1, T, N, D) : 0;
+  if (cache_row) rows = rows < lim / cache_row ? rows : lim / cache_row;
+  if (batch_stride == 0) rows = rows < lim / (tnd * es * c.S) ? rows : lim / (tnd * es * c.S);
+  else {
+    const size_t below = (size_t)(c.S - 1) * batch_stride * tnd * es;
+    const size_t r = below >= lim ? 0 : (lim - below) / (tnd * es);
+    rows = rows < r ? rows : r;
+  }
+  return (int)(rows > 0x3fffffff ? 0x3fffffff : rows);
+}
+
 size_t frnn_fused_workspace_bytes(int function, int dtype, int B, int T, int N, int D, int backward) {
   if (check_problem(function, dtype, B, T, N, D)) return 0;
   Plan p;
@@ -578,7 +601,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   Plan p;
   if (!pick_plan(fx, dtype, B, N, D, 0, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused kernel for function %d dtype %d head dim %d", function, dtype, D);
-  e = check_fused_sizes(fx, dtype, B, T, N, D);
+  e = check_fused_sizes(fx, dtype, B, T, N, D, o.bs, training && !o.rc);
   if (e) return e;
   CHECK_PTR(Wx) CHECK_PTR(R) CHECK_PTR(b) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(workspace)
   if (o.rc) {
@@ -614,7 +637,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   a.ll = w.ll; a.status = w.status;
   a.xcd = (p.kw > 1 && !step && near_stores_allowed()) ? w.xcd : nullptr;
   a.carry = carry; a.step = step;
-  a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
+  a.B = B; a.BS = o.bs ? o.bs : B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
@@ -709,7 +732,7 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   if (!pick_plan(fx, dtype, B, N, D, o.rc ? 2 : 1, &p))
     return fail(FRNN_E_UNSUPPORTED, "no fused%s kernel for function %d dtype %d head dim %d", o.rc ? " recompute-mode" : "",
                 function, dtype, D);
-  e = check_fused_sizes(fx, dtype, B, T, N, D);
+  e = check_fused_sizes(fx, dtype, B, T, N, D, o.bs, !o.rc);
   if (e) return e;
   CHECK_PTR(R) CHECK_PTR(s0) CHECK_PTR(states) CHECK_PTR(dstates)
   CHECK_PTR(dWx) CHECK_PTR(ds0) CHECK_PTR(dR) CHECK_PTR(db) CHECK_PTR(workspace)
@@ -741,7 +764,7 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   a.dWx = dWx; a.dgx = w.dgx; a.ds0 = ds0; a.dbp = w.dbp;
   a.ll = w.ll; a.status = w.status;
   a.xcd = (p.kw > 1 && near_stores_allowed()) ? w.xcd : nullptr;
-  a.B = B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
+  a.B = B; a.BS = o.bs ? o.bs : B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
   // measured best, as in the forward call (exchange stores kept in the XCD's L2): the gated cells 0-2 units at every
@@ -903,7 +926,7 @@ int frnn_fused_decode_open(int function, int dtype, int B, int N, int D,
   a.ll = (u64*)(mb + dp.l.exch_off); a.status = (int*)mb + MB_STATUS;
   a.xcd = (p.kw > 1 && near_stores_allowed()) ? (int*)(mb + dp.l.xcd_off) : nullptr;
   a.carry = carry; a.step = 0;
-  a.B = B; a.T = max_tokens; a.N = N; a.grp0 = 0; a.groups = dp.groups; a.groups_total = dp.groups; a.tile_rows = 4;
+  a.B = B; a.BS = B; a.T = max_tokens; a.N = N; a.grp0 = 0; a.groups = dp.groups; a.groups_total = dp.groups; a.tile_rows = 4;
   a.training = 0;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(function, dtype, p, 4));

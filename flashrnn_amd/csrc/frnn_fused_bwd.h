@@ -46,6 +46,7 @@ struct BwdArgs {
   u64* ll; int* status;
   int* xcd;        // 32 words per group for xcd_handshake (zero at launch), or null: exchange stores stay agent scope
   int B, T, N;
+  int BS;  // rows between the state planes of s0, states, dstates and ds0 ([S, BS, ...]); B unless the call covers a range of a larger batch
   int grp0, groups, groups_total, tile_rows;
   int spin_limit, poll_delay;
   float g_clip;  // > 0: cotangent carried into h_t clamped to [-g_clip, g_clip] (gradient_recurrent_clipval)
@@ -155,7 +156,7 @@ fused_bwd_kernel(const BwdArgs a) {
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
   const int grp = a.grp0 + grp_l;
-  const int N = a.N, Tn = a.T, B = a.B;
+  const int N = a.N, Tn = a.T, B = a.B, BS = a.BS;
   const int n = grp % N, bt = grp / N;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
@@ -166,9 +167,9 @@ fused_bwd_kernel(const BwdArgs a) {
   const T* __restrict__ Rt = static_cast<const T*>(a.Rt);
   const unsigned ND = (unsigned)N * D;
 
-  const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
-  const rsrc_t rS0 = make_rsrc(a.s0, (size_t)S * B * ND * ES);
-  const rsrc_t rDs = make_rsrc(a.dstates, (size_t)S * B * Tn * ND * ES);
+  const rsrc_t rSt = make_rsrc(a.states, ((size_t)(S - 1) * BS + B) * Tn * ND * ES);
+  const rsrc_t rS0 = make_rsrc(a.s0, ((size_t)(S - 1) * BS + B) * ND * ES);
+  const rsrc_t rDs = make_rsrc(a.dstates, ((size_t)(S - 1) * BS + B) * Tn * ND * ES);
   constexpr int NCP = CacheBlk<T, NCA>::NCP, NWC = CacheBlk<T, NCA>::template Words<E>::value;
   const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * (NC ? NCP : 0) * ES);
   const rsrc_t rDw = make_rsrc(a.dWx, (size_t)B * Tn * GW * ND * ES);
@@ -213,8 +214,8 @@ fused_bwd_kernel(const BwdArgs a) {
         const int c = lane + 64 * i, half = c & 1, pr = (c >> 1) % TR, ptile = ((c >> 1) / TR) % UT_WG, pk = (c >> 1) / (TR * UT_WG);
         const bool ok = c < SP_TOT && bt * TR + pr < B;
         const unsigned col = n * D + slice * DL + ptile * 16 + half * 8;
-        svo[i] = ok ? ((((unsigned)(pk * B + bt * TR + pr) * Tn) * ND + col) * ES) : kInvalidOff;   // + t * ND * ES
-        s0o[i] = ok ? (((unsigned)(pk * B + bt * TR + pr) * ND + col) * ES) : kInvalidOff;
+        svo[i] = ok ? ((((unsigned)(pk * BS + bt * TR + pr) * Tn) * ND + col) * ES) : kInvalidOff;   // + t * ND * ES
+        s0o[i] = ok ? (((unsigned)(pk * BS + bt * TR + pr) * ND + col) * ES) : kInvalidOff;
         sl[i] = c < SP_TOT ? ((pk * UT_WG + ptile) * TR + pr) * 16 + half * 8 : -1;
       }
       struct Ops { Dw<4> ca[NPC > 0 ? NPC : 1], sp[NPS], dso[NPS]; };
@@ -507,9 +508,9 @@ fused_bwd_kernel(const BwdArgs a) {
         p.cache[u] = buf_load_wide<NWC>(rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
 #pragma unroll
       for (int k = 0; k < S; ++k) {
-        const unsigned so = ((unsigned)k * B * Tn + t) * ND * ES;
+        const unsigned so = ((unsigned)k * BS * Tn + t) * ND * ES;
         p.dso[u][k] = buf_load<ND_, SB>(rDs, st_v[u], so);
-        p.sp[u][k] = buf_load<ND_, SB>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * B * ND * ES : so - ND * ES);
+        p.sp[u][k] = buf_load<ND_, SB>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * BS * ND * ES : so - ND * ES);
       }
     }
   };
@@ -519,7 +520,7 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
   for (int u = 0; u < UTW; ++u)
 #pragma unroll
-    for (int k = 0; k < S; ++k) sn[u][k] = buf_load<ND_, SB>(rSt, st_v[u], ((unsigned)k * B * Tn + (Tn - 1)) * ND * ES);
+    for (int k = 0; k < S; ++k) sn[u][k] = buf_load<ND_, SB>(rSt, st_v[u], ((unsigned)k * BS * Tn + (Tn - 1)) * ND * ES);
   // exchange stores may stay in the L2 of the XCD once the group is known to share one
   if (KW > 1 && w == 0) {
     const int r = (a.xcd && !a.cut) ? xcd_handshake<KW>(a.xcd + (size_t)grp * 32, slice, lane, a.status, a.spin_limit) : 0;
@@ -1094,7 +1095,7 @@ fused_bwd_kernel(const BwdArgs a) {
   }
 
   // ---- cotangent of the initial state, bias partial sums ----------------------------------
-  const rsrc_t rD0 = make_rsrc(a.ds0, (size_t)S * B * ND * ES);
+  const rsrc_t rD0 = make_rsrc(a.ds0, ((size_t)(S - 1) * BS + B) * ND * ES);
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
 #pragma unroll
@@ -1102,7 +1103,7 @@ fused_bwd_kernel(const BwdArgs a) {
       float v[E];
 #pragma unroll
       for (int e = 0; e < E; ++e) v[e] = ds[u][e][k];
-      buf_store<ND_, SB>(pack<E>(v, (T*)0), rD0, s0_v[u], (unsigned)k * B * ND * ES);
+      buf_store<ND_, SB>(pack<E>(v, (T*)0), rD0, s0_v[u], (unsigned)k * BS * ND * ES);
     }
 #pragma unroll
     for (int g = 0; g < GT; ++g)

@@ -31,6 +31,7 @@ struct FwdArgs {
   u64* ll; int* status;
   int* xcd;          // 32 words per group for xcd_handshake (zero at launch), or null: exchange stores stay agent scope
   int B, T, N;
+  int BS;  // rows between the state planes of s0 and states ([S, BS, ...]); B unless the call covers a range of a larger batch
   int grp0, groups, groups_total;  // this launch handles groups [grp0, grp0 + groups)
   int tile_rows;                   // batch rows per group: 4, 8 or 16
   int training, spin_limit, poll_delay;
@@ -133,7 +134,7 @@ fused_fwd_kernel(const FwdArgs a) {
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
   const int grp = a.grp0 + grp_l;
-  const int N = a.N, Tn = a.T, B = a.B;
+  const int N = a.N, Tn = a.T, B = a.B, BS = a.BS;
   const int n = grp % N, bt = grp / N;
   const int tid = threadIdx.x, lane = tid & 63, w = tid >> 6;
   const int r16 = lane & 15, q4 = lane >> 4;
@@ -152,7 +153,7 @@ fused_fwd_kernel(const FwdArgs a) {
   if constexpr (KW == 1) { if (blockIdx.x == 0 && tid == 0) *a.status = 0; }
 
   const rsrc_t rWx = make_rsrc(a.Wx, (size_t)B * Tn * GW * ND * ES);
-  const rsrc_t rSt = make_rsrc(a.states, (size_t)S * B * Tn * ND * ES);
+  const rsrc_t rSt = make_rsrc(a.states, ((size_t)(S - 1) * BS + B) * Tn * ND * ES);
   constexpr int NCP = CacheBlk<T, NCA>::NCP, NWC = CacheBlk<T, NCA>::template Words<E>::value;
   const rsrc_t rCa = make_rsrc(a.cache, (size_t)Tn * N * Bpad * D * (NC ? NCP : 0) * ES);
 
@@ -193,7 +194,7 @@ fused_fwd_kernel(const FwdArgs a) {
       for (int i = 0; i < NSP; ++i) {
         const int c = lane + 64 * i, ch = c % (D / 8), pr = (c / (D / 8)) % TR, pk = c / ((D / 8) * TR);
         const bool ok = c < SP_TOT && bt * TR + pr < B;
-        svo[i] = ok ? ((((unsigned)(pk * B + bt * TR + pr) * Tn) * ND + n * D + ch * 8) * ES) : kInvalidOff;
+        svo[i] = ok ? ((((unsigned)(pk * BS + bt * TR + pr) * Tn) * ND + n * D + ch * 8) * ES) : kInvalidOff;
         sl[i] = c < SP_TOT ? (pk * TR + pr) * OBR + ch * 8 : 0;
       }
 #pragma unroll
@@ -353,7 +354,7 @@ fused_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int k = 0; k < S; ++k)
         s[u][e][k] = !bvalid ? 0.f : a.carry ? a.carry[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e]
-                                              : (float)s0[((size_t)k * B + bg) * ND + (size_t)n * D + ub[u] + esub + e];
+                                              : (float)s0[((size_t)k * BS + bg) * ND + (size_t)n * D + ub[u] + esub + e];
     }
   }
 
@@ -667,7 +668,7 @@ fused_fwd_kernel(const FwdArgs a) {
       } else {
 #pragma unroll
       for (int k = 0; k < S; ++k)
-        buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * B * Tn + t) * ND * ES);
+        buf_store<ND_, SB>(pack<E>(so[k], (T*)0), rSt, st_v[u], ((unsigned)k * BS * Tn + t) * ND * ES);
       // private cache layout [t][head][unit tile][batch row][16 units][value]: one store per tile
       if constexpr (NC > 0)
         buf_store_wide<NWC>(cache_pack<T, NCA, E>(cv), rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);

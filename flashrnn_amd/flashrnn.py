@@ -163,12 +163,12 @@ def _entry(backend: str, name: str):
     return getattr(_lib.load_library(), prefix + name)
 
 
-def _options(cfg: "FlashRNNConfig"):
+def _options(cfg: "FlashRNNConfig", batch_stride: int = 0):
     import ctypes
 
     return ctypes.byref(_lib.Options(float(cfg.forward_clipval or 0.0), float(cfg.gradient_recurrent_clipval or 0.0),
                                      int(bool(cfg.gradient_recurrent_cut)),
-                                     int(bool(cfg.recompute_gates) and cfg.backend == "hip_fused")))
+                                     int(bool(cfg.recompute_gates) and cfg.backend == "hip_fused"), int(batch_stride)))
 
 
 def _workspace_bytes(cfg: "FlashRNNConfig", f_id, d_id, B, T, N, D, backward: int) -> int:
@@ -380,8 +380,10 @@ def _cast_inputs(Wx, R, b, s0, cfg: FlashRNNConfig):
             s0.detach().to(kdt).reshape(S, B, N, D).contiguous())
 
 
-def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
-    """One forward call of the library on kernel-typed, contiguous tensors: (states [S,B,T,N,D], gate cache)."""
+def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool, out=None, batch_stride: int = 0):
+    """One forward call of the library on kernel-typed, contiguous tensors: (states [S,B,T,N,D], gate cache).
+    out / batch_stride: the call covers a range of rows of a larger batch; s0_k and out are then the slices
+    [:, b0:b1] of the full tensors [S, batch_stride, ...], used in place (see frnn_options.batch_stride)."""
     kdt = DTYPE_DICT[cfg.dtype]
     f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
     B, T, Gw, N, D = Wx_k.shape
@@ -395,7 +397,7 @@ def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
             rc = _lib.load_library().frnn_fused_recompute_supported(f_id, d_id, B, N, D)
         if rc != 0:
             _raise(rc, f"{cfg.backend} backend")
-        states = torch.empty((S, B, T, N, D), dtype=kdt, device=Wx_k.device)
+        states = out if out is not None else torch.empty((S, B, T, N, D), dtype=kdt, device=Wx_k.device)
         cache_bytes = _entry(cfg.backend, "cache_bytes_opt")(f_id, d_id, B, T, N, D, _options(cfg)) if training else 0
         cache = torch.empty(max(cache_bytes, 16), dtype=torch.uint8, device=Wx_k.device)
         ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 0)
@@ -404,7 +406,7 @@ def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
         rc = _entry(cfg.backend, "forward_opt")(
             f_id, d_id, int(training), B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(),
             s0_k.data_ptr(), states.data_ptr(), cache.data_ptr() if training else None,
-            ws.data_ptr(), ws.numel(), stream, _options(cfg))
+            ws.data_ptr(), ws.numel(), stream, _options(cfg, batch_stride))
         if rc != 0:
             _raise(rc, f"{cfg.backend} forward")
         if cfg.backend == "hip_fused":
@@ -415,16 +417,18 @@ def _run_forward(Wx_k, R_k, b_k, s0_k, cfg: FlashRNNConfig, training: bool):
     return states, cache
 
 
-def _run_backward(cfg: FlashRNNConfig, R_k, b_k, s0_k, states, cache, Wx_k, ds, dWx):
+def _run_backward(cfg: FlashRNNConfig, R_k, b_k, s0_k, states, cache, Wx_k, ds, dWx, ds0=None, batch_stride: int = 0):
     """One backward call of the library; ds [S,B,T,N,D] contiguous in the kernel type, dWx [B,T,G_w,N,D] is written.
-    Returns (dR, db, ds0 [S,B,N,D]); dR and db are fp32."""
+    Returns (dR, db, ds0 [S,B,N,D]); dR and db are fp32.  ds0 / batch_stride: as in _run_forward, the state-shaped
+    tensors (s0_k, states, ds, ds0) are slices [:, b0:b1] of full tensors of batch_stride rows, used in place."""
     kdt = DTYPE_DICT[cfg.dtype]
     f_id, d_id = _lib.FUNCTION_IDS[cfg.function], _lib.DTYPE_IDS[cfg.dtype]
     S, B, T, N, D = states.shape
     Gr, Gt = cfg.num_gates_r, cfg.num_gates_t
     dev = states.device
     with _on_device(dev):
-        ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
+        if ds0 is None:
+            ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dev)
         dR = torch.empty((Gr, N, D, D), dtype=torch.float32, device=dev)
         db = torch.empty((Gt, N, D), dtype=torch.float32, device=dev)
         ws_bytes = _workspace_bytes(cfg, f_id, d_id, B, T, N, D, 1)
@@ -434,12 +438,12 @@ def _run_backward(cfg: FlashRNNConfig, R_k, b_k, s0_k, states, cache, Wx_k, ds, 
             rc = _lib.load_library().frnn_fused_backward_recompute(
                 f_id, d_id, B, T, N, D, Wx_k.data_ptr(), R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(),
                 states.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
-                ws.data_ptr(), ws.numel(), stream, _options(cfg))
+                ws.data_ptr(), ws.numel(), stream, _options(cfg, batch_stride))
         else:
             rc = _entry(cfg.backend, "backward_opt")(
                 f_id, d_id, B, T, N, D, R_k.data_ptr(), b_k.data_ptr(), s0_k.data_ptr(), states.data_ptr(),
                 cache.data_ptr(), ds.data_ptr(), dWx.data_ptr(), ds0.data_ptr(), dR.data_ptr(), db.data_ptr(),
-                ws.data_ptr(), ws.numel(), stream, _options(cfg))
+                ws.data_ptr(), ws.numel(), stream, _options(cfg, batch_stride))
         if rc != 0:
             _raise(rc, f"{cfg.backend} backward")
         if cfg.backend == "hip_fused":
@@ -487,10 +491,13 @@ class _FlashRNNFunction(torch.autograd.Function):
 class _FlashRNNRangesFunction(torch.autograd.Function):
     """The same over ranges of `rows` batch rows, one library call each (see _apply_in_batch_ranges).  A range of Wx
     and of dWx is contiguous (the batch is their leading axis), so the calls read and write the full tensors in
-    place; the state tensors [S,B,...] are copied range by range."""
+    place.  The state-shaped tensors [S,B,...] have the batch as their second axis: with `inplace` the calls name the
+    full tensors' plane stride (frnn_options.batch_stride) and use their slices as they are, nothing is copied and
+    the states are held once; where even that does not fit 32-bit offsets (the planes of the later states lie too far
+    apart: sLSTM at very large batches) each range gets contiguous copies of its slices."""
 
     @staticmethod
-    def forward(ctx, Wx, R, b, s0, cfg: FlashRNNConfig, training: bool, rows: int):
+    def forward(ctx, Wx, R, b, s0, cfg: FlashRNNConfig, training: bool, rows: int, inplace: bool):
         if not Wx.is_cuda:
             raise RuntimeError("flashrnn_amd runs on a GPU only (got a CPU tensor); there is no CPU fallback")
         _status.poll()
@@ -502,11 +509,18 @@ class _FlashRNNRangesFunction(torch.autograd.Function):
         saved = []
         for b0 in range(0, B, rows):
             b1 = min(B, b0 + rows)
-            s0_r = s0_k[:, b0:b1].contiguous()
-            states_r, cache_r = _run_forward(Wx_k[b0:b1], R_k, b_k, s0_r, cfg, training)
-            states[:, b0:b1].copy_(states_r)
-            saved += [s0_r, states_r, cache_r]
-        ctx.cfg, ctx.training, ctx.rows = cfg, training, rows
+            if inplace:
+                _, cache_r = _run_forward(Wx_k[b0:b1], R_k, b_k, s0_k[:, b0:b1], cfg, training, out=states[:, b0:b1],
+                                          batch_stride=B)
+                saved.append(cache_r)
+            else:
+                s0_r = s0_k[:, b0:b1].contiguous()
+                states_r, cache_r = _run_forward(Wx_k[b0:b1], R_k, b_k, s0_r, cfg, training)
+                states[:, b0:b1].copy_(states_r)
+                saved += [s0_r, states_r, cache_r]
+        ctx.cfg, ctx.training, ctx.rows, ctx.inplace, ctx.batch = cfg, training, rows, inplace, B
+        if inplace:
+            saved = [s0_k, states] + saved
         ctx.save_for_backward(R_k, b_k, Wx_k if cfg.recompute_gates else R_k, *saved)
         return states
 
@@ -515,28 +529,34 @@ class _FlashRNNRangesFunction(torch.autograd.Function):
     def backward(ctx, dstates):
         if not ctx.training:
             raise RuntimeError("FlashRNN backward can only be called in training mode")
-        cfg, rows = ctx.cfg, ctx.rows
+        cfg, rows, B = ctx.cfg, ctx.rows, ctx.batch
         R_k, b_k, Wx_k, *saved = ctx.saved_tensors
         S, _, T, N, D = dstates.shape
-        B = sum(saved[3 * i].shape[1] for i in range(len(saved) // 3))
         kdt = DTYPE_DICT[cfg.dtype]
         _backward_devices.add(dstates.device.index if dstates.device.index is not None else torch.cuda.current_device())
         _status.poll()
         ds = dstates.to(kdt)
+        if ctx.inplace:
+            ds = ds.contiguous()
+            s0_k, states, *caches = saved
         with _on_device(dstates.device):
             dWx = torch.empty((B, T, cfg.num_gates_w, N, D), dtype=kdt, device=dstates.device)
             ds0 = torch.empty((S, B, N, D), dtype=kdt, device=dstates.device)
         dR = db = None
         for i, b0 in enumerate(range(0, B, rows)):
             b1 = min(B, b0 + rows)
-            s0_r, states_r, cache_r = saved[3 * i:3 * i + 3]
             wx_r = Wx_k[b0:b1] if cfg.recompute_gates else Wx_k
-            dR_r, db_r, ds0_r = _run_backward(cfg, R_k, b_k, s0_r, states_r, cache_r, wx_r,
-                                              ds[:, b0:b1].contiguous(), dWx[b0:b1])
-            ds0[:, b0:b1].copy_(ds0_r)
+            if ctx.inplace:
+                dR_r, db_r, _ = _run_backward(cfg, R_k, b_k, s0_k[:, b0:b1], states[:, b0:b1], caches[i], wx_r,
+                                              ds[:, b0:b1], dWx[b0:b1], ds0=ds0[:, b0:b1], batch_stride=B)
+            else:
+                s0_r, states_r, cache_r = saved[3 * i:3 * i + 3]
+                dR_r, db_r, ds0_r = _run_backward(cfg, R_k, b_k, s0_r, states_r, cache_r, wx_r,
+                                                  ds[:, b0:b1].contiguous(), dWx[b0:b1])
+                ds0[:, b0:b1].copy_(ds0_r)
             dR = dR_r if dR is None else dR.add_(dR_r)
             db = db_r if db is None else db.add_(db_r)
-        return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None, None
+        return dWx, dR, db, ds0.reshape(S, B, 1, N, D), None, None, None, None
 
 
 def _get_config(Wx, R, b, function, backend, dtype) -> FlashRNNConfig:
@@ -617,28 +637,31 @@ def flashrnn(
     return _permuted(out, "SBTHD", config.output_shape), _permuted(out[:, :, -1:], "SBTHD", config.output_shape)
 
 
-_FUSED_TENSOR_LIMIT = 1 << 31  # the fused kernels address each tensor with 32-bit byte offsets
-
-
 def _apply_in_batch_ranges(Wx, R, b, states, config, training):
     """Batch rows are independent, so a fused problem one of whose tensors (Wx, the states or the gate cache)
-    would reach 2 GiB runs as several library calls over ranges of the batch (_FlashRNNRangesFunction), dR and db
-    summed over the ranges."""
+    would reach 2 GiB (32-bit offsets inside the fused kernels) runs as several library calls over ranges of the batch
+    (_FlashRNNRangesFunction), dR and db summed over the ranges.  How many rows a call can take is the library's
+    answer (frnn_fused_max_batch), for calls that use the full tensors in place and for calls on copies."""
     B, T, Gw, N, D = Wx.shape
     if config.backend != "hip_fused":
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
-    es = 4 if config.dtype == "float32" else 2
     f_id, d_id = _lib.FUNCTION_IDS[config.function], _lib.DTYPE_IDS[config.dtype]
-    cache_row = _lib.load_library().frnn_fused_cache_bytes_opt(f_id, d_id, 1, T, N, D, _options(config)) if training else 0
-    per_row = max(T * N * D * es * max(Gw, config.num_states), cache_row)  # bytes per batch row of the largest tensor
-    rows = max(1, (_FUSED_TENSOR_LIMIT - 1) // per_row)
+    max_batch = lambda stride: _lib.load_library().frnn_fused_max_batch(f_id, d_id, T, N, D, stride, int(training), _options(config))
+    limit = os.environ.get("FRNN_TEST_MAX_BATCH")  # (tests: pretend that a call takes no more rows than this)
+    rows = max_batch(0) if limit is None else min(max_batch(0), int(limit))
     if rows >= B:
         return _FlashRNNFunction.apply(Wx, R, b, states, config, training)
+    rows_in_place = max_batch(B) if limit is None else min(max_batch(B), int(limit))
+    inplace = rows_in_place >= min(16, rows) and os.environ.get("FRNN_RANGES_COPY") != "1"
+    if inplace:
+        rows = rows_in_place
+    if rows < 1:
+        raise ValueError("flashrnn_amd: one batch row of this problem already reaches 2 GiB per tensor; use backend='hip'")
     rows = max(16, rows // 16 * 16) if rows >= 16 else rows  # whole batch tiles
     if rows >= 16:  # ranges of about the same size, still whole tiles
         n_ranges = -(-B // rows)
         rows = min(rows, -(-B // (16 * n_ranges)) * 16)
-    return _FlashRNNRangesFunction.apply(Wx, R, b, states, config, training, rows)
+    return _FlashRNNRangesFunction.apply(Wx, R, b, states, config, training, rows, inplace)
 
 
 def flashrnn_step(

@@ -49,7 +49,9 @@ enum {
   FRNN_E_NULL = -3,        /* a required pointer is null */
   FRNN_E_ALIGN = -4,       /* a pointer is not 16-byte aligned */
   FRNN_E_WORKSPACE = -5,   /* workspace smaller than frnn_*_workspace_bytes() */
-  FRNN_E_DEVICE = -6       /* current device is not usable (query failed, too few CUs) */
+  FRNN_E_DEVICE = -6,      /* current device is not usable (query failed, too few CUs) */
+  FRNN_E_TOO_LARGE = -7    /* fused backend: a tensor of this call reaches 2 GiB (32-bit offsets inside the kernels); run the
+                            * batch as ranges of at most frnn_fused_max_batch() rows, see frnn_options.batch_stride */
 };
 
 /* Thread-local text of the last error returned on this thread ("" if none). */
@@ -171,11 +173,23 @@ typedef struct frnn_options {
   float gradient_recurrent_clipval;
   int gradient_recurrent_cut;
   int recompute;  /* fused backend: no gate cache, see frnn_fused_backward_recompute */
+  int batch_stride;  /* fused backend, 0 = B.  The call covers B rows of a batch of batch_stride rows: the state tensors
+                      * (s0 and ds0: [S, batch_stride, N, D]; states and dstates: [S, batch_stride, T, N, D]) keep the full
+                      * batch's plane stride, and the pointers handed over point at the first row of the range in
+                      * plane 0.  Wx, dWx and the gate cache have the batch as their leading axis, so a range of them is
+                      * a contiguous block of its own (the gate cache is private to the call that wrote it); dR and db are
+                      * the range's own sums.  This is how a batch whose tensors reach 2 GiB runs as several calls that
+                      * read and write the caller's tensors in place. */
 } frnn_options;
 
 /* Gate-cache size under options: an Elman cell under forward_clipval caches the unclamped h (one value per
  * element, as elman_fused_pointwise.cuh:44-47), without it nothing.  opt == NULL: as the plain queries. */
 size_t frnn_fused_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt);
+/* The most batch rows one fused call can take before one of its tensors reaches 2 GiB (FRNN_E_TOO_LARGE), given the plane
+ * stride of the state tensors (batch_stride rows; 0: each call's tensors are its own, stride = its B) and whether the
+ * gate cache is written (training, and not opt->recompute).  0: not even one row fits at this stride.  The reference
+ * has no such limit (fused/flashrnn.cc:68-144 allocates whatever the shape needs). */
+int frnn_fused_max_batch(int function, int dtype, int T, int N, int D, int batch_stride, int training, const frnn_options* opt);
 size_t frnn_alt_cache_bytes_opt(int function, int dtype, int B, int T, int N, int D, const frnn_options* opt);
 
 int frnn_fused_forward_opt(int function, int dtype, int training, int B, int T, int N, int D,

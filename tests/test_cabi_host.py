@@ -106,8 +106,11 @@ def test_small_batches_get_the_tiling_with_more_workgroups_per_head(lib):
 
 
 def _fwd(lib, entry, function=0, dtype=0, B=8, T=4, N=1, D=64, Wx=FAKE, R=FAKE, b=FAKE, s0=FAKE, states=FAKE,
-         cache=FAKE, ws=FAKE, ws_bytes=0, training=1):
-    return getattr(lib, entry)(function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, ws, ws_bytes, None)
+         cache=FAKE, ws=FAKE, ws_bytes=0, training=1, opt=None):
+    args = [function, dtype, training, B, T, N, D, Wx, R, b, s0, states, cache, ws, ws_bytes, None]
+    if entry.endswith("_opt"):
+        args.append(ctypes.byref(opt) if opt is not None else None)
+    return getattr(lib, entry)(*args)
 
 
 @pytest.mark.parametrize("entry", ["frnn_fused_forward", "frnn_alt_forward"])
@@ -146,8 +149,26 @@ def test_backward_rejects_bad_arguments_before_launch(lib, entry):
 
 def test_fused_refuses_tensors_of_2_gib(lib):
     # 32-bit byte offsets inside the fused kernels: B*T*N*D*G_w*2 bytes must stay below 2 GiB
-    assert _fwd(lib, "frnn_fused_forward", B=64, T=16384, N=4, D=256) == _lib.E_ARG
+    # (a code of its own, so that a binding can tell "split the batch" from a bad argument)
+    assert _fwd(lib, "frnn_fused_forward", B=64, T=16384, N=4, D=256) == _lib.E_TOO_LARGE
     assert b"2 GiB" in lib.frnn_last_error()
+    L, S = _lib.FUNCTION_IDS["lstm"], _lib.FUNCTION_IDS["slstm"]
+    T, N, D = 1024, 12, 64
+    row = T * N * D * 2                                          # bytes of one batch row of one bf16 plane
+    lim = (1 << 31) - 1
+    # each call on tensors of its own: Wx (4 gates) and the gate cache (4 values) bound an LSTM call, 341 rows
+    assert lib.frnn_fused_max_batch(L, 0, T, N, D, 0, 1, None) == lim // (4 * row) == 341
+    # ranges of a batch of 512 rows used in place: the c plane starts 512 rows behind the h plane
+    assert lib.frnn_fused_max_batch(L, 0, T, N, D, 512, 1, None) == min(341, (lim - 512 * row) // row) == 341
+    assert lib.frnn_fused_max_batch(L, 0, T, N, D, 1200, 1, None) == (lim - 1200 * row) // row == 165
+    # sLSTM: four planes; at 512 rows the fourth lies beyond 2 GiB from the first: no row fits in place
+    assert lib.frnn_fused_max_batch(S, 0, T, N, D, 512, 1, None) == 0
+    assert lib.frnn_fused_max_batch(S, 0, T, N, D, 0, 1, None) == lim // (6 * row) == 227   # (its cache: 5 values padded to 6)
+    o = _lib.Options(0.0, 0.0, 0, 0, 512)
+    assert _fwd(lib, "frnn_fused_forward_opt", B=341, T=T, N=N, D=D, opt=o) != _lib.E_TOO_LARGE
+    assert _fwd(lib, "frnn_fused_forward_opt", B=342, T=T, N=N, D=D, opt=o) == _lib.E_TOO_LARGE
+    o = _lib.Options(0.0, 0.0, 0, 0, 100)
+    assert _fwd(lib, "frnn_fused_forward_opt", B=128, T=8, N=2, D=64, opt=o) == _lib.E_ARG   # stride smaller than the call's rows
 
 
 def test_python_api_argument_errors():
@@ -275,7 +296,7 @@ def test_options_carry_their_size(lib):
     with the later ones off, one that does not set the size is refused."""
     L = _lib.FUNCTION_IDS["lstm"]
     o = _lib.Options(0.5, 0.0, 0, 0)
-    assert o.struct_size == ctypes.sizeof(_lib.Options) == 20
+    assert o.struct_size == ctypes.sizeof(_lib.Options) == 24
     assert lib.frnn_fused_cache_bytes_opt(L, 0, 4, 8, 2, 64, ctypes.byref(o)) > 0
     o.struct_size = 0
     assert lib.frnn_fused_cache_bytes_opt(L, 0, 4, 8, 2, 64, ctypes.byref(o)) == 0 and b"struct_size" in lib.frnn_last_error()

@@ -282,27 +282,31 @@ def test_launches_sized_by_the_room_of_an_xcd(gpu, monkeypatch, function, B, N, 
     check_case(gpu, function, B, 3, N, D, "bfloat16", "hip_fused", seed=27, init="randn")
 
 
+@pytest.mark.parametrize("copies", [False, True])
 @pytest.mark.parametrize("function,options", [("lstm", None), ("gru", None), ("slstm", None), ("elman", None),
                                               ("lstm", {"recompute_gates": True})])
-def test_batch_ranges_for_tensors_beyond_32_bit_offsets(gpu, monkeypatch, function, options):
-    """flashrnn() splits a fused problem whose tensors would reach 2 GiB into calls over batch ranges (the
-    kernels use 32-bit byte offsets); dR and db are summed over the ranges.  The limit is lowered
-    here so that a small problem splits into ranges of 16, 16 and 8 rows."""
+def test_batch_ranges_for_tensors_beyond_32_bit_offsets(gpu, monkeypatch, function, options, copies):
+    """flashrnn() splits a fused problem whose tensors would reach 2 GiB into calls over batch ranges (the kernels use
+    32-bit byte offsets); dR and db are summed over the ranges.  The ranges use the full state tensors in place
+    (frnn_options.batch_stride), or contiguous copies of their slices where the planes lie too far apart (forced here
+    with FRNN_RANGES_COPY).  FRNN_TEST_MAX_BATCH makes the wrapper believe that a call takes at most 17 rows, so that
+    a small problem splits into ranges of 16, 16 and 8 rows; the real limit is crossed by
+    test_a_problem_whose_tensors_pass_2_gib_at_its_real_size."""
     import importlib
 
     from parity import check_case
 
     mod = importlib.import_module("flashrnn_amd.flashrnn")  # (the package attribute of that name is the function)
-    print(f"case batch ranges {function} {options}", flush=True)
+    print(f"case batch ranges {function} {options} copies={copies}", flush=True)
     B, T, N, D = 40, 6, 2, 64
-    # 17 rows of an LSTM's Wx (4 gates, bf16); Elman has one gate
-    monkeypatch.setattr(mod, "_FUSED_TENSOR_LIMIT", T * N * D * 2 * (1 if function == "elman" else 4) * 17)
+    monkeypatch.setenv("FRNN_TEST_MAX_BATCH", "17")
+    if copies:
+        monkeypatch.setenv("FRNN_RANGES_COPY", "1")
     calls = []
     real = mod._run_forward
-    monkeypatch.setattr(mod, "_run_forward", lambda *a: (calls.append(a[0].shape[0]), real(*a))[1])
+    monkeypatch.setattr(mod, "_run_forward", lambda *a, **k: (calls.append((a[0].shape[0], k.get("batch_stride", 0))), real(*a, **k))[1])
     check_case(gpu, function, B, T, N, D, "bfloat16", "hip_fused", seed=28, init="randn", options=options)
-    # (the other cells' largest tensor differs, and with it the size of a range)
-    assert calls == [16, 16, 8] if function == "lstm" else (len(calls) >= 2 and sum(calls) == B), calls
+    assert calls == [(16, 0 if copies else B), (16, 0 if copies else B), (8, 0 if copies else B)], calls
 
 
 @pytest.mark.parametrize("backend", ["hip_fused", "hip"])

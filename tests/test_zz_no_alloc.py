@@ -21,7 +21,7 @@ DT = {"bfloat16": 0, "float32": 1, "float16": 2}
 class Options(ctypes.Structure):
     _fields_ = [("struct_size", ctypes.c_uint), ("forward_clipval", ctypes.c_float),
                 ("gradient_recurrent_clipval", ctypes.c_float), ("gradient_recurrent_cut", ctypes.c_int),
-                ("recompute", ctypes.c_int)]
+                ("recompute", ctypes.c_int), ("batch_stride", ctypes.c_int)]
 
 
 def _open():
