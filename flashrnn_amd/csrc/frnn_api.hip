@@ -644,13 +644,11 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   a.poll_delay = env_int("FRNN_POLL_DELAY", fwd_poll_delay_default(fx, dtype, p, tr));
   a.h_clip = o.h_clip;
   a.mailbox = nullptr; a.inbox_off = a.outbox_off = a.in_slot = a.out_slot = 0; a.slots = 1; a.idle_limit = 0;
-  // producer-wave stores: for launches that fill the device, where the kernel is bound by its memory traffic (measured,
-  // bf16 T = 1024, forward kernel with the producer wave storing against the compute lanes storing: LSTM N12 D64 B256 0.82
-  // against 1.04 ms, B128 0.50 / 0.66, B64 0.39 / 0.38, B16 0.31 / 0.30; sLSTM N12 D64 B128 0.70 / 0.97; LSTM N24 D32 B256
-  // 1.04 / 1.32; the GRU, with less to store, only gains when the device is fuller still: N12 D64 B256 0.65 / 0.78 but
-  // B128 0.51 / 0.46); FRNN_PRODUCER_STORES=0/1 overrides
-  a.pst = step ? 0 : env_int("FRNN_PRODUCER_STORES",
-                             tr == 4 && p.kw == 1 && groups > (fx == FRNN_GRU ? 2 : 1) * device_cus() ? 1 : 0);
+  // producer-wave stores: for launches that put some load on the memory system (measured, bf16 T = 1024, forward kernel
+  // with the producer wave storing against the compute lanes storing: LSTM N12 D64 B256 0.82 against 1.03 ms, B128 0.50 / 0.65,
+  // B64 0.38 / 0.38, B16 0.30 / 0.295; sLSTM N12 D64 B128 0.68 / 0.97; GRU N12 D64 B256 0.66 / 0.78; LSTM N24 D32 B256
+  // 1.11 / 1.33); FRNN_PRODUCER_STORES=0/1 overrides
+  a.pst = step ? 0 : env_int("FRNN_PRODUCER_STORES", tr == 4 && p.kw == 1 && 2 * groups > device_cus() ? 1 : 0);
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);
@@ -773,12 +771,11 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   // rebuild: best without a delay for every cell
   a.poll_delay = env_int("FRNN_POLL_DELAY_BWD", o.rc ? 0 : c.GR == 1 ? (p.kw > 4 ? 8 : 4) : 2);
   a.g_clip = o.g_clip; a.cut = o.cut;
-  // producer-wave stores of dWx.  The reverse kernel's producer wave already moves five operand pieces per step, so the
-  // extra stores only pay where it has little else to do (measured, bf16 T = 1024, reverse kernel: heads of 32 units,
-  // two compute waves: LSTM N24 D32 B256 1.20 against 1.54 ms, B128 0.71 / 0.75, GRU 1.02 / 1.27, sLSTM B128 0.93 / 1.03;
-  // heads of 64 units: GRU N12 D64 B256 0.90 / 0.98 but B128 0.74 / 0.61, LSTM B256 1.39 / 1.26, sLSTM the same)
-  a.pst = env_int("FRNN_PRODUCER_STORES",
-                  tr == 4 && p.kw == 1 && groups > 2 * device_cus() && (p.waves <= 2 || (fx == FRNN_GRU && p.waves <= 4)) ? 1 : 0);
+  // producer-wave stores of dWx, under the same condition (reverse kernel: LSTM N12 D64 B256 1.16 against 1.26 ms, B128
+  // 0.64 / 0.76, B64 0.48 / 0.49, B16 0.41 / 0.41; GRU N12 D64 B256 0.79 / 0.97; sLSTM N12 D64 B128 0.80 / 1.00; LSTM N24 D32
+  // B256 1.22 / 1.53.  With the stores issued in front of the loads of an iteration the same kernels lost up to 25 %:
+  // a wave's memory operations complete in order, and the stores are acknowledged late)
+  a.pst = env_int("FRNN_PRODUCER_STORES", tr == 4 && p.kw == 1 && 2 * groups > device_cus() ? 1 : 0);
   a.trace = nullptr;
 #ifdef FRNN_TRACE
   a.trace = (long long*)((char*)workspace + w.zero_bytes);

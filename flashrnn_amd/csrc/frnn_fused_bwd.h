@@ -286,8 +286,13 @@ fused_bwd_kernel(const BwdArgs a) {
         auto iter = [&](int i, const Ops& next, Ops& refill) __attribute__((always_inline)) {
           if (barrier_or(false, dead_flag)) { pdead = true; return; }
           put(next, i + 2);
+#ifdef FRNN_PST_DRAIN_FIRST
           if constexpr (PST) drain(i);
           fetch(refill, i + 4);
+#else
+          fetch(refill, i + 4);  // (loads before stores: see the forward kernel)
+          if constexpr (PST) drain(i);
+#endif
         };
         int i = 0;
         for (; i + 2 < Tn && !pdead; i += 3) {
@@ -470,7 +475,9 @@ fused_bwd_kernel(const BwdArgs a) {
   for (int j = 0; j < NCHK; ++j) {
     const int piece = tid + j * NT;
     h_in[j] = piece < HPIECES;
-    h_row[j] = piece / (D / HC); h_k0[j] = (piece % (D / HC)) * HC;
+    // (consecutive threads take the TR rows of one piece position: in fragment order a row's pieces lie 256 bytes
+    // apart, i.e. in the same banks, and a wave that writes 64 pieces of one row does so in 32 passes)
+    h_row[j] = piece % TR; h_k0[j] = (piece / TR) * HC;
     const bool ok = h_in[j] && bt * TR + h_row[j] < B;
     hs_v[j] = ok ? ((unsigned)(bt * TR + h_row[j]) * Tn * ND + n * D + h_k0[j]) * ES : kInvalidOff;
     h0_v[j] = ok ? ((unsigned)(bt * TR + h_row[j]) * ND + n * D + h_k0[j]) * ES : kInvalidOff;

@@ -228,8 +228,16 @@ fused_fwd_kernel(const FwdArgs a) {
           else lds_barrier();
         }
         put(next, t + 1);
+#ifdef FRNN_PST_DRAIN_FIRST
         if constexpr (PST) { if (t > 0) drain(t - 1); }
         fetch(refill, t + 3);
+#else
+        // (loads before stores: a wave's memory operations complete in order, and a store is acknowledged late when the
+        // device is writing at its limit; issued in front of them, the loads that the hand-over two steps on waits for
+        // only have stores of an earlier step ahead of them)
+        fetch(refill, t + 3);
+        if constexpr (PST) { if (t > 0) drain(t - 1); }
+#endif
       };
       int t = 0;
       for (; t + 2 < Tn && !pdead; t += 3) {
