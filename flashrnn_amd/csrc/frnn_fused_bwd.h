@@ -108,7 +108,9 @@ fused_bwd_kernel(const BwdArgs a) {
   typedef typename X::Frag Frag;
   typedef Own<TR> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
-  constexpr int NT = WAVES * 64, UT_WG = WAVES * UTW;
+  // (DSP = 2: pairs of waves share a tile position and split the destinations between them, see bwd_dest_split)
+  constexpr int DSP = bwd_dest_split(GR, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC), NPOS = WAVES / DSP;
+  constexpr int NT = WAVES * 64, UT_WG = NPOS * UTW;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
   constexpr int DL = D / KW;            // units owned by this workgroup
   constexpr int KDL = GR * DL;          // contraction length handled by this workgroup
@@ -131,10 +133,12 @@ fused_bwd_kernel(const BwdArgs a) {
   // (the values of one block broadcast to all 16), one instruction per k: KDL instructions of 8 cycles per 4
   // destinations instead of KDL / 4 of 32 per destination.
   constexpr int NG4 = (KW + 3) / 4;  // groups of 4 destinations
+  constexpr int NGH = (NG4 + DSP - 1) / DSP;  // of them per wave: group qq of wave half hf is group qq * DSP + hf
   // (the whole operand, a register per destination group and own gate row, in the registers of a wave: wherever the
   // 16x16x4 form keeps it there too, and up to 320 registers at one wave per SIMD)
   constexpr bool M44 = sizeof(T) == 4 && TR == 4 && KW >= 2 && !RC &&
-                       (bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)) == 0 || (WAVES <= 4 && NG4 * UTW * KDL <= 320));
+                       (bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)) == 0 || (WAVES <= 4 && NGH * UTW * KDL <= 320));
+  static_assert(DSP == 1 || M44, "destinations are split between wave pairs in the 4x4x1 form only");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);
@@ -163,7 +167,11 @@ fused_bwd_kernel(const BwdArgs a) {
   const int brow = O::row(r16), esub = O::sub(r16, q4);
   const int bg = bt * TR + brow;
   const unsigned Bpad = (unsigned)a.B;  // rows of the gate cache: padded rows are never read or written
-  const bool bvalid = bg < B;
+  // wave w of a pair-split workgroup: tile position w / 2, destination groups of parity w % 2; the lanes of a second
+  // wave own no element (every load of theirs returns zero, every store is dropped)
+  const int w_u = __builtin_amdgcn_readfirstlane(w);
+  const int hf = DSP > 1 ? w_u % DSP : 0, wp = DSP > 1 ? w_u / DSP : w, wp_u = DSP > 1 ? w_u / DSP : w_u;
+  const bool rvalid = bg < B, bvalid = rvalid && hf == 0;
   const T* __restrict__ Rt = static_cast<const T*>(a.Rt);
   const unsigned ND = (unsigned)N * D;
 
@@ -316,7 +324,7 @@ fused_bwd_kernel(const BwdArgs a) {
   unsigned wx_v[UTW], st_v[UTW], s0_v[UTW], ca_v[UTW];
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
-    ub[u] = (slice * UT_WG + w * UTW + u) * 16;
+    ub[u] = (slice * UT_WG + wp * UTW + u) * 16;
     const unsigned d0 = n * D + ub[u] + esub;
     wx_v[u] = bvalid ? ((unsigned)bg * Tn * GW * ND + d0) * ES : kInvalidOff;
     st_v[u] = bvalid ? ((unsigned)bg * Tn * ND + d0) * ES : kInvalidOff;
@@ -330,16 +338,16 @@ fused_bwd_kernel(const BwdArgs a) {
   constexpr int PIN_REGS = RC ? 0 : RTF_REGS > 160 ? (RTF_REGS < 232 ? RTF_REGS : 232) : 0;
   Frag rtf[KWR][UTW][KS];
   // 4x4x1 form: lane 4*blk + j holds row p = (tile of destination 4q + j, unit blk) of R^T, one register per own k
-  float rtb[M44 ? NG4 : 1][M44 ? UTW : 1][M44 ? KDL : 1];
+  float rtb[M44 ? NGH : 1][M44 ? UTW : 1][M44 ? KDL : 1];
   if constexpr (M44) {
     const int blk = lane >> 2, j = lane & 3;
 #pragma unroll
-    for (int q = 0; q < NG4; ++q) {
-      const int r = 4 * q + j;
+    for (int q = 0; q < NGH; ++q) {
+      const int r = 4 * (q * DSP + hf) + j;
       const int x = (slice + (r < KW ? r : 0)) % KW;
 #pragma unroll
       for (int u = 0; u < UTW; ++u) {
-        const float* row = reinterpret_cast<const float*>(Rt) + ((size_t)n * D + (x * UT_WG + w * UTW + u) * 16 + blk) * (GR * D) + slice * DL;
+        const float* row = reinterpret_cast<const float*>(Rt) + ((size_t)n * D + (x * UT_WG + wp * UTW + u) * 16 + blk) * (GR * D) + slice * DL;
 #pragma unroll
         for (int kk = 0; kk < KDL; kk += 4) {
           const float4 v = *reinterpret_cast<const float4*>(row + (kk / DL) * D + (kk % DL));
@@ -352,9 +360,9 @@ fused_bwd_kernel(const BwdArgs a) {
     // what does not fit the architectural VGPRs beside the working set is pinned to accumulation registers, where the
     // MFMA reads it in place (left to the register allocator it is copied back before every use)
     // (384 registers: the 152 that would stay in VGPRs leave too little for the working set; left alone there)
-    constexpr int ALL44 = NG4 * UTW * KDL, PIN44 = ALL44 > 344 ? 0 : ALL44 - 112 > 232 ? 232 : ALL44 - 112;
+    constexpr int ALL44 = NGH * UTW * KDL, PIN44 = ALL44 > 344 ? 0 : ALL44 - 112 > 232 ? 232 : ALL44 - 112;
 #pragma unroll
-    for (int q = 0; q < NG4; ++q)
+    for (int q = 0; q < NGH; ++q)
 #pragma unroll
       for (int u = 0; u < UTW; ++u)
 #pragma unroll
@@ -537,7 +545,6 @@ fused_bwd_kernel(const BwdArgs a) {
   const int near_i = KW > 1 ? __builtin_amdgcn_readfirstlane(near_word) : 0;  // 1: stores stay in the XCD's L2, -1: wait ran out
   u64 near_m;  // lane mask for ll_store_sel: all ones or zero, in scalar registers
   asm("s_cmp_gt_i32 %1, 0\n\ts_cselect_b64 %0, -1, 0" : "=s"(near_m) : "s"(near_i) : "scc");
-  const int w_u = __builtin_amdgcn_readfirstlane(w);
 
 #ifdef FRNN_TRACE
   long long tr[5] = {0, 0, 0, 0, 0};
@@ -642,7 +649,7 @@ fused_bwd_kernel(const BwdArgs a) {
     FRNN_STAMP(c0);
     // (readfirstlane: the compiler otherwise forms max(t - PD, 0) with a saturating VALU subtract
     // and then wraps a buffer load that uses it as a scalar offset into a waterfall loop)
-    if constexpr (!(PW && !cut)) load_pre(pn, __builtin_amdgcn_readfirstlane(t >= PD ? t - PD : 0));
+    if constexpr (!(PW && !cut)) { if (DSP == 1 || hf == 0) load_pre(pn, __builtin_amdgcn_readfirstlane(t >= PD ? t - PD : 0)); }
     // dWx_t (and the GRU's g-gate cotangent).  With an exchange the stores are issued after the
     // partial sums are sent, where they fill the wait for the other workgroups instead of delaying
     // the barrier (a vector memory instruction costs ~30 cycles to issue)
@@ -653,6 +660,7 @@ fused_bwd_kernel(const BwdArgs a) {
       for (int g = 0; g < GW; ++g) buf_store<ND_, SB>(dwp[u][g], rDw, wx_v[u], ((unsigned)t * GW + g) * ND * ES);
       if (F == FRNN_GRU) buf_store<ND_, SB>(dxp[u], rDx, st_v[u], (unsigned)t * ND * ES);
     };
+    if (DSP == 1 || hf == 0) {  // (wave-uniform: the second wave of a pair owns no element)
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float cv[NCA][E], spv[S][E], snv[S][E], dsov[S][E];
@@ -713,6 +721,7 @@ fused_bwd_kernel(const BwdArgs a) {
         }
       }
     }
+    }
     if constexpr (RC) {
       if (t > 0) stage_h(pm, t - 1);  // uniform
     }
@@ -759,7 +768,7 @@ fused_bwd_kernel(const BwdArgs a) {
     constexpr bool GROUPED = OWN_LAST && KW - 1 > 8;
     constexpr int RI = 4;
     static_assert(!GROUPED || RLD % RI == 0, "LDS-resident destinations come in whole groups");
-    float p44[M44 ? NG4 : 1][M44 ? UTW : 1][4];  // 4x4x1 form: partial sums of the lane's element, destination 4q + i
+    float p44[M44 ? NGH : 1][M44 ? UTW : 1][4];  // 4x4x1 form: partial sums of the lane's element, destination 4 (q DSP + hf) + i
     if constexpr (M44) {
       const float* gfl = reinterpret_cast<const float*>(gb) + lane;
       float ga[KDL / 16];
@@ -767,7 +776,7 @@ fused_bwd_kernel(const BwdArgs a) {
       for (int v = 0; v < KDL / 16; ++v) ga[v] = gfl[64 * v];
       __builtin_amdgcn_sched_barrier(0);
 #pragma unroll
-      for (int q = 0; q < NG4; ++q)
+      for (int q = 0; q < NGH; ++q)
 #pragma unroll
         for (int u = 0; u < UTW; ++u) {
           f32x4 ac[4];
@@ -780,7 +789,7 @@ fused_bwd_kernel(const BwdArgs a) {
           quad_transpose(p44[q][u], lane);
         }
 #pragma unroll
-      for (int u = 0; u < UTW; ++u) ds[u][0][0] += p44[0][u][0];
+      for (int u = 0; u < UTW; ++u) ds[u][0][0] += p44[0][u][0];  // (the own tiles: destination 0 of the first wave)
     }
     f32x4 accp[NACC][GROUPED ? 1 : KW][UTW];
     const Frag* gf = reinterpret_cast<const Frag*>(gb) + lane;
@@ -799,7 +808,7 @@ fused_bwd_kernel(const BwdArgs a) {
     // keep the reads up here: issued just in time they would expose the LDS latency once per chunk
     __builtin_amdgcn_sched_barrier(0);
     if constexpr (GROUPED) {
-      const unsigned sslot = ((unsigned)(bvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
+      const unsigned sslot = ((unsigned)(rvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
       auto send_group = [&](int r0, int nr, f32x4 (&ag)[RI][UTW]) __attribute__((always_inline)) {
         if (nr == RI) {  // (compile-time at every call site) four destinations with one switch of the store form
 #pragma unroll
@@ -944,9 +953,25 @@ fused_bwd_kernel(const BwdArgs a) {
     FRNN_STAMP(c3);
     if constexpr (KW > 1) {
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
-      const unsigned sslot = ((unsigned)(bvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
+      const unsigned sslot = ((unsigned)(rvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
+      if constexpr (DSP > 1) {  // this wave's destination groups
 #pragma unroll
-      for (int r = 1; r < (GROUPED ? 0 : KW); ++r) {
+        for (int q = 0; q < NGH; ++q)
+#pragma unroll
+          for (int j = 0; j < 4; ++j) {
+            const int r = 4 * (q * DSP + hf) + j;
+            if (r < 1 || r >= KW) continue;  // (uniform)
+            const int x = (slice + r) % KW;
+#pragma unroll
+            for (int u = 0; u < UTW; ++u) {
+              IW wv[E];
+              wv[0] = part_pack((PT*)0, p44[q][u][j], t);
+              ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * NPOS + wp_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
+            }
+          }
+      }
+#pragma unroll
+      for (int r = 1; r < (GROUPED || DSP > 1 ? 0 : KW); ++r) {
         const int x = (slice + r) % KW;
 #pragma unroll
         for (int u = 0; u < UTW; ++u) {
@@ -961,8 +986,10 @@ fused_bwd_kernel(const BwdArgs a) {
         }
       }
       if constexpr (DW_LATE) {
+        if (DSP == 1 || hf == 0) {
 #pragma unroll
-        for (int u = 0; u < UTW; ++u) store_dw(u);
+          for (int u = 0; u < UTW; ++u) store_dw(u);
+        }
       }
       if constexpr (OWN_LAST) {
         // the product for the own tiles, while the words just sent travel
@@ -980,7 +1007,8 @@ fused_bwd_kernel(const BwdArgs a) {
         }
       }
       // receive: KW-1 partial sums of the own tiles, PSRC sources at a time
-      const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * WAVES + w) * UTW) * KW * 256 + lane;
+      const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * NPOS + wp) * UTW) * KW * 256 + lane;
+      if (DSP == 1 || hf == 0) {
 #pragma unroll
       for (int r0 = 1; r0 < KW; r0 += PSRC) {
         constexpr int NWR = PSRC * UTW * E;
@@ -1023,6 +1051,7 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
               for (int e = 0; e < E; ++e) ds[u][e][0] += part_value((PT*)0, v[(rr * UTW + u) * E + e]);
           }
+      }
       }
     }
     if constexpr (RC && KW == 1) {
@@ -1120,7 +1149,7 @@ fused_bwd_kernel(const BwdArgs a) {
         v += __shfl_xor(v, 1); v += __shfl_xor(v, 2);
         if (TR >= 8) v += __shfl_xor(v, 4);
         if (TR == 16) v += __shfl_xor(v, 8);
-        if (brow == 0) a.dbp[(((size_t)bt * GT + g) * N + n) * D + ub[u] + esub + e] = v;
+        if (brow == 0 && (DSP == 1 || hf == 0)) a.dbp[(((size_t)bt * GT + g) * N + n) * D + ub[u] + esub + e] = v;
       }
   }
 }

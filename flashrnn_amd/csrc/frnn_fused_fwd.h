@@ -78,7 +78,9 @@ fused_fwd_kernel(const FwdArgs a) {
   typedef typename X::Frag Frag;
   typedef Own<TR> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
-  constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW;
+  // (KSP = 2: the fp32 4x4x1 form of heads from 384 units on, two waves per tile, each with one half of k)
+  constexpr int KSP = fwd_k_split(GR, D, WAVES, UTW, TR, (int)sizeof(T)), DK = D / KSP;
+  constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW / KSP;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
   constexpr int LLW = 16 * D / X::EPW;  // 64-bit words per exchange slot
   // words a thread polls per step: the TR rows of the tile, without the workgroup's own slice
@@ -98,8 +100,8 @@ fused_fwd_kernel(const FwdArgs a) {
   // instruction computes 16 columns, 12 of them padding, at the same rate).  Block = unit of the tile, the 4
   // columns of a block = the gates of that unit, A = h (the values of one block broadcast to all 16), one
   // instruction per k: D instructions of 8 cycles per tile and step instead of G_r * D / 4 of 32.
-  constexpr int RLK = fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
   constexpr bool M44 = fwd_form_4x4x1(GR, D, WAVES, UTW, TR, (int)sizeof(T));  // (the whole operand, D registers per tile, in registers)
+  constexpr int RLK = M44 ? 0 : fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
   // Own slice first: of the h_(t-1) a step multiplies with, the workgroup's own D / KW units are in LDS as soon as
   // its waves have finished step t-1; the k-steps over them run before the wait for the other workgroups' slices
   // (behind one more LDS barrier) and leave the critical path.  Each workgroup keeps R and h rotated along k so
@@ -130,6 +132,7 @@ fused_fwd_kernel(const FwdArgs a) {
   __shared__ __attribute__((aligned(16))) T obuf[PST ? 2 * OB : 1];
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
+  __shared__ f32x4 psum[KSP > 1 ? UT_WG * 64 : 1];  // partial sums of the second wave of a pair: [tile][lane]
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -140,7 +143,10 @@ fused_fwd_kernel(const FwdArgs a) {
   const int r16 = lane & 15, q4 = lane >> 4;
   const int brow = O::row(r16), esub = O::sub(r16, q4);
   const int bg = bt * TR + brow;  // batch row this lane does the gate math for
-  const bool bvalid = bg < B;
+  // wave w of a pair-split workgroup: tile w / 2 of the workgroup, half w % 2 of k; the lanes of a second-half wave
+  // own no element (every load of theirs returns zero, every store is dropped)
+  const int kh = KSP > 1 ? w % KSP : 0, wt = KSP > 1 ? w / KSP : w;
+  const bool bvalid = bg < B && kh == 0;
   const int rows_valid = min(TR, B - bt * TR);
   const unsigned Bpad = (unsigned)B;  // rows of the gate cache: padded rows are never read or written
   const T* __restrict__ R = static_cast<const T*>(a.R);
@@ -270,7 +276,7 @@ fused_fwd_kernel(const FwdArgs a) {
   unsigned wx_v[UTW], st_v[UTW], ca_v[UTW];  // per-lane byte offsets; out of range for padded rows
 #pragma unroll
   for (int u = 0; u < UTW; ++u) {
-    ub[u] = (slice * UT_WG + w * UTW + u) * 16;
+    ub[u] = (slice * UT_WG + wt * UTW + u) * 16;
     const unsigned d0 = n * D + ub[u] + esub;
     if constexpr (MB) {
       mi_v[u] = bvalid ? ((unsigned)bg * ND + d0) * RI::BYTES : kInvalidOff;
@@ -288,14 +294,14 @@ fused_fwd_kernel(const FwdArgs a) {
   const int rot_ks = OWN_FIRST ? slice * KSO : 0, rot_u = OWN_FIRST ? slice * (D / KW) : 0;  // rotation in k-steps, in units
   Frag* const rl = rlds + (size_t)w * RLK * UTW * GR * 64 + lane;
   // 4x4x1 form: lane 4*blk + j holds row (gate j, unit blk of the tile) of R, one register per k
-  float rb[M44 ? UTW : 1][M44 ? D : 1];
+  float rb[M44 ? UTW : 1][M44 ? DK : 1];
   if constexpr (M44) {
     const int blk = lane >> 2, j = lane & 3;
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-      const float* row = reinterpret_cast<const float*>(R) + ((size_t)((j < GR ? j : 0) * N + n) * D + ub[u] + blk) * D;
+      const float* row = reinterpret_cast<const float*>(R) + ((size_t)((j < GR ? j : 0) * N + n) * D + ub[u] + blk) * D + kh * DK;
 #pragma unroll
-      for (int k = 0; k < D; k += 4) {
+      for (int k = 0; k < DK; k += 4) {
         const float4 v = *reinterpret_cast<const float4*>(row + k);
         rb[u][k] = j < GR ? v.x : 0.f; rb[u][k + 1] = j < GR ? v.y : 0.f;
         rb[u][k + 2] = j < GR ? v.z : 0.f; rb[u][k + 3] = j < GR ? v.w : 0.f;
@@ -303,10 +309,10 @@ fused_fwd_kernel(const FwdArgs a) {
 #ifndef FRNN_NO_AGPR_PIN
       // (as for the fragments below: what does not fit the architectural VGPRs beside the working set is pinned to
       // accumulation registers, where the MFMA reads it in place, instead of being copied back before every use)
-      constexpr int PIN44 = UTW * D - 128 > 232 ? 232 : UTW * D - 128;
+      constexpr int PIN44 = UTW * DK - 128 > 232 ? 232 : UTW * DK - 128;
 #pragma unroll
-      for (int k = 0; k < D; ++k)
-        if (u * D + (D - 1 - k) < PIN44) asm volatile("" : "+a"(rb[u][k]));
+      for (int k = 0; k < DK; ++k)
+        if (u * DK + (DK - 1 - k) < PIN44) asm volatile("" : "+a"(rb[u][k]));
 #endif
     }
   }
@@ -500,23 +506,32 @@ fused_fwd_kernel(const FwdArgs a) {
     f32x4 acc[UTW][GR];
     float ry44[M44 ? UTW : 1][4];  // 4x4x1 form: the lane's element, gates 0..3
     if constexpr (M44) {
-      const float* hf = reinterpret_cast<const float*>(hbuf[cur]) + lane;
-      float ha[D / 16];
+      const float* hf = reinterpret_cast<const float*>(hbuf[cur]) + lane + kh * DK * 4;  // (this wave's half of k)
+      float ha[DK / 16];
 #pragma unroll
-      for (int v = 0; v < D / 16; ++v) ha[v] = hf[64 * v];
+      for (int v = 0; v < DK / 16; ++v) ha[v] = hf[64 * v];
       __builtin_amdgcn_sched_barrier(0);
       f32x4 ac[UTW][4];  // 4 independent accumulation chains per tile
 #pragma unroll
-      for (int v = 0; v < D / 16; ++v) {
+      for (int v = 0; v < DK / 16; ++v) {
 #pragma unroll
         for (int u = 0; u < UTW; ++u) mfma_4x4x1_bcast16(ha[v], &rb[u][16 * v], ac[u], v == 0);
       }
+      f32x4 sum[UTW];
 #pragma unroll
       for (int u = 0; u < UTW; ++u) {
-        const f32x4 sum = (ac[u][0] + ac[u][1]) + (ac[u][2] + ac[u][3]);
+        sum[u] = (ac[u][0] + ac[u][1]) + (ac[u][2] + ac[u][3]);
+        if constexpr (KSP > 1) { if (kh != 0) psum[(wt * UTW + u) * 64 + lane] = sum[u]; }
+      }
+      // (the buffer is free again before the second wave's next write: the barrier of the next step's exchange wait,
+      // which every pair-split tiling has, lies in between)
+      if constexpr (KSP > 1) lds_barrier();
+#pragma unroll
+      for (int u = 0; u < UTW; ++u) {
+        if constexpr (KSP > 1) { if (kh == 0) sum[u] += psum[(wt * UTW + u) * 64 + lane]; }
         // lane 4*blk + j holds (gate j, unit blk) of batch rows 0..3; after the transpose lane 4*blk + b holds
         // gates 0..3 of (batch row b, unit blk): the element that Own<4> gives this lane
-        ry44[u][0] = sum[0]; ry44[u][1] = sum[1]; ry44[u][2] = sum[2]; ry44[u][3] = sum[3];
+        ry44[u][0] = sum[u][0]; ry44[u][1] = sum[u][1]; ry44[u][2] = sum[u][2]; ry44[u][3] = sum[u][3];
         quad_transpose(ry44[u], lane);
       }
     }
@@ -615,6 +630,7 @@ fused_fwd_kernel(const FwdArgs a) {
       asm volatile("" ::"v"(sink)); }
 #endif
     FRNN_STAMP(c2);
+    if (KSP == 1 || kh == 0) {  // (wave-uniform: the second wave of a pair has handed its sums over)
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
       float ryv[GR][E], wxv[GW][E];
@@ -681,6 +697,7 @@ fused_fwd_kernel(const FwdArgs a) {
       if constexpr (NC > 0)
         buf_store_wide<NWC>(cache_pack<T, NCA, E>(cv), rCa, ca_v[u], (((unsigned)t * N + n) * (D / 16)) * Bpad * 16 * NCP * ES);
       }
+    }
     }
 #ifdef FRNN_TRACE
     FRNN_STAMP(c3);

@@ -40,8 +40,14 @@ constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
 // Forward kernel, fp32 at 4-row tiles, cells with 3 or 4 recurrent gates: the product runs on v_mfma_f32_4x4x1_16B_f32
 // (see the kernel), when the whole operand, D registers per tile in that form, fits the registers of a wave
 // (workgroups of up to 4 waves: 512 registers each).
+// Heads from 384 units on: the four waves of a workgroup pair up over two tiles, each wave of a pair keeps R for one half
+// of k (D / 2 registers) and multiplies it with that half of h; the second wave hands its partial sums to the first
+// through LDS, which alone does the gate math of the tile.  D = 16 * (WAVES / 2) * KW for these tilings.
+constexpr int fwd_k_split(int GR, int D, int WAVES, int UTW, int TR, int esize) {
+  return esize == 4 && TR == 4 && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 ? 2 : 1;
+}
 constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esize) {
-  return esize == 4 && TR == 4 && GR >= 3 && WAVES <= 4 && UTW * D <= 384;
+  return esize == 4 && TR == 4 && GR >= 3 && WAVES <= 4 && UTW * D / fwd_k_split(GR, D, WAVES, UTW, TR, esize) <= 384;
 }
 // Forward kernel: one more wave per workgroup that fetches Wx for the compute waves.  A vector memory instruction that a
 // compute wave issues behind the exchange wait delays its MFMAs (~70 cycles each on the chain of dependent steps), one
@@ -86,6 +92,13 @@ constexpr int bwd_producer_bytes(int nc, int s, int ut_wg, int TR, int esize) {
 constexpr bool bwd_producer_stores(int GR, int nc, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
   return bwd_producer_wave(GR, nc, D, WAVES, UTW, KW, TR, esize, rc) && WAVES <= 6;
 }
+// Backward kernel, fp32 4x4x1 form, gated cells at heads from 384 units on: the four waves of a workgroup pair up over two
+// tile positions, and each wave of a pair keeps R^T (own gate rows x destinations) for every second group of 4
+// destination workgroups (G_r * D / 8 registers instead of G_r * D / 4) and sends those groups' partial sums itself;
+// the first wave of a pair alone owns the pair's elements (gate math, loads, stores, receive).  D = 16 * (WAVES / 2) * KW.
+constexpr int bwd_dest_split(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
+  return esize == 4 && TR == 4 && !rc && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 && KW >= 8 ? 2 : 1;
+}
 // Backward kernel: LDS bytes of the two dWx hand-over buffers of the producer-store instantiations
 // ([gate][row][unit], and [row][unit] for the GRU's g-gate cotangent), behind the operand hand-over buffers
 constexpr int bwd_producer_store_bytes(int gw, bool gru, int D, int TR, int esize) {
@@ -125,21 +138,23 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
   X(160, 2, 2, 1, 5, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 4, 1, 3, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
-// fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave, so D = 512 is as far as one tile per
-// wave goes (2 waves per workgroup from D = 448 on, part of R in LDS); larger heads run on the alternating backend
+// fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave (D in the 4x4x1 form of the 4-row tiles), so
+// D = 512 is as far as the fused kernels go; larger heads run on the alternating backend.  Forward, D = 384 .. 512:
+// workgroups of two wave pairs, 4-row tiles only (see fwd_k_split; D = 16 * (WAVES / 2) * KW)
 #define FRNN_PLANS_GR4_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
-  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 8) X(448, 0, 2, 1, 14, 4) X(512, 0, 2, 1, 16, 4)
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
+// (backward, D = 384 .. 512: workgroups of two wave pairs, 4-row tiles only; see bwd_dest_split)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
   X(320, 2, 1, 1, 20, 4) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
-  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 4) X(448, 0, 2, 1, 14, 8) X(512, 0, 1, 1, 32, 4)
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
 // slstm fp32 backward: the same without the 20-workgroup tiling of D = 320 (with four states its kernel spills)
 #define FRNN_BWD_PLANS_SLSTM_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
-  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 6, 4) X(448, 0, 2, 1, 14, 8) X(512, 0, 1, 1, 32, 4)
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
@@ -150,11 +165,11 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_PLANS_GR3_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
-  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 8) X(512, 0, 4, 1, 8, 8)
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
 #define FRNN_BWD_PLANS_GR3_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
-  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 8) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 8)
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \

@@ -61,7 +61,8 @@ FUSED_SMALL = [
     ("slstm", 4, 6, 1, 640, "bfloat16"),
     ("gru", 6, 4, 1, 640, "bfloat16"),
     ("elman", 12, 5, 1, 640, "bfloat16"),
-    # fp32 beyond D = 256 (5 to 32 workgroups per head; from 384 on part of R / R^T lives in LDS)
+    # fp32 beyond D = 256 (5 to 16 workgroups per head; gated cells from 384 on: workgroups of two wave pairs, the waves
+    # of a pair split k (forward) or the destination workgroups (backward) between them)
     ("lstm", 6, 5, 1, 160, "float32"),
     ("gru", 5, 6, 2, 160, "float32"),
     ("elman", 9, 5, 1, 160, "float32"),      # 10 waves
@@ -71,14 +72,17 @@ FUSED_SMALL = [
     ("lstm", 9, 4, 1, 384, "float32"),
     ("gru", 6, 5, 1, 384, "float32"),
     ("elman", 5, 6, 1, 384, "float32"),
-    ("lstm", 5, 5, 1, 448, "float32"),       # 14 workgroups of 2 waves
+    ("slstm", 7, 6, 2, 384, "float32"),      # 12 workgroups per head: 3 groups of 4 destinations, 2 + 1 over a wave pair
+    ("lstm", 5, 5, 1, 448, "float32"),       # 14 workgroups per head
     ("gru", 7, 4, 1, 448, "float32"),
-    ("lstm", 6, 6, 1, 512, "float32"),       # forward 16 workgroups of 2 waves, backward 32 of one wave
+    ("slstm", 3, 5, 1, 448, "float32"),
+    ("lstm", 6, 6, 1, 512, "float32"),       # 16 workgroups per head
     ("slstm", 4, 5, 1, 512, "float32"),
     ("gru", 9, 4, 1, 512, "float32"),
     ("elman", 7, 5, 1, 768, "float32"),
     ("elman", 10, 4, 1, 1024, "float32"),
-    ("lstm", 37, 4, 1, 512, "float32"),      # 10 groups of 4 rows: two backward launches (8 groups of 32 workgroups each)
+    ("lstm", 37, 4, 1, 512, "float32"),      # 10 groups of 4 rows, the last with one valid row
+    ("gru", 70, 4, 1, 384, "float32"),       # 18 groups of 12 workgroups: two launches
     # elman fp32 from D = 128 on: D / 64 workgroups of one tile per wave
     ("elman", 6, 5, 2, 128, "float32"),
     ("elman", 21, 4, 1, 192, "float32"),
