@@ -28,7 +28,7 @@ WORKLOADS = {
     "C5": dict(function="elman", dtype="bfloat16", B=32, T=1024, N=1, D=1024, init="zeros", grad_on="all", bwd=True, seed=1005),
 }
 GATES_R = {"lstm": 4, "slstm": 4, "gru": 3, "elman": 1}
-PEAK_TFLOPS = {"bfloat16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, published
+PEAK_TFLOPS = {"bfloat16": 2500.0, "float16": 2500.0, "float32": 157.3}  # MI355X dense MFMA, published
 # roofline.traffic comes from the committed counter profiles of the same commands, never from a constant in this file:
 # a profile holds one "traffic:" line per kernel template it measured (FETCH_SIZE and WRITE_SIZE in KiB per dispatch
 # and the factors a plain 256 MiB copy gave in the same run; for the alternating backend per call, all step launches
@@ -470,7 +470,7 @@ def main():
                   else f"tokens/s {describe(w)}",
         "value": tokens / (ms * 1e-3), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": ms, "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16" if w["dtype"] == "bfloat16" else "f32", "data": "synthetic",
+        "dtype": {"bfloat16": "bf16", "float16": "f16", "float32": "f32"}[w["dtype"]], "data": "synthetic",
         "config": {"workload": f"{args.workload}: {describe(w)}", "backend": backend, "seed": w["seed"],
                    "gate_cache": "recomputed in the backward pass" if args.recompute and backend == "hip_fused" else "stored",
                    "timed": "flashrnn() + torch.autograd.grad through the C ABI, inputs resident in HBM"},

@@ -287,7 +287,8 @@ static int check_problem(int function, int dtype, int B, int T, int N, int D) {
 }
 // gate cache of the fused kernels: NC values per element, padded to whole dwords (CacheBlk in frnn_common.h)
 static size_t fused_cache_bytes_of(int function, int dtype, int B, int T, int N, int D) {
-  const int nc = cell_dims(function).NC, ncp = dtype_size(dtype) == 2 ? (nc + 1) / 2 * 2 : nc;
+  const int nc = cell_dims(function).NC + (cache_carried_state(function, (int)dtype_size(dtype), D) >= 0 ? 1 : 0);
+  const int ncp = dtype_size(dtype) == 2 ? (nc + 1) / 2 * 2 : nc;
   return (size_t)T * N * B * D * ncp * dtype_size(dtype);
 }
 // the fused kernels address each tensor with 32-bit byte offsets

@@ -47,6 +47,20 @@ inline CellDims cell_dims(int f) {
 }
 inline int dtype_size(int dt) { return dt == FRNN_F32 ? 4 : 2; }
 
+// Gate cache of the fused kernels: a value of s_(t-1) that the adjoint of step t needs may travel in the cache line of
+// step t (the forward kernel has it in a register when it writes the line), so that the reverse kernel issues one load
+// less per step (a vector memory instruction costs a wave ~30 cycles to issue, in front of the step's chain).
+//   sLSTM, 16-bit types: c_(t-1) in the sixth slot, which the padding of its five values to whole dwords leaves free:
+//          B16 T1024 N4 D192 backward 1.002 -> 0.977 ms, B16 T4096 N4 D192 fwd+bwd 7.97 -> 7.85, N3 D256 +-1 %.
+//   LSTM:  measured with c_(t-1) as a fifth value for heads from 256 units on (4 -> 6 padded values, 12 instead of 8
+//          bytes per element and step): backward D = 256 +1 %, D = 512 -2.6 %, D = 768 -1.5 %; not worth half as much
+//          cache again, so its lines stay at four values.  fp32 lines have no padding.
+// Returns the index of the carried state, or -1.  The layout depends on (function, storage type, head dim) only, never
+// on the tiling.
+constexpr int cache_carried_state(int function, int esize, int /*D*/) {
+  return esize == 2 && function == FRNN_SLSTM ? 1 : -1;
+}
+
 // ---------------------------------------------------------------------------------------
 // Storage-type traits.
 //  KM   : K extent of one MFMA (bf16: v_mfma_f32_16x16x32_bf16, f32: v_mfma_f32_16x16x4_f32)

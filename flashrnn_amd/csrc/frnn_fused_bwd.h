@@ -117,7 +117,9 @@ fused_bwd_kernel(const BwdArgs a) {
   constexpr int KS = KDL / X::KM;
   static_assert(KDL % X::KM == 0 && DL % 8 == 0, "own gate rows must fill whole k-steps");
   constexpr int KE = X::KM / 4;         // consecutive k held by one lane of a fragment
-  constexpr int NCA = NC > 0 ? NC : 1;
+  // (values per element of a cache line: the cell's NC and, where cache_carried_state says so, one state of step t-1)
+  constexpr int CXS = RC ? -1 : cache_carried_state(F, (int)sizeof(T), D), NCX = NC + (CXS >= 0 ? 1 : 0);
+  constexpr int NCA = NCX > 0 ? NCX : 1;
   // remote sources polled together: every round of polling costs at least one trip to L2 and back,
   // so as few rounds as 16 words per lane and probe allow, of equal size (no dummy loads)
   constexpr int RC_MAX = 16 / (UTW * (TR / 4)) > 0 ? 16 / (UTW * (TR / 4)) : 1;
@@ -193,7 +195,10 @@ fused_bwd_kernel(const BwdArgs a) {
   constexpr bool PW = bwd_producer_wave(GR, NC, D, WAVES, UTW, KW, TR, (int)sizeof(T), RC);
   // one buffer: [cache: tile][row][16 units][NCP values] [s_(t-1): state][tile][row][16 units] [cotangent: the same]
   constexpr int PB_CA = NC > 0 ? UT_WG * TR * 16 * NCP : 0, PB_ST = S * UT_WG * TR * 16, PB = PB_CA + 2 * PB_ST;
-  static_assert(!PW || 2 * PB * (int)sizeof(T) + 16 == bwd_producer_bytes(NC, S, UT_WG, TR, (int)sizeof(T)), "hand-over buffer size");
+  static_assert(!PW || 2 * PB * (int)sizeof(T) + 16 == bwd_producer_bytes(NCX, S, UT_WG, TR, (int)sizeof(T)), "hand-over buffer size");
+  // the carried state comes out of the cache line instead of a load of its own (the kernels with a producer wave keep the
+  // load: it is the producer's, off the compute waves' chain)
+  constexpr bool CXU = CXS >= 0 && !PW;
   T* const pbuf = reinterpret_cast<T*>(smem_raw + bwd_lds_bytes(GR, D, WAVES, UTW, KW, (int)sizeof(T)));
   // Producer-wave stores (PSTV instantiations, chosen on the host for launches that fill the device; see the forward
   // kernel): the compute waves leave dWx_t (and the GRU's g-gate cotangent) in LDS as they lie in memory, two buffers by
@@ -525,6 +530,7 @@ fused_bwd_kernel(const BwdArgs a) {
       for (int k = 0; k < S; ++k) {
         const unsigned so = ((unsigned)k * BS * Tn + t) * ND * ES;
         p.dso[u][k] = buf_load<ND_, SB>(rDs, st_v[u], so);
+        if (CXU && k == CXS) continue;
         p.sp[u][k] = buf_load<ND_, SB>(rPrev, first ? s0_v[u] : st_v[u], first ? (unsigned)k * BS * ND * ES : so - ND * ES);
       }
     }
@@ -673,7 +679,14 @@ fused_bwd_kernel(const BwdArgs a) {
       }
 #pragma unroll
       for (int k = 0; k < S; ++k) {
-        unpack<E>(pc.sp[u][k], spv[k], (T*)0); unpack<E>(sn[u][k], snv[k], (T*)0); unpack<E>(pc.dso[u][k], dsov[k], (T*)0);
+        unpack<E>(sn[u][k], snv[k], (T*)0); unpack<E>(pc.dso[u][k], dsov[k], (T*)0);
+        if (CXU && k == CXS) {  // (from the cache line; packed again, exactly, for the next step)
+#pragma unroll
+          for (int e = 0; e < E; ++e) spv[k][e] = cv[NC][e];
+          sn[u][k] = pack<E>(cv[NC], (T*)0);
+          continue;
+        }
+        unpack<E>(pc.sp[u][k], spv[k], (T*)0);
         sn[u][k] = pc.sp[u][k];  // s_(t-1) is the s_t of the next step
       }
       float dgr[GR][E], dgw[GW][E];

@@ -89,7 +89,9 @@ fused_fwd_kernel(const FwdArgs a) {
   // 16-bit types fetch two adjacent words with one 16-byte load when a thread polls more than one
   constexpr bool PAIRS = X::EPW == 2 && NP_ > 1;
   constexpr int NP = NP_ <= 16 ? (PAIRS ? (NP_ + 1) / 2 * 2 : NP_) : (NP_ + 15) / 16 * 16;
-  constexpr int NCA = NC > 0 ? NC : 1;
+  // (values per element of a cache line: the cell's NC and, where cache_carried_state says so, one state of step t-1)
+  constexpr int CXS = cache_carried_state(F, (int)sizeof(T), D), NCX = NC + (CXS >= 0 ? 1 : 0);
+  constexpr int NCA = NCX > 0 ? NCX : 1;
   constexpr int GX = GT - GR > 0 ? GT - GR : 1;
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
   constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
@@ -124,7 +126,7 @@ fused_fwd_kernel(const FwdArgs a) {
   // the compute waves leave the step's states and cache values in LDS as they lie in memory, two buffers by step
   // parity, and the producer wave stores them one step later in 16-byte pieces.
   constexpr bool PST = PSTV && PW && KW == 1;
-  constexpr int NCP_O = CacheBlk<T, (NC > 0 ? NC : 1)>::NCP;
+  constexpr int NCP_O = CacheBlk<T, NCA>::NCP;
   // (rows of the state part are D + 8 elements apart: at a stride of 128 bytes, D = 64, rows 0 and 2 of a tile would meet
   // in the same banks under the lanes' 2-byte writes)
   constexpr int OBR = D + 8;
@@ -657,10 +659,11 @@ fused_fwd_kernel(const FwdArgs a) {
         for (int g = 0; g < GR; ++g) ry[g] = ryv[g][e];
 #pragma unroll
         for (int g = 0; g < GW; ++g) wx[g] = wxv[g][e];
+        if constexpr (CXS >= 0) cc[NC] = s[u][e][CXS];  // (before the step overwrites it)
         CM::fwd(ry, wx, bx[u][e], s[u][e], cc);
         s[u][e][0] = clamp_if(s[u][e][0], a.h_clip);
 #pragma unroll
-        for (int c = 0; c < NC; ++c) cv[c][e] = cc[c];
+        for (int c = 0; c < NCX; ++c) cv[c][e] = cc[c];
 #pragma unroll
         for (int k = 0; k < S; ++k) so[k][e] = s[u][e][k];
       }

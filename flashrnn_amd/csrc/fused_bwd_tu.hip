@@ -25,7 +25,7 @@ int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream
   const bool pw = bwd_producer_wave(Cell<FRNN_F>::GR, Cell<FRNN_F>::NC, p.D, p.waves, p.utw, p.kw, a.tile_rows, (int)sizeof(FRNN_TU_T), rc);
   const bool pst = a.pst && !a.cut && bwd_producer_stores(Cell<FRNN_F>::GR, Cell<FRNN_F>::NC, p.D, p.waves, p.utw, p.kw, a.tile_rows, (int)sizeof(FRNN_TU_T), rc);  // (the truncated scan has no barrier per step to hand over at)
   const size_t lds = bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T), rc) + 16 +
-                     (pw ? bwd_producer_bytes(Cell<FRNN_F>::NC, Cell<FRNN_F>::S, p.waves * p.utw, a.tile_rows, (int)sizeof(FRNN_TU_T)) : 0) +
+                     (pw ? bwd_producer_bytes(Cell<FRNN_F>::NC + (cache_carried_state(FRNN_F, (int)sizeof(FRNN_TU_T), p.D) >= 0 ? 1 : 0), Cell<FRNN_F>::S, p.waves * p.utw, a.tile_rows, (int)sizeof(FRNN_TU_T)) : 0) +
                      (pst ? bwd_producer_store_bytes(Cell<FRNN_F>::GW, FRNN_F == FRNN_GRU, p.D, a.tile_rows, (int)sizeof(FRNN_TU_T)) : 0);
 #define FRNN_CASE_(RCV, Dv, VAR, W, U, K, MTR)                                                          \
   if (rc == RCV && p.D == Dv && p.waves == W && p.utw == U && p.kw == K) {                               \

@@ -79,7 +79,7 @@ def test_plan_and_sizes(lib):
     waves, utw, kw, active = (o.value for o in out)
     # workgroups = heads x batch tiles (of 4, 8 or 16 rows, by the compute units at hand) x kw
     assert 16 * waves * utw * kw == 256 and active in (3 * kw, 6 * kw)
-    # gate cache: T * N * B * D * values (padded to whole dwords: sLSTM bf16 5 -> 6) * bytes
+    # gate cache: T * N * B * D * values (padded to whole dwords: sLSTM bf16 5 -> 6, the sixth carries c_(t-1)) * bytes
     assert lib.frnn_fused_cache_bytes(L, 0, 8, 1024, 3, 256) == 1024 * 3 * 8 * 256 * 4 * 2
     assert lib.frnn_fused_cache_bytes(_lib.FUNCTION_IDS["slstm"], 0, 8, 16, 3, 256) == 16 * 3 * 8 * 256 * 6 * 2
     assert lib.frnn_fused_cache_bytes(_lib.FUNCTION_IDS["slstm"], 1, 8, 16, 3, 256) == 16 * 3 * 8 * 256 * 5 * 4
