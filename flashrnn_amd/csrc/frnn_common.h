@@ -22,17 +22,21 @@ typedef unsigned long long u64;
 // R fills the first GR of the GI interacting slots, Wx the last GW, b covers all GT.
 // NC = values cached per element for the backward pass (private layout; LSTM: the four activated
 // gates, GRU: g, r, z and the candidate n, sLSTM: i', f', tanh z, sigmoid o, sigmoid(-f)).
+// SPM / DSM = bit masks of the state planes that the adjoint reads at all: plane k of s_(t-1) (as the previous state of
+// step t or as the new state of step t-1), plane k of the cotangent of the states.  The LSTM's adjoint never reads h, the
+// sLSTM's neither m nor a cotangent of m.  A wave that loads operands for others (the reverse kernel's producer wave)
+// skips the planes outside the masks; a lane that loads for itself needs no mask, its unused loads are never emitted.
 // ---------------------------------------------------------------------------------------
 template <int F> struct Cell;
-template <> struct Cell<FRNN_LSTM>  { static constexpr int GR = 4, GW = 4, GT = 4, S = 2, NC = 4; };
-template <> struct Cell<FRNN_SLSTM> { static constexpr int GR = 4, GW = 4, GT = 4, S = 4, NC = 5; };
-template <> struct Cell<FRNN_GRU>   { static constexpr int GR = 3, GW = 3, GT = 4, S = 1, NC = 4; };
-template <> struct Cell<FRNN_ELMAN> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 0; };
+template <> struct Cell<FRNN_LSTM>  { static constexpr int GR = 4, GW = 4, GT = 4, S = 2, NC = 4, SPM = 0x2, DSM = 0x3; };
+template <> struct Cell<FRNN_SLSTM> { static constexpr int GR = 4, GW = 4, GT = 4, S = 4, NC = 5, SPM = 0x7, DSM = 0x7; };
+template <> struct Cell<FRNN_GRU>   { static constexpr int GR = 3, GW = 3, GT = 4, S = 1, NC = 4, SPM = 0x1, DSM = 0x1; };
+template <> struct Cell<FRNN_ELMAN> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 0, SPM = 0x1, DSM = 0x1; };
 // Internal variant of the Elman cell for forward_clipval: the stored h is clamped, so the adjoint cannot
 // rebuild tanh' from it and the forward pass caches the unclamped value, as the reference does
 // (flashrnn/flashrnn/fused/elman_fused_pointwise.cuh:34-60).  Not a function id of the C ABI.
 enum { FRNN_ELMAN_CLIP = 4 };
-template <> struct Cell<FRNN_ELMAN_CLIP> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 1; };
+template <> struct Cell<FRNN_ELMAN_CLIP> { static constexpr int GR = 1, GW = 1, GT = 1, S = 1, NC = 1, SPM = 0x0, DSM = 0x1; };
 
 struct CellDims { int GR, GW, GT, S, NC; };
 inline CellDims cell_dims(int f) {

@@ -214,7 +214,7 @@ fused_bwd_kernel(const BwdArgs a) {
       constexpr int CPR = NCP * 2;  // 16-byte pieces per (tile, batch row) of the cache
       constexpr int CP_TOT = NC > 0 ? UT_WG * TR * CPR : 0, NPC = (CP_TOT + 63) / 64;
       constexpr int SP_TOT = S * UT_WG * TR * 2, NPS = (SP_TOT + 63) / 64;  // pieces of 8 units of one state, tile and row
-      unsigned cvo[NPC > 0 ? NPC : 1], svo[NPS], s0o[NPS]; int cl[NPC > 0 ? NPC : 1], sl[NPS];
+      unsigned cvo[NPC > 0 ? NPC : 1], svo[NPS], spo[NPS], s0o[NPS]; int cl[NPC > 0 ? NPC : 1], sl[NPS];
 #pragma unroll
       for (int i = 0; i < NPC; ++i) {
         const int c = lane + 64 * i, q = c % CPR, pr = (c / CPR) % TR, ptile = c / (CPR * TR);
@@ -227,8 +227,11 @@ fused_bwd_kernel(const BwdArgs a) {
         const int c = lane + 64 * i, half = c & 1, pr = (c >> 1) % TR, ptile = ((c >> 1) / TR) % UT_WG, pk = (c >> 1) / (TR * UT_WG);
         const bool ok = c < SP_TOT && bt * TR + pr < B;
         const unsigned col = n * D + slice * DL + ptile * 16 + half * 8;
-        svo[i] = ok ? ((((unsigned)(pk * BS + bt * TR + pr) * Tn) * ND + col) * ES) : kInvalidOff;   // + t * ND * ES
-        s0o[i] = ok ? (((unsigned)(pk * BS + bt * TR + pr) * ND + col) * ES) : kInvalidOff;
+        // (planes that the cell's adjoint never reads: out of range, no memory traffic; their LDS slots hold zeros)
+        const bool oks = ok && ((C::SPM >> pk) & 1), okd = ok && ((C::DSM >> pk) & 1);
+        svo[i] = okd ? ((((unsigned)(pk * BS + bt * TR + pr) * Tn) * ND + col) * ES) : kInvalidOff;   // + t * ND * ES
+        spo[i] = oks ? ((((unsigned)(pk * BS + bt * TR + pr) * Tn) * ND + col) * ES) : kInvalidOff;
+        s0o[i] = oks ? (((unsigned)(pk * BS + bt * TR + pr) * ND + col) * ES) : kInvalidOff;
         sl[i] = c < SP_TOT ? ((pk * UT_WG + ptile) * TR + pr) * 16 + half * 8 : -1;
       }
       struct Ops { Dw<4> ca[NPC > 0 ? NPC : 1], sp[NPS], dso[NPS]; };
@@ -242,7 +245,7 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
         for (int i = 0; i < NPS; ++i) {
           o.dso[i] = buf_load<4>(rDs, svo[i], (unsigned)t * ND * ES);
-          o.sp[i] = buf_load<4>(rPrev, first ? s0o[i] : svo[i], first ? 0u : (unsigned)(t - 1) * ND * ES);
+          o.sp[i] = buf_load<4>(rPrev, first ? s0o[i] : spo[i], first ? 0u : (unsigned)(t - 1) * ND * ES);
         }
       };
       // (no branch on the lane: behind one the compiler waits for every load in flight, the latest ones included;
