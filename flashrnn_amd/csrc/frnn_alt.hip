@@ -89,9 +89,41 @@ __global__ void __launch_bounds__(256) alt_step_fwd_kernel(const AltStepFwdArgs 
     f32x4 acc[GR];
 #pragma unroll
     for (int g = 0; g < GR; ++g) acc[g] = f32x4{0.f, 0.f, 0.f, 0.f};
+    // fp32: a fragment of v_mfma_f32_16x16x4_f32 is one float per lane, and a load of 4 bytes per lane and k-step
+    // left the step waiting for hundreds of tiny loads (LSTM fp32 D = 1024: 52 us per step).  A lane takes 4
+    // consecutive k with one 16-byte load instead (k = 16 kg + 4 q4 .. + 3) and MFMA i of the group uses element i of
+    // every lane: both operands are read the same way, so every k still meets itself, in another order.
+    if constexpr (sizeof(T) == 4) {
+      const int KG = D / 16;
+      for (int kg0 = w; kg0 < KG; kg0 += 16) {  // 4 groups of this wave per round, requested together
+        float4 vf[4], af[4][GR];
+#pragma unroll
+        for (int j = 0; j < 4; ++j) {
+          const int kg = kg0 + 4 * j;
+          vf[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+#pragma unroll
+          for (int g = 0; g < GR; ++g) af[j][g] = make_float4(0.f, 0.f, 0.f, 0.f);
+          if (kg < KG) {  // uniform over the wave
+            if (bvalid) vf[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(vrow) + kg * 16 + q4 * 4);
+#pragma unroll
+            for (int g = 0; g < GR; ++g)
+              af[j][g] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(R) + ((size_t)(g * N + n) * D + d0 + r16) * D + kg * 16 + q4 * 4);
+          }
+        }
+#pragma unroll
+        for (int j = 0; j < 4; ++j)
+#pragma unroll
+          for (int g = 0; g < GR; ++g) {
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j][g].x, vf[j].x, acc[g], 0, 0, 0);
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j][g].y, vf[j].y, acc[g], 0, 0, 0);
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j][g].z, vf[j].z, acc[g], 0, 0, 0);
+            acc[g] = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j][g].w, vf[j].w, acc[g], 0, 0, 0);
+          }
+      }
+    }
     // 4 k-steps of this wave per round: all their fragments are requested before the first MFMA,
     // so a round costs one trip to L2 instead of four
-    for (int ks0 = w; ks0 < KS; ks0 += 16) {
+    for (int ks0 = w; ks0 < (sizeof(T) == 4 ? 0 : KS); ks0 += 16) {
       Frag vf[4], af[4][GR];
 #pragma unroll
       for (int j = 0; j < 4; ++j) {
@@ -196,7 +228,27 @@ __global__ void __launch_bounds__(256) alt_step_bwd_kernel(const AltStepBwdArgs 
     const T* vrow = static_cast<const T*>(a.dg_in) + ((size_t)(bvalid ? bm : 0) * N + n) * K;
     f32x4 acc = {0.f, 0.f, 0.f, 0.f};
     f32x4 acc2 = {0.f, 0.f, 0.f, 0.f};  // two chains: a dependent MFMA waits ~3x longer than an independent one
-    for (int ks0 = w; ks0 < KS; ks0 += 32) {  // 8 k-steps of this wave per round, requested together
+    if constexpr (sizeof(T) == 4) {  // (16-byte loads of 4 consecutive k per lane: see the forward kernel)
+      const int KG = K / 16;
+      for (int kg0 = w; kg0 < KG; kg0 += 32) {
+        float4 vf[8], af[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          const int kg = kg0 + 4 * j, kc = kg < KG ? kg : KG - 1;
+          vf[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(vrow) + kc * 16 + q4 * 4);
+          af[j] = *reinterpret_cast<const float4*>(reinterpret_cast<const float*>(arow) + kc * 16 + q4 * 4);
+          if (!bvalid || kg >= KG) vf[j] = make_float4(0.f, 0.f, 0.f, 0.f);
+        }
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j].x, vf[j].x, acc, 0, 0, 0);
+          acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j].y, vf[j].y, acc2, 0, 0, 0);
+          acc = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j].z, vf[j].z, acc, 0, 0, 0);
+          acc2 = __builtin_amdgcn_mfma_f32_16x16x4f32(af[j].w, vf[j].w, acc2, 0, 0, 0);
+        }
+      }
+    }
+    for (int ks0 = w; ks0 < (sizeof(T) == 4 ? 0 : KS); ks0 += 32) {  // 8 k-steps of this wave per round, requested together
       Frag vf[8], af[8];
 #pragma unroll
       for (int j = 0; j < 8; ++j) {  // out-of-range k-steps load the last one and are zeroed: branch-free (measured faster here)
