@@ -193,14 +193,15 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
 
 // ---- reverse scan in recompute mode (no gate cache): R and R^T are both resident, so only the head
 // dims whose two operands fit the registers beside the working set; same tilings as above where those
-// fit (gru D = 192 runs as 3 workgroups of 4 waves here: 12 waves have 168 registers each)
+// fit (gru D = 192 runs as 3 workgroups of 4 waves here: 12 waves have 168 registers each).  D = 320 (and 384 for the
+// GRU, three gate rows) at 4-row tiles only; the 4-gate cells spill at D = 384, the GRU at D = 512.
 #define FRNN_BWD_RC_PLANS_GR4_BF16(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) X(320, 0, 4, 1, 5, 4)
 // slstm: D = 192 stops at 8-row tiles (its 16-row kernel, with both operands resident and four states, spills)
 #define FRNN_BWD_RC_PLANS_SLSTM_BF16(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 8) X(256, 0, 4, 1, 4, 8)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 4) X(128, 0, 4, 1, 2, 16) X(192, 0, 4, 1, 3, 8) X(256, 0, 4, 1, 4, 8) X(320, 0, 4, 1, 5, 4)
 #define FRNN_BWD_RC_PLANS_GR3_BF16(X) \
-  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16)
+  X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 4) X(384, 0, 4, 1, 6, 4)
 #define FRNN_BWD_RC_PLANS_GR4_F32(X) X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16)
 #define FRNN_BWD_RC_PLANS_GR3_F32(X) X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16)
 #define FRNN_BWD_RC_PLANS_NONE(X)

@@ -22,17 +22,22 @@ CASES = [
     ("lstm", 7, 9, 1, 192, "bfloat16"),      # 3 workgroups per head
     ("lstm", 8, 16, 3, 256, "bfloat16"),     # 4 workgroups per head
     ("lstm", 33, 4, 1, 256, "float16"),
+    ("lstm", 6, 7, 1, 320, "bfloat16"),      # 5 workgroups per head: the largest head whose two operands fit the registers
+    ("lstm", 9, 5, 1, 320, "float16"),
     ("lstm", 5, 9, 2, 64, "float32"),
     ("lstm", 4, 6, 1, 32, "float32"),
     ("gru", 5, 9, 2, 64, "bfloat16"),
     ("gru", 16, 8, 4, 128, "bfloat16"),
     ("gru", 6, 5, 1, 192, "bfloat16"),
     ("gru", 7, 5, 1, 256, "bfloat16"),
+    ("gru", 5, 6, 1, 320, "bfloat16"),
+    ("gru", 10, 5, 1, 384, "bfloat16"),      # (three gate rows: one head dim further than the 4-gate cells)
     ("gru", 3, 6, 2, 32, "float32"),
     ("slstm", 8, 6, 2, 64, "bfloat16"),
     ("slstm", 6, 7, 1, 96, "bfloat16"),
     ("slstm", 16, 12, 2, 192, "bfloat16"),
     ("slstm", 12, 5, 2, 256, "bfloat16"),
+    ("slstm", 7, 6, 1, 320, "bfloat16"),
     ("slstm", 5, 8, 1, 64, "float32"),
     ("elman", 16, 7, 2, 128, "bfloat16"),    # nothing is cached for elman: the flag changes nothing
 ]
