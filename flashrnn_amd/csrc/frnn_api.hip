@@ -189,16 +189,21 @@ static bool pick_plan(int function, int dtype, int B, int N, int D, int backward
 // Batch rows per group: 4, 8 or 16.  Fewer rows per tile mean less gate math per lane and fewer
 // words to poll per step (the larger costs of a step) at the price of more workgroups and copies
 // of R, so the smallest tile is used for which every workgroup of the call still gets a compute
-// unit of its own.  Heads that run as one small workgroup (up to 4 waves, no exchange) may share a
-// compute unit four at a time (eight of up to 2 waves): one workgroup's gate math then runs while another
-// waits for memory, and only the 4-row kernels have the producer wave (measured, LSTM bf16 T = 1024, 4-row
-// against 8-row tiles: B = 340 N = 12 D = 64, 1020 workgroups, 4.07 against 4.80 ms; B = 336 N = 24 D = 32,
-// 2016 workgroups, 4.63 against 4.98; with 8 waves, D = 128, a gain for the LSTM and a loss for the GRU).
+// unit of its own.  Heads that run as one workgroup (no exchange) may share a compute unit, many at a time: one
+// workgroup's gate math then runs while another waits for memory, and in the 16-bit types only the 4-row kernels
+// have the producer wave and its 16-byte stores.  Measured (bf16, T = 1024 unless noted, 4- against 8- against 16-row
+// tiles, ms per step): LSTM B = 340 N12 D64, 1020 workgroups, 4.07 / 4.80; B = 1024 T = 256 N12 D64, 3072 workgroups, 2.52 /
+// 2.83 / 2.66; N8 D96 B = 1024 T = 256, 2048 workgroups of 6 waves, 3.60 / 3.98 / 3.66; N6 D128 (8 waves) B = 256, 384
+// workgroups, LSTM 3.04 / 3.51 / 5.46, GRU 2.52 / 2.51 / 4.20, Elman 1.06 / 1.14 / 1.52; B = 1024 T = 256, 1536 workgroups,
+// LSTM 2.64 / 2.60 / 3.00, GRU 2.27 / 2.18 / 2.56.  So: 4-row tiles up to 16 workgroups per compute unit for up to 4 waves,
+// 8 for up to 6, 4 for up to 8 (fp32, without the producer wave: 8 / 4 / 4 / 1 for 2 / 4 / 6 / more waves).
 // `largest` is the tallest tile the tiling is compiled for (Plan::max_tr: taller ones would spill registers).
-static int tile_rows_for(int B, int N, int kw, int waves, int largest) {
+static int tile_rows_for(int B, int N, int kw, int waves, int largest, int dtype) {
   const int forced = env_int("FRNN_TILE_ROWS", 0);
   if (forced == 4 || forced == 8 || forced == 16) return forced < largest ? forced : largest;
-  const long room = kw > 1 ? groups_per_launch(kw) : (long)device_cus() * (waves <= 2 ? 8 : waves <= 4 ? 4 : 1);
+  const int share = dtype != FRNN_F32 ? (waves <= 4 ? 16 : waves <= 6 ? 8 : waves <= 8 ? 4 : 1)
+                                      : (waves <= 2 ? 8 : waves <= 4 ? 4 : 1);
+  const long room = kw > 1 ? groups_per_launch(kw) : (long)device_cus() * share;
   for (int tr = 4; tr < largest; tr *= 2)
     if ((long)N * ((B + tr - 1) / tr) <= room) return tr;
   return largest;
@@ -317,7 +322,7 @@ static FusedFwdWs carve_fused_fwd(void* ws, int dtype, int B, int N, int D, cons
   Bump bp{(unsigned char*)ws, 0};
   FusedFwdWs w;
   w.status = (int*)bp.take(256);
-  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr, dtype);
   const size_t groups = (size_t)N * ((B + tr - 1) / tr);
   const size_t llw = (size_t)16 * D / (dtype == FRNN_F32 ? 1 : 2);
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * llw * 8 : 0);
@@ -336,7 +341,7 @@ static FusedBwdWs carve_fused_bwd(void* ws, int function, int dtype, int B, int 
   Bump bp{(unsigned char*)ws, 0};
   FusedBwdWs w;
   w.status = (int*)bp.take(256);
-  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr, dtype);
   const size_t bt = (B + tr - 1) / tr, groups = (size_t)N * bt;
   w.ll = (u64*)bp.take(p.kw > 1 ? groups * 3 * bwd_inbox_words(D, p.kw) * 8 : 0);
   w.xcd = (int*)bp.take(p.kw > 1 ? groups * 32 * 4 : 0);  // words of xcd_handshake
@@ -525,7 +530,7 @@ int frnn_fused_plan(int function, int dtype, int B, int N, int D, int backward,
   if (waves) *waves = p.waves;
   if (tiles_per_wave) *tiles_per_wave = p.utw;
   if (wgs_per_head) *wgs_per_head = p.kw;
-  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr, dtype);
   if (active_wgs) *active_wgs = N * ((B + tr - 1) / tr) * p.kw;
   return 0;
 }
@@ -626,7 +631,7 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
     const size_t one_group = 256 + (p.kw > 1 ? (size_t)3 * 16 * D / (dtype == FRNN_F32 ? 1 : 2) * 8 + 256 : 0);
     if (workspace_bytes < one_group) return fail(FRNN_E_WORKSPACE, "step scratch %zu < %zu bytes", workspace_bytes, one_group);
   }
-  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr, dtype);
   const int groups = N * ((B + tr - 1) / tr);
   int per_launch = groups;
   if (p.kw > 1) {  // workgroups that wait for each other must all be resident
@@ -750,7 +755,7 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   e = launch_transpose_r(dtype, R, w.Rt, N, D, c.GR, st);
   prof_end(st);
   if (e) return hip_fail(e, "R transpose");
-  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr);
+  const int tr = tile_rows_for(B, N, p.kw, p.waves, p.max_tr, dtype);
   const int bt = (B + tr - 1) / tr, groups = N * bt;
   int per_launch = groups;
   if (p.kw > 1) {
