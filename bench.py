@@ -92,10 +92,10 @@ def make_gpu_inputs(w, device):
     import torch
     from oracle import make_inputs
 
-    rt = torch.bfloat16 if w["dtype"] == "bfloat16" else None
+    kdt = {"bfloat16": torch.bfloat16, "float16": torch.float16, "float32": torch.float32}[w["dtype"]]
+    rt = kdt if kdt != torch.float32 else None
     inp = make_inputs(w["function"], w["B"], w["T"], w["N"], w["D"], w["seed"], init=w["init"], round_to=rt,
                       grad_on=w["grad_on"], forget_bias_linspace=w.get("forget_bias_linspace", False))
-    kdt = torch.bfloat16 if w["dtype"] == "bfloat16" else torch.float32
     dev = {k: v.to(device=device, dtype=kdt) for k, v in inp.items()}
     return inp, dev
 
