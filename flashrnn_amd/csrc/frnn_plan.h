@@ -87,8 +87,9 @@ constexpr bool bwd_producer_wave(int GR, int nc, int D, int WAVES, int UTW, int 
 constexpr int bwd_producer_bytes(int nc, int s, int ut_wg, int TR, int esize) {
   return 2 * ut_wg * TR * 16 * ((nc + 1) / 2 * 2 + 2 * s) * esize + 16;
 }
-// Backward kernel: may the producer wave also store dWx (see fwd_producer_stores)?  Not the 8-wave kernels: nine waves
-// have 170 registers each and the fp16 LSTM kernel spills with the extra addresses.
+// Backward kernel: may the producer wave also store dWx (see fwd_producer_stores)?  Not the 8-wave kernels (D = 128): one
+// workgroup of nine waves per compute unit is all that their 166 registers allow, and there the variant measured slower
+// (LSTM bf16 B256 T1024 N6 D128 reverse kernel 1.46 -> 1.58 ms, GRU 1.18 -> 1.21).
 constexpr bool bwd_producer_stores(int GR, int nc, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
   return bwd_producer_wave(GR, nc, D, WAVES, UTW, KW, TR, esize, rc) && WAVES <= 6;
 }

@@ -297,7 +297,10 @@ def test_slstm_mixed_fresh_and_running_elements(gpu):
 
 @pytest.mark.parametrize("function,B,T,N,D,dtype", [
     ("lstm", 336, 24, 12, 64, "bfloat16"), ("slstm", 300, 16, 12, 64, "bfloat16"), ("lstm", 340, 16, 24, 32, "bfloat16"),
-    ("gru", 336, 24, 12, 64, "float16"), ("lstm", 160, 16, 12, 64, "float32")])
+    ("gru", 336, 24, 12, 64, "float16"), ("lstm", 160, 16, 12, 64, "float32"),
+    # 8 compute waves and the producer wave, which also stores here
+    ("lstm", 300, 12, 6, 128, "bfloat16"), ("gru", 290, 10, 6, 128, "float16"), ("lstm", 270, 8, 6, 128, "float16"),
+    ("lstm", 330, 10, 8, 96, "bfloat16")])
 def test_small_heads_at_large_batches(gpu, function, B, T, N, D, dtype):
     """Heads of one workgroup keep 4-row tiles while at most four workgroups (eight of up to two waves) share a
     compute unit: here 1008, 900, 2040, 1008 and 480 workgroups in one launch."""

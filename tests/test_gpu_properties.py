@@ -341,7 +341,8 @@ def test_slstm_backward_through_the_carried_state_of_two_calls(gpu, backend):
 @pytest.mark.parametrize("function,B,T,N,D,dtype", [
     ("lstm", 9, 11, 3, 64, "bfloat16"), ("lstm", 6, 7, 5, 32, "bfloat16"), ("lstm", 5, 6, 2, 128, "bfloat16"),
     ("slstm", 7, 9, 2, 64, "bfloat16"), ("slstm", 4, 5, 3, 32, "float16"), ("gru", 10, 8, 2, 64, "bfloat16"),
-    ("gru", 3, 6, 4, 32, "bfloat16"), ("gru", 6, 5, 1, 96, "float16"), ("lstm", 4, 1, 2, 64, "bfloat16")])
+    ("gru", 3, 6, 4, 32, "bfloat16"), ("gru", 6, 5, 1, 96, "float16"), ("lstm", 4, 1, 2, 64, "bfloat16"),
+    ("gru", 7, 6, 2, 128, "bfloat16"), ("lstm", 6, 5, 1, 128, "float16")])
 def test_producer_wave_stores_give_the_same_bits(gpu, monkeypatch, function, B, T, N, D, dtype):
     """The instantiations whose producer wave stores the outputs (forward: states and gate cache; backward: dWx), which
     the host picks for launches that fill the device, only move data differently: every output and gradient must come
