@@ -302,7 +302,8 @@ def test_slstm_mixed_fresh_and_running_elements(gpu):
     ("lstm", 300, 12, 6, 128, "bfloat16"), ("gru", 290, 10, 6, 128, "float16"), ("lstm", 270, 8, 6, 128, "float16"),
     ("lstm", 330, 10, 8, 96, "bfloat16")])
 def test_small_heads_at_large_batches(gpu, function, B, T, N, D, dtype):
-    """Heads of one workgroup keep 4-row tiles while at most four workgroups (eight of up to two waves) share a
-    compute unit: here 1008, 900, 2040, 1008 and 480 workgroups in one launch."""
+    """Heads of one workgroup keep 4-row tiles up to many workgroups per compute unit (16 of up to 4 waves, 8 of up to 6,
+    4 of up to 8 in the 16-bit types): here 450 to 2040 workgroups in one launch, with the producer wave and, up to 6
+    waves, its stores in both passes."""
     print(f"case large batch {function} B{B} T{T} N{N} D{D} {dtype}", flush=True)
     check_case(gpu, function, B, T, N, D, dtype, "hip_fused", seed=5, init="randn")
