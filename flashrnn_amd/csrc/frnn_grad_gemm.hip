@@ -125,8 +125,14 @@ __global__ void __launch_bounds__(64 * WD * WD) grad_gemm16_kernel(const GradGem
   const long r_begin = (long)split * a.rows_per_split;
   const long r_end = min(rows, r_begin + a.rows_per_split);
   const size_t ND = (size_t)N * a.D;
-  // (a row of 128 units fills the 64 banks once: 8 rows, 8 groups of 8 banks; shorter rows share them)
-  auto fz = [](int row) { return TM >= 128 ? 2 * (row % 8) : 2 * ((row / (128 / TM)) % (CPR / 2)); };
+  // (a row of 128 units fills the 64 banks once: 8 rows, 8 groups of 8 banks; shorter rows share them.  Rows of 96 or
+  // 160 units, 12 or 20 chunks, start 16 banks apart modulo 64, so rows r, r + 4, r + 8, r + 12 would meet: they are
+  // shifted by 0, 2, 4, 6 chunks, with wrap-around instead of the exclusive or, which then puts two of the 16 rows of a
+  // read on every bank, as few as there can be)
+  constexpr bool POW2 = (CPR & (CPR - 1)) == 0;
+  auto fz = [](int row) { return !POW2 ? 2 * ((row / 4) % 4) : TM >= 128 ? 2 * (row % 8) : 2 * ((row / (128 / TM)) % (CPR / 2)); };
+  auto swz = [](int chunk, int f) { return POW2 ? (chunk ^ f) : (chunk + f) % CPR; };        // position of a chunk in its row
+  auto unswz = [](int pos, int f) { return POW2 ? (pos ^ f) : (pos - f + CPR) % CPR; };      // chunk at a position
 
   const T* __restrict__ G = static_cast<const T*>(a.gsrc[g]) + (size_t)n * a.D + dt * TM;
   const long gld = a.gld[g];
@@ -146,7 +152,7 @@ __global__ void __launch_bounds__(64 * WD * WD) grad_gemm16_kernel(const GradGem
     const int q = w + NW * i, j = q % (CPR / 2);
     const bool isb = q >= CPR / 2;  // uniform
     const int P = 64 * j + lane;
-    lrow[i] = P / CPR; lchunk[i] = (P % CPR) ^ fz(lrow[i]);
+    lrow[i] = P / CPR; lchunk[i] = unswz(P % CPR, fz(lrow[i]));
     voff[i] = (unsigned)(((size_t)lrow[i] * (isb ? ND : (size_t)gld) + lchunk[i] * 8) * sizeof(T));
   }
   auto dma = [&](const T* p, lds_byte* dst) __attribute__((always_inline)) {
@@ -202,8 +208,8 @@ __global__ void __launch_bounds__(64 * WD * WD) grad_gemm16_kernel(const GradGem
   int oa1[WT], ob1[WT];
 #pragma unroll
   for (int i = 0; i < WT; ++i) {
-    oa1[i] = ro1 + (((ga0 + 2 * i) ^ f1) << 4);
-    ob1[i] = OPB + ro1 + (((gb0 + 2 * i) ^ f1) << 4);
+    oa1[i] = ro1 + (swz(ga0 + 2 * i, f1) << 4);
+    ob1[i] = OPB + ro1 + (swz(gb0 + 2 * i, f1) << 4);
   }
   constexpr int O2 = 16 * TM * 2;
 
@@ -333,10 +339,14 @@ __global__ void __launch_bounds__(256) grad_gemm32_kernel(const GradGemmArgs a) 
   gemm_store_partial<WT>(a, TM, g, n, split, dt, pt, wm, wn, r16, q4, acc, TM / WD);
 }
 
-// side of the square workgroup tile: the largest of 256, 128 (16-bit types only), 64, 32 that divides D
+// side of the square workgroup tile: the largest of 256, 128 (16-bit types only), 64, 32 that divides D; 96 and 160
+// (16-bit types) for the head dims that only much smaller powers of two divide: every pair of tiles of a gate streams
+// both of its operand slabs, so D = 96 as 9 pairs of 32-unit tiles took 1.30 ms at B256 T1024 N8 against 0.40 for D = 64
 static int gemm_tile_side(int dtype, int D) {
   if (dtype != FRNN_F32 && D % 256 == 0) return 256;
   if (dtype != FRNN_F32 && D % 128 == 0) return 128;
+  if (dtype != FRNN_F32 && D % 96 == 0 && D / 96 <= 2) return 96;     // 96, 192
+  if (dtype != FRNN_F32 && D % 160 == 0 && D / 160 <= 3) return 160;  // 160, 320, 480
   return (D % 64 == 0) ? 64 : 32;
 }
 
@@ -380,6 +390,8 @@ static int launch_gemm16_any(int TM, const GradGemmArgs& a, dim3 grid, hipStream
   if (TM == 256) return launch_gemm16<T, 256, 4>(a, grid, st);
   if (TM == 128) return launch_gemm16<T, 128, 2>(a, grid, st);
   if (TM == 64) return launch_gemm16<T, 64, 2>(a, grid, st);
+  if (TM == 96) return launch_gemm16<T, 96, 2>(a, grid, st);
+  if (TM == 160) return launch_gemm16<T, 160, 2>(a, grid, st);
   return launch_gemm16<T, 32, 2>(a, grid, st);
 }
 
