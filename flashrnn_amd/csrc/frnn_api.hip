@@ -118,6 +118,7 @@ bool find_plan(int function, int dtype, int D, int variant, int backward, Plan* 
   return false;
 }
 
+
 static int env_int(const char* name, int dflt) {
   const char* v = getenv(name);
   return (v && *v) ? atoi(v) : dflt;

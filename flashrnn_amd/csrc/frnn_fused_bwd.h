@@ -140,12 +140,14 @@ fused_bwd_kernel(const BwdArgs a) {
   // 16x16x4 form keeps it there too, and up to 320 registers at one wave per SIMD)
   constexpr bool M44 = sizeof(T) == 4 && TR == 4 && KW >= 2 && !RC &&
                        (bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)) == 0 || (WAVES <= 4 && NGH * UTW * KDL <= 320));
-  static_assert(DSP == 1 || M44, "destinations are split between wave pairs in the 4x4x1 form only");
+  constexpr bool DS16 = DSP > 1 && sizeof(T) == 2;  // 16-bit kernels whose wave pairs split the destinations
+  constexpr int NL = DS16 ? KW / DSP : KW;          // destinations whose fragments a wave keeps: hf * NL .. hf * NL + NL - 1
+  static_assert(DSP == 1 || M44 || DS16, "destinations are split between wave pairs in these two forms only");
 
   extern __shared__ __attribute__((aligned(16))) unsigned char smem_raw[];
   T* const gbuf0 = reinterpret_cast<T*>(smem_raw);
   T* const gbuf1 = gbuf0 + 16 * KDL;
-  constexpr int RLD = bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)), KWR = KW - RLD;
+  constexpr int RLD = DS16 ? 0 : bwd_lds_tiles(GR, D, WAVES, UTW, KW, (int)sizeof(T)), KWR = NL - RLD;
   // this lane's fragments of the last RLD destination tiles: [wave][tile][u][ks][lane]
   Frag* const rl = reinterpret_cast<Frag*>(smem_raw + (size_t)2 * 16 * KDL * sizeof(T)) +
                    (size_t)(threadIdx.x >> 6) * RLD * UTW * KS * 64 + (threadIdx.x & 63);
@@ -379,11 +381,11 @@ fused_bwd_kernel(const BwdArgs a) {
 #endif
   }
 #pragma unroll
-  for (int r = 0; r < (M44 ? 0 : KW); ++r) {
-    const int x = (slice + r) % KW;
+  for (int r = 0; r < (M44 ? 0 : NL); ++r) {
+    const int x = (slice + hf * NL + r) % KW;  // (hf = 0 unless wave pairs split the destinations)
 #pragma unroll
     for (int u = 0; u < UTW; ++u) {
-      const T* row = Rt + ((size_t)n * D + (x * UT_WG + w * UTW + u) * 16 + r16) * (GR * D) + slice * DL;
+      const T* row = Rt + ((size_t)n * D + (x * UT_WG + wp * UTW + u) * 16 + r16) * (GR * D) + slice * DL;
 #pragma unroll
       for (int ks = 0; ks < KS; ++ks) {
         const int kk0 = ks * X::KM + q4 * KE;
@@ -784,6 +786,8 @@ fused_bwd_kernel(const BwdArgs a) {
     constexpr bool GROUPED = OWN_LAST && KW - 1 > 8;
     constexpr int RI = 4;
     static_assert(!GROUPED || RLD % RI == 0, "LDS-resident destinations come in whole groups");
+    static_assert(!DS16 || GROUPED, "wave pairs split the destinations of the grouped product only");
+    const int hfo = DS16 ? hf * NL : 0;  // first destination of this wave (uniform)
     float p44[M44 ? NGH : 1][M44 ? UTW : 1][4];  // 4x4x1 form: partial sums of the lane's element, destination 4 (q DSP + hf) + i
     if constexpr (M44) {
       const float* gfl = reinterpret_cast<const float*>(gb) + lane;
@@ -833,8 +837,8 @@ fused_bwd_kernel(const BwdArgs a) {
             IW wv[RI][E];
 #pragma unroll
             for (int rr = 0; rr < RI; ++rr) {
-              const int x = (slice + r0 + rr) % KW;
-              base[rr] = inbox + (size_t)(((x * WAVES + w_u) * UTW + u) * KW + slice) * 256;
+              const int x = (slice + hfo + r0 + rr) % KW;
+              base[rr] = inbox + (size_t)(((x * NPOS + wp_u) * UTW + u) * KW + slice) * 256;
               float part[E];
               own_elems<TR>(ag[rr][u], part);
 #pragma unroll
@@ -847,7 +851,7 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
         for (int rr = 0; rr < RI; ++rr) {
           if (rr >= nr) continue;
-          const int x = (slice + r0 + rr) % KW;
+          const int x = (slice + hfo + r0 + rr) % KW;
 #pragma unroll
           for (int u = 0; u < UTW; ++u) {
             float part[E];
@@ -856,7 +860,7 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
             for (int e = 0; e < E; ++e) wv[e] = part_pack((PT*)0, part[e], t);
             // (the destination's place in the area is uniform and goes into the scalar base; the lane's offset is the same for all)
-            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * WAVES + w_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
+            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * NPOS + wp_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
           }
         }
       };
@@ -970,7 +974,7 @@ fused_bwd_kernel(const BwdArgs a) {
     if constexpr (KW > 1) {
       // send: partial sums of the tiles owned by workgroup (slice + r) % KW, same wave position
       const unsigned sslot = ((unsigned)(rvalid ? (t & 1) : 2) * (unsigned)INW + lane) * (unsigned)sizeof(IW);  // byte offset of the area + lane
-      if constexpr (DSP > 1) {  // this wave's destination groups
+      if constexpr (DSP > 1 && M44) {  // this wave's destination groups (4x4x1 form)
 #pragma unroll
         for (int q = 0; q < NGH; ++q)
 #pragma unroll
@@ -998,7 +1002,7 @@ fused_bwd_kernel(const BwdArgs a) {
 #pragma unroll
           for (int e = 0; e < E; ++e) wv[e] = part_pack((PT*)0, part[e], t);
           // (the destination's place in the area is uniform and goes into the scalar base; the lane's offset is the same for all)
-            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * WAVES + w_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
+            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((x * NPOS + wp_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
         }
       }
       if constexpr (DW_LATE) {
@@ -1018,8 +1022,15 @@ fused_bwd_kernel(const BwdArgs a) {
         for (int u = 0; u < UTW; ++u) {
           float own[E];
           own_elems<TR>(accp[0][0][u], own);
+          if (DS16 && hf != 0) {  // (uniform) the second wave's first destination is no tile of its own: sent like the others
+            IW wv[E];
 #pragma unroll
-          for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
+            for (int e = 0; e < E; ++e) wv[e] = part_pack((PT*)0, own[e], t);
+            ll_store_sel<E, 64 * (int)sizeof(IW)>(inbox + (size_t)(((((slice + hfo) % KW) * NPOS + wp_u) * UTW + u) * KW + slice) * 256, sslot, wv, near_m);
+          } else {
+#pragma unroll
+            for (int e = 0; e < E; ++e) ds[u][e][0] += own[e];
+          }
         }
       }
       // receive: KW-1 partial sums of the own tiles, PSRC sources at a time

@@ -103,7 +103,9 @@ fused_fwd_kernel(const FwdArgs a) {
   // columns of a block = the gates of that unit, A = h (the values of one block broadcast to all 16), one
   // instruction per k: D instructions of 8 cycles per tile and step instead of G_r * D / 4 of 32.
   constexpr bool M44 = fwd_form_4x4x1(GR, D, WAVES, UTW, TR, (int)sizeof(T));  // (the whole operand, D registers per tile, in registers)
-  constexpr int RLK = M44 ? 0 : fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KS - RLK;
+  constexpr bool KS16 = fwd_k_split16(GR, D, WAVES, UTW, TR, (int)sizeof(T));  // 16-bit kernels whose wave pairs split k
+  constexpr int KSW = KS16 ? KS / KSP : KS;  // k-steps of a wave
+  constexpr int RLK = M44 || KS16 ? 0 : fwd_lds_ksteps(GR, D, WAVES, UTW, (int)sizeof(T)), KSR = KSW - RLK;
   // Own slice first: of the h_(t-1) a step multiplies with, the workgroup's own D / KW units are in LDS as soon as
   // its waves have finished step t-1; the k-steps over them run before the wait for the other workgroups' slices
   // (behind one more LDS barrier) and leave the critical path.  Each workgroup keeps R and h rotated along k so
@@ -134,7 +136,7 @@ fused_fwd_kernel(const FwdArgs a) {
   __shared__ __attribute__((aligned(16))) T obuf[PST ? 2 * OB : 1];
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
-  __shared__ f32x4 psum[KSP > 1 ? UT_WG * 64 : 1];  // partial sums of the second wave of a pair: [tile][lane]
+  __shared__ f32x4 psum[KSP > 1 ? UT_WG * (KS16 ? GR : 1) * 64 : 1];  // partial sums of the second wave of a pair: [tile][(gate)][lane]
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -324,9 +326,10 @@ fused_fwd_kernel(const FwdArgs a) {
     for (int g = 0; g < GR; ++g) {
       const T* row = R + ((size_t)(g * N + n) * D + ub[u] + r16) * D;
 #pragma unroll
-      for (int ks = 0; ks < KS; ++ks) {
-        const int kh = OWN_FIRST ? (ks + rot_ks < KS ? ks + rot_ks : ks + rot_ks - KS) : ks;  // k-step of the head
-        const Frag f = load_frag<T>(row, kh, q4);
+      for (int ks = 0; ks < KSW; ++ks) {
+        // k-step of the head (own slice first: rotated; wave pairs that split k: this wave's half)
+        const int kstep = OWN_FIRST ? (ks + rot_ks < KS ? ks + rot_ks : ks + rot_ks - KS) : KS16 ? kh * KSW + ks : ks;
+        const Frag f = load_frag<T>(row, kstep, q4);
         if (ks < KSR) {
           rf[u][g][ks < KSR ? ks : 0] = f;
 #ifndef FRNN_NO_AGPR_PIN
@@ -357,7 +360,7 @@ fused_fwd_kernel(const FwdArgs a) {
       if constexpr (BIAS_C) {
         float v[4];
         unpack4<T>(*reinterpret_cast<const Vec4*>(bias_g + (size_t)(g * N + n) * D + ub[u] + q4 * 4), v);
-        biasc[u][g] = f32x4{v[0], v[1], v[2], v[3]};
+        biasc[u][g] = kh == 0 ? f32x4{v[0], v[1], v[2], v[3]} : f32x4{0.f, 0.f, 0.f, 0.f};  // (once per pair of waves)
       } else {
 #pragma unroll
         for (int e = 0; e < E; ++e) bown[u][g][e] = (float)bias_g[(size_t)(g * N + n) * D + ub[u] + esub + e];
@@ -538,7 +541,9 @@ fused_fwd_kernel(const FwdArgs a) {
       }
     }
     if constexpr (!M44) {
-    const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane + KSO * 64;  // (the own k-steps are done)
+    // (the own k-steps are done; wave pairs that split k: this wave's half of h)
+    const Frag* hf = reinterpret_cast<const Frag*>(hbuf[cur]) + lane + KSO * 64 + (KS16 ? kh * KSW * 64 : 0);
+    constexpr int KS = KSW;  // (k-steps of this wave, in this block)
     constexpr int KC = chunk_of(KS - KSO);
     static_assert((KS - KSO) % KC == 0, "k-steps must split into whole chunks");
     Frag hq[2][KC];
@@ -598,6 +603,19 @@ fused_fwd_kernel(const FwdArgs a) {
 #pragma unroll
         for (int j = 1; j < NACC; ++j) acc[u][g] += accp[j][u][g];
       }
+    if constexpr (KS16) {
+      // the second wave of a pair hands its accumulators over (the buffer is free again before its next write: the
+      // barrier of the next step's exchange wait lies in between)
+#pragma unroll
+      for (int u = 0; u < UTW; ++u)
+#pragma unroll
+        for (int g = 0; g < GR; ++g) { if (kh != 0) psum[((wt * UTW + u) * GR + g) * 64 + lane] = acc[u][g]; }
+      lds_barrier();
+#pragma unroll
+      for (int u = 0; u < UTW; ++u)
+#pragma unroll
+        for (int g = 0; g < GR; ++g) { if (kh == 0) acc[u][g] += psum[((wt * UTW + u) * GR + g) * 64 + lane]; }
+    }
     }  // !M44
 
     if constexpr (WX_LATE) {

@@ -43,11 +43,19 @@ constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
 // Heads from 384 units on: the four waves of a workgroup pair up over two tiles, each wave of a pair keeps R for one half
 // of k (D / 2 registers) and multiplies it with that half of h; the second wave hands its partial sums to the first
 // through LDS, which alone does the gate math of the tile.  D = 16 * (WAVES / 2) * KW for these tilings.
+// The same split for the 16-bit kernels of the 4-gate cells at D = 1024 (16x16x32 form: a tile of R is 512 registers, with
+// the split 256 per wave, nothing of it in LDS, and room for the working sets of the 8- and 16-row tiles): the second
+// wave hands over its G_r accumulators.
 constexpr int fwd_k_split(int GR, int D, int WAVES, int UTW, int TR, int esize) {
+  if (esize == 2) return GR == 4 && D == 1024 && WAVES == 4 && UTW == 1 ? 2 : 1;
   return esize == 4 && TR == 4 && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 ? 2 : 1;
 }
 constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esize) {
   return esize == 4 && TR == 4 && GR >= 3 && WAVES <= 4 && UTW * D / fwd_k_split(GR, D, WAVES, UTW, TR, esize) <= 384;
+}
+// (16-bit kernels whose waves split k: the whole operand in registers)
+constexpr bool fwd_k_split16(int GR, int D, int WAVES, int UTW, int TR, int esize) {
+  return esize == 2 && fwd_k_split(GR, D, WAVES, UTW, TR, esize) > 1;
 }
 // Forward kernel: one more wave per workgroup that fetches Wx for the compute waves.  A vector memory instruction that a
 // compute wave issues behind the exchange wait delays its MFMAs (~70 cycles each on the chain of dependent steps), one
@@ -97,7 +105,10 @@ constexpr bool bwd_producer_stores(int GR, int nc, int D, int WAVES, int UTW, in
 // tile positions, and each wave of a pair keeps R^T (own gate rows x destinations) for every second group of 4
 // destination workgroups (G_r * D / 8 registers instead of G_r * D / 4) and sends those groups' partial sums itself;
 // the first wave of a pair alone owns the pair's elements (gate math, loads, stores, receive).  D = 16 * (WAVES / 2) * KW.
+// The same for the 16-bit kernels of the 4-gate cells at D = 1024 (16x16x32 form, every tile height): each wave of a
+// pair keeps the fragments of one half of the 32 destination workgroups, 256 registers, none of them in LDS.
 constexpr int bwd_dest_split(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
+  if (esize == 2) return !rc && GR == 4 && D == 1024 && WAVES == 4 && UTW == 1 && KW == 32 ? 2 : 1;
   return esize == 4 && TR == 4 && !rc && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 && KW >= 8 ? 2 : 1;
 }
 // Backward kernel: LDS bytes of the two dWx hand-over buffers of the producer-store instantiations
@@ -111,7 +122,7 @@ constexpr int bwd_producer_store_bytes(int gw, bool gru, int D, int TR, int esiz
 // (with the two-part product they spill).  The host reads this for the delay of the first probe.
 constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize) {
   const int KM = esize == 4 ? 4 : 32, KS = D / KM;
-  return KW > 1 && KW <= 16 && !fwd_form_4x4x1(GR, D, WAVES, UTW, TR, esize) &&
+  return KW > 1 && KW <= 16 && !fwd_form_4x4x1(GR, D, WAVES, UTW, TR, esize) && !fwd_k_split16(GR, D, WAVES, UTW, TR, esize) &&
          (fwd_lds_ksteps(GR, D, WAVES, UTW, esize) == 0 || KW <= 12) && (D / KW) % KM == 0 &&
          !(esize == 4 && UTW * GR * KS >= 256 && TR >= (KW > 8 ? 8 : 16));
 }
@@ -122,23 +133,26 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
 // with several tiles each; when it does not fit, 4 waves with one tile each and more workgroups
 // beat fewer, fuller workgroups (the step is a dependency chain, not a throughput problem).
 // ---- 4 recurrent gate rows per unit (lstm, slstm) --------------------------------------------
+// (D = 1024, forward and backward: workgroups of two wave pairs, see fwd_k_split / bwd_dest_split; the reverse kernels
+// stop at 8-row tiles: at 16 rows the sLSTM's, with four states, and the fp16 LSTM's spill, and the bf16 LSTM's, which
+// does not, takes twice as long per launch as at 8 rows: LSTM bf16 B256 T512 12.5 against 12.8 ms)
 #define FRNN_PLANS_GR4_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 12, 1, 1, 4) \
-  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 32, 16)
 #define FRNN_BWD_PLANS_GR4_BF16(X) \
   X(160, 2, 2, 1, 5, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 4) X(192, 0, 4, 1, 3, 16) \
-  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 32, 8)
 // slstm backward: as above, but D = 160 as 5 workgroups of 2 waves (10 waves of 168 registers each spill at every tile height)
 #define FRNN_BWD_PLANS_SLSTM_BF16(X) \
   X(128, 2, 4, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 8) X(128, 0, 8, 1, 1, 8) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) \
-  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 32, 8)
 // slstm: its heavier gate math tips D = 192 forward to 3 workgroups of 4 waves (1.19 against 1.26 ms)
 #define FRNN_PLANS_SLSTM_BF16(X) \
   X(160, 2, 2, 1, 5, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 4, 1, 3, 16) \
-  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 2, 1, 32, 4)
+  X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 32, 16)
 // fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave (D in the 4x4x1 form of the 4-row tiles), so
 // D = 512 is as far as the fused kernels go; larger heads run on the alternating backend.  Forward, D = 384 .. 512:
 // workgroups of two wave pairs, 4-row tiles only (see fwd_k_split; D = 16 * (WAVES / 2) * KW)

@@ -24,7 +24,10 @@ int fused_bwd_launch<FRNN_F, FRNN_DT>(const Plan& p, const BwdArgs& a, hipStream
   // (one more wave and its hand-over buffers where the kernel has a producer wave: the same predicate as in the kernel)
   const bool pw = bwd_producer_wave(Cell<FRNN_F>::GR, Cell<FRNN_F>::NC, p.D, p.waves, p.utw, p.kw, a.tile_rows, (int)sizeof(FRNN_TU_T), rc);
   const bool pst = a.pst && !a.cut && bwd_producer_stores(Cell<FRNN_F>::GR, Cell<FRNN_F>::NC, p.D, p.waves, p.utw, p.kw, a.tile_rows, (int)sizeof(FRNN_TU_T), rc);  // (the truncated scan has no barrier per step to hand over at)
-  const size_t lds = bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T), rc) + 16 +
+  // (wave pairs that split the destinations keep every fragment in registers: the two dg buffers only)
+  const bool ds16 = sizeof(FRNN_TU_T) == 2 && bwd_dest_split(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, a.tile_rows, (int)sizeof(FRNN_TU_T), rc) > 1;
+  const size_t lds = (ds16 ? (size_t)2 * 16 * Cell<FRNN_F>::GR * (p.D / p.kw) * sizeof(FRNN_TU_T)
+                           : bwd_lds_bytes(Cell<FRNN_F>::GR, p.D, p.waves, p.utw, p.kw, (int)sizeof(FRNN_TU_T), rc)) + 16 +
                      (pw ? bwd_producer_bytes(Cell<FRNN_F>::NC + (cache_carried_state(FRNN_F, (int)sizeof(FRNN_TU_T), p.D) >= 0 ? 1 : 0), Cell<FRNN_F>::S, p.waves * p.utw, a.tile_rows, (int)sizeof(FRNN_TU_T)) : 0) +
                      (pst ? bwd_producer_store_bytes(Cell<FRNN_F>::GW, FRNN_F == FRNN_GRU, p.D, a.tile_rows, (int)sizeof(FRNN_TU_T)) : 0);
 #define FRNN_CASE_(RCV, Dv, VAR, W, U, K, MTR)                                                          \

@@ -21,7 +21,8 @@ def _device_inputs(gpu, function, B, T, N, D, dtype, seed):
 CASES = [(f, B, N, D, "bfloat16") for f in ("lstm", "slstm", "gru", "elman") for (B, N, D) in ((8, 2, 64), (3, 2, 192), (8, 3, 256))]
 CASES += [("lstm", 5, 2, 64, "float32"), ("gru", 4, 1, 256, "float16"), ("slstm", 4, 1, 128, "float32"),
           ("elman", 6, 1, 512, "bfloat16"), ("lstm", 1, 12, 32, "bfloat16"),
-          ("lstm", 5, 1, 448, "float32"), ("gru", 4, 1, 512, "float32")]  # (fp32 from D = 384: waves in pairs, each with half of k)
+          ("lstm", 5, 1, 448, "float32"), ("gru", 4, 1, 512, "float32"),  # (fp32 from D = 384: waves in pairs, each with half of k)
+          ("lstm", 3, 1, 1024, "bfloat16")]                               # (the same in the 16-bit kernels at D = 1024)
 
 
 @pytest.mark.parametrize("function,B,N,D,dtype", CASES)

@@ -47,7 +47,7 @@ FUSED_SMALL = [
     ("lstm", 17, 4, 1, 768, "float16"),
     ("elman", 11, 6, 1, 768, "bfloat16"),
     ("gru", 7, 5, 1, 1024, "bfloat16"),      # 16 workgroups per head
-    ("lstm", 6, 7, 1, 1024, "bfloat16"),     # 32 workgroups of 2 waves per head; part of R in LDS
+    ("lstm", 6, 7, 1, 1024, "bfloat16"),     # 32 workgroups of two wave pairs per head (k / the destinations split over a pair)
     ("slstm", 5, 5, 1, 1024, "bfloat16"),
     ("lstm", 18, 4, 1, 1024, "float16"),
     ("lstm", 6, 5, 2, 160, "bfloat16"),      # 10 waves
@@ -127,6 +127,8 @@ TILINGS = [
     ("slstm", 6, 8, 2, 192, "bfloat16"),
     ("elman", 18, 5, 1, 1024, "bfloat16"),
     ("elman", 3, 6, 2, 32, "float32"),
+    ("lstm", 37, 5, 1, 1024, "bfloat16"),    # wave pairs, at every tile height they are compiled for (reverse: up to 8 rows)
+    ("slstm", 21, 4, 1, 1024, "float16"),
 ]
 
 
