@@ -222,7 +222,7 @@ int frnn_alt_backward_opt(int function, int dtype, int B, int T, int N, int D,
  * stored states.  Results equal those of the cached path up to the rounding of the stored states (lstm, gru:
  * the same bits in fp32 storage; slstm: its stabilised gates are rebuilt from the stored, rounded m).
  * Available where R and R^T fit the registers together (frnn_fused_recompute_supported; bf16 / fp16: D = 32, 64,
- * 96, 128, 192, 256; fp32: 32, 64), else FRNN_E_UNSUPPORTED.  For FRNN_ELMAN, which caches nothing, the flag
+ * 96, 128, 192, 256, 320, and 384 for the gru; fp32: 32, 64), else FRNN_E_UNSUPPORTED.  For FRNN_ELMAN, which caches nothing, the flag
  * changes nothing.  The workspace size depends on the mode: frnn_fused_workspace_bytes_opt. */
 int frnn_fused_recompute_supported(int function, int dtype, int B, int N, int D);
 size_t frnn_fused_workspace_bytes_opt(int function, int dtype, int B, int T, int N, int D, int backward,
