@@ -138,6 +138,9 @@ static bool near_stores_allowed() { return env_int("FRNN_AGENT_STORES", 0) == 0;
 //   lstm, slstm D=768 (12 workgroups) 0-1;  the others: lstm D=1024 (32 workgroups of 2 waves) 3-6.
 static int fwd_poll_delay_default(int function, int dtype, const Plan& p, int tile_rows) {
   if (p.kw <= 1) return 0;
+  // groups that span the device exchange through memory, at agent scope: a round trip takes several times as long as
+  // one to the L2 of an XCD (lstm fp32 D=1024, forward, 1024 steps: delay 0 6.09 ms, 8 4.81, 16 4.37, 24 3.92, 32 4.00, 48 4.36)
+  if (p.kw > kXcdWorkgroups) return 24;
   const bool elman = function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP;
   // kernels that multiply the workgroup's own slice in front of the wait: little is left to sleep through
   if (fwd_own_slice_first(cell_dims(function).GR, p.D, p.waves, p.utw, p.kw, tile_rows, dtype == FRNN_F32 ? 4 : 2)) {
@@ -171,7 +174,10 @@ static int device_cus() {
 // for each other, so all of them must be resident, and a group is pinned to one XCD (decode_block): what
 // counts is the room of an XCD (an eighth of the compute units, one such workgroup per compute unit), not
 // of the device: with KW = 12 an XCD of 32 compute units holds 2 groups, the device 16, not 256 / 12 = 21.
-static int groups_per_launch(int kw) { return 8 * ((device_cus() / 8) / kw); }
+// Heads of more than 32 workgroups (kXcdWorkgroups) spread over the whole device: what counts is the device.
+static int groups_per_launch(int kw) { return kw > kXcdWorkgroups ? device_cus() / kw : 8 * ((device_cus() / 8) / kw); }
+// (such groups never share an XCD: no handshake, every exchange store at agent scope)
+static bool near_stores_possible(const Plan& p) { return p.kw > 1 && p.kw <= kXcdWorkgroups; }
 
 // The tiling of a call: the table's default for the head dim, or its small-batch alternative (variant 2) while all
 // groups of the call fit one launch with 4-row tiles.  FRNN_FUSED_VARIANT picks a variant by hand.
@@ -637,12 +643,12 @@ static int fused_forward_impl(int function, int dtype, int training, int B, int 
   int per_launch = groups;
   if (p.kw > 1) {  // workgroups that wait for each other must all be resident
     per_launch = groups_per_launch(p.kw);
-    if (per_launch < 1) return fail(FRNN_E_DEVICE, "an eighth of the device has fewer compute units than the %d workgroups of one head", p.kw);
+    if (per_launch < 1) return fail(FRNN_E_DEVICE, "the device has too few compute units for the %d workgroups of one head", p.kw);
   }
   FwdArgs a;
   a.Wx = Wx; a.R = R; a.b = b; a.s0 = s0; a.states = states; a.cache = cache;
   a.ll = w.ll; a.status = w.status;
-  a.xcd = (p.kw > 1 && !step && near_stores_allowed()) ? w.xcd : nullptr;
+  a.xcd = (near_stores_possible(p) && !step && near_stores_allowed()) ? w.xcd : nullptr;
   a.carry = carry; a.step = step;
   a.B = B; a.BS = o.bs ? o.bs : B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.training = need_cache ? 1 : 0;
@@ -761,14 +767,14 @@ static int fused_backward_impl(int function, int dtype, int B, int T, int N, int
   int per_launch = groups;
   if (p.kw > 1) {
     per_launch = groups_per_launch(p.kw);
-    if (per_launch < 1) return fail(FRNN_E_DEVICE, "an eighth of the device has fewer compute units than the %d workgroups of one head", p.kw);
+    if (per_launch < 1) return fail(FRNN_E_DEVICE, "the device has too few compute units for the %d workgroups of one head", p.kw);
   }
   BwdArgs a;
   a.Rt = w.Rt; a.s0 = s0; a.states = states; a.cache = o.rc ? nullptr : cache; a.dstates = dstates;
   a.Wx = Wx; a.R = R; a.b = b;
   a.dWx = dWx; a.dgx = w.dgx; a.ds0 = ds0; a.dbp = w.dbp;
   a.ll = w.ll; a.status = w.status;
-  a.xcd = (p.kw > 1 && near_stores_allowed()) ? w.xcd : nullptr;
+  a.xcd = (near_stores_possible(p) && near_stores_allowed()) ? w.xcd : nullptr;
   a.B = B; a.BS = o.bs ? o.bs : B; a.T = T; a.N = N; a.groups_total = groups; a.tile_rows = tr;
   a.spin_limit = env_int("FRNN_SPIN_LIMIT", 1 << 22);
   p.cooperative = env_int("FRNN_COOPERATIVE", 0);
@@ -928,7 +934,7 @@ int frnn_fused_decode_open(int function, int dtype, int B, int N, int D,
   FwdArgs a;
   a.Wx = nullptr; a.R = R; a.b = b; a.s0 = s_in; a.states = nullptr; a.cache = nullptr;
   a.ll = (u64*)(mb + dp.l.exch_off); a.status = (int*)mb + MB_STATUS;
-  a.xcd = (p.kw > 1 && near_stores_allowed()) ? (int*)(mb + dp.l.xcd_off) : nullptr;
+  a.xcd = (near_stores_possible(p) && near_stores_allowed()) ? (int*)(mb + dp.l.xcd_off) : nullptr;
   a.carry = carry; a.step = 0;
   a.B = B; a.BS = B; a.T = max_tokens; a.N = N; a.grp0 = 0; a.groups = dp.groups; a.groups_total = dp.groups; a.tile_rows = 4;
   a.training = 0;

@@ -481,12 +481,20 @@ enum { STATUS_OK = 0, STATUS_WAIT_EXPIRED = 1 };
 // Workgroup -> (group, slice) mapping.  Workgroups are dispatched round-robin over the 8
 // XCDs, so the KW workgroups of one (head, batch-tile) group take ids that are congruent
 // mod 8 and share one XCD's L2.  grid = 8 * KW * ceil(groups / 8).
+// Groups of more than 32 workgroups (fp32 gated cells beyond 512 units: one workgroup per compute unit, and an XCD has
+// 32) spread over the whole device instead, consecutive ids, and exchange at agent scope.  grid = KW * groups.
+constexpr int kXcdWorkgroups = 32;
 __device__ __forceinline__ bool decode_block(int groups, int KW, int& grp, int& slice) {
+  if (KW > kXcdWorkgroups) {
+    grp = blockIdx.x / KW;
+    slice = blockIdx.x % KW;
+    return grp < groups;
+  }
   const int xcd = blockIdx.x & 7, q = blockIdx.x >> 3;
   grp = (q / KW) * 8 + xcd;
   slice = q % KW;
   return grp < groups;
 }
-inline int grid_for(int groups, int KW) { return 8 * KW * ((groups + 7) / 8); }
+inline int grid_for(int groups, int KW) { return KW > kXcdWorkgroups ? KW * groups : 8 * KW * ((groups + 7) / 8); }
 
 }  // namespace frnn

@@ -126,6 +126,14 @@ fused_bwd_kernel(const BwdArgs a) {
   constexpr int ROUNDS = KW == 1 ? 1 : (KW - 1 + RC_MAX - 1) / RC_MAX;
   constexpr int PSRC = KW == 1 ? 1 : (KW - 1 + ROUNDS - 1) / ROUNDS;  // sources polled per round
   constexpr size_t INW = bwd_inbox_words(D, KW);
+  // Waves that split the destinations of a tile position (DSP > 1) also split its sources where one wave would poll them
+  // in several rounds, each a trip to memory and back: wave hf polls sources 1 + hf * SRC_W .. and hands its sum to the
+  // first wave through LDS.  Measured, reverse kernel, 1024 steps: LSTM fp32 D = 1024 (63 sources at agent scope, 4 rounds of
+  // 16 become one per wave) 8.68 -> 6.30 ms, bf16 D = 1024 B16 2.67 -> 2.39; also from 13 sources on, where one round
+  // shrinks to half the words: fp32 D = 512 2.62 -> 2.52, D = 448 2.61 -> 2.55 (D = 384, 11 sources: 2.49 -> 2.54, left alone).
+  constexpr bool RSP = DSP > 1 && (ROUNDS > 1 || KW >= 14);
+  constexpr int SRC_W = RSP ? (KW - 1 + DSP - 1) / DSP : 1;                    // sources per wave
+  constexpr int ROUNDS_W = (SRC_W + RC_MAX - 1) / RC_MAX, PSRC_W = (SRC_W + ROUNDS_W - 1) / ROUNDS_W;
   constexpr int E = O::E, ND_ = NDW<T, E>::value;
   constexpr bool SB = NDW<T, E>::SUB;  // single bf16 elements: 16-bit memory operations
   constexpr unsigned ES = sizeof(T);
@@ -160,6 +168,7 @@ fused_bwd_kernel(const BwdArgs a) {
   // load in flight (measured: the operand prefetch's full HBM latency, once per step)
   __shared__ int dead_flag_word, near_word;
   int* const dead_flag = &dead_flag_word;
+  __shared__ float rsum[RSP ? NPOS * (DSP - 1) * UTW * O::E * 64 : 1];  // sums of the sources polled by the other waves: [position][wave - 1][tile][element][lane]
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -1035,7 +1044,59 @@ fused_bwd_kernel(const BwdArgs a) {
       }
       // receive: KW-1 partial sums of the own tiles, PSRC sources at a time
       const IW* const mine = inbox + (size_t)(t & 1) * INW + ((size_t)(slice * NPOS + wp) * UTW) * KW * 256 + lane;
-      if (DSP == 1 || hf == 0) {
+      if constexpr (RSP) {
+        const int rbeg = 1 + hf * SRC_W;  // (uniform) this wave's sources: rbeg .. rbeg + SRC_W - 1, below KW
+        float rs[UTW][E];
+#pragma unroll
+        for (int u = 0; u < UTW; ++u)
+#pragma unroll
+          for (int e = 0; e < E; ++e) rs[u][e] = 0.f;
+#pragma unroll
+        for (int k0 = 0; k0 < SRC_W; k0 += PSRC_W) {
+          constexpr int NWR = PSRC_W * UTW * E;
+          int off[NWR]; bool need[NWR]; IW v[NWR];
+#pragma unroll
+          for (int rr = 0; rr < PSRC_W; ++rr) {
+            const bool in = k0 + rr < SRC_W && rbeg + k0 + rr < KW;
+            const int src = (slice + (in ? rbeg + k0 + rr : 1)) % KW;
+#pragma unroll
+            for (int u = 0; u < UTW; ++u)
+#pragma unroll
+              for (int e = 0; e < E; ++e) {
+                off[(rr * UTW + u) * E + e] = (u * KW + src) * 256 + e * 64;
+                need[(rr * UTW + u) * E + e] = rvalid && in;
+              }
+          }
+          if (!fail) fail = poll_words_staggered<PT, NWR>(mine, off, need, t, v, a.status, a.spin_limit, k0 == 0 ? a.poll_delay : 0);
+#pragma unroll
+          for (int rr = 0; rr < PSRC_W; ++rr) {
+            const bool in = k0 + rr < SRC_W && rbeg + k0 + rr < KW;
+#pragma unroll
+            for (int u = 0; u < UTW; ++u)
+#pragma unroll
+              for (int e = 0; e < E; ++e) rs[u][e] += in ? part_value((PT*)0, v[(rr * UTW + u) * E + e]) : 0.f;
+          }
+        }
+        // (the buffer is free again before the next write: the barrier of the next step lies in between)
+        if (hf != 0) {
+#pragma unroll
+          for (int u = 0; u < UTW; ++u)
+#pragma unroll
+            for (int e = 0; e < E; ++e) rsum[(((wp_u * (DSP - 1) + hf - 1) * UTW + u) * E + e) * 64 + lane] = rs[u][e];
+        }
+        lds_barrier();
+        if (hf == 0) {
+#pragma unroll
+          for (int u = 0; u < UTW; ++u)
+#pragma unroll
+            for (int e = 0; e < E; ++e) {
+              float sum = rs[u][e];
+#pragma unroll
+              for (int i = 0; i < DSP - 1; ++i) sum += rsum[(((wp_u * (DSP - 1) + i) * UTW + u) * E + e) * 64 + lane];
+              ds[u][e][0] += sum;
+            }
+        }
+      } else if (DSP == 1 || hf == 0) {
 #pragma unroll
       for (int r0 = 1; r0 < KW; r0 += PSRC) {
         constexpr int NWR = PSRC * UTW * E;

@@ -78,10 +78,11 @@ fused_fwd_kernel(const FwdArgs a) {
   typedef typename X::Frag Frag;
   typedef Own<TR> O;
   constexpr int GR = C::GR, GW = C::GW, GT = C::GT, S = C::S, NC = C::NC;
-  // (KSP = 2: the fp32 4x4x1 form of heads from 384 units on, two waves per tile, each with one half of k)
+  // (KSP = 2: the fp32 4x4x1 form of heads from 384 units on, two waves per tile, each with one half of k; 4 beyond 512 units)
   constexpr int KSP = fwd_k_split(GR, D, WAVES, UTW, TR, (int)sizeof(T)), DK = D / KSP;
   constexpr int KS = D / X::KM, NT = WAVES * 64, UT_WG = WAVES * UTW / KSP;
   static_assert(UT_WG * KW * 16 == D, "tiling must cover the head");
+  static_assert(KSP <= 2 || (sizeof(T) == 4 && UTW == 1), "more than two waves per tile: the fp32 4x4x1 form only");
   constexpr int LLW = 16 * D / X::EPW;  // 64-bit words per exchange slot
   // words a thread polls per step: the TR rows of the tile, without the workgroup's own slice
   // (polled 16 at a time: longer lists are padded to whole rounds with entries that wait for nothing)
@@ -136,7 +137,7 @@ fused_fwd_kernel(const FwdArgs a) {
   __shared__ __attribute__((aligned(16))) T obuf[PST ? 2 * OB : 1];
   // [wave][k-step][u][g][lane]: each lane reads back what it wrote
   __shared__ __attribute__((aligned(16))) Frag rlds[RLK > 0 ? WAVES * RLK * UTW * GR * 64 : 1];
-  __shared__ f32x4 psum[KSP > 1 ? UT_WG * (KS16 ? GR : 1) * 64 : 1];  // partial sums of the second wave of a pair: [tile][(gate)][lane]
+  __shared__ f32x4 psum[KSP > 1 ? UT_WG * (KS16 ? GR : KSP - 1) * 64 : 1];  // partial sums of the other waves of a tile: [tile][(gate | wave)][lane]
 
   int grp_l, slice;
   if (!decode_block(a.groups, KW, grp_l, slice)) return;
@@ -526,14 +527,19 @@ fused_fwd_kernel(const FwdArgs a) {
 #pragma unroll
       for (int u = 0; u < UTW; ++u) {
         sum[u] = (ac[u][0] + ac[u][1]) + (ac[u][2] + ac[u][3]);
-        if constexpr (KSP > 1) { if (kh != 0) psum[(wt * UTW + u) * 64 + lane] = sum[u]; }
+        if constexpr (KSP > 1) { if (kh != 0) psum[((wt * UTW + u) * (KSP - 1) + kh - 1) * 64 + lane] = sum[u]; }
       }
       // (the buffer is free again before the second wave's next write: the barrier of the next step's exchange wait,
       // which every pair-split tiling has, lies in between)
       if constexpr (KSP > 1) lds_barrier();
 #pragma unroll
       for (int u = 0; u < UTW; ++u) {
-        if constexpr (KSP > 1) { if (kh == 0) sum[u] += psum[(wt * UTW + u) * 64 + lane]; }
+        if constexpr (KSP > 1) {
+          if (kh == 0) {
+#pragma unroll
+            for (int i = 0; i < KSP - 1; ++i) sum[u] += psum[((wt * UTW + u) * (KSP - 1) + i) * 64 + lane];
+          }
+        }
         // lane 4*blk + j holds (gate j, unit blk) of batch rows 0..3; after the transpose lane 4*blk + b holds
         // gates 0..3 of (batch row b, unit blk): the element that Own<4> gives this lane
         ry44[u][0] = sum[u][0]; ry44[u][1] = sum[u][1]; ry44[u][2] = sum[u][2]; ry44[u][3] = sum[u][3];

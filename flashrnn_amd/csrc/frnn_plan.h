@@ -46,9 +46,12 @@ constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
 // The same split for the 16-bit kernels of the 4-gate cells at D = 1024 (16x16x32 form: a tile of R is 512 registers, with
 // the split 256 per wave, nothing of it in LDS, and room for the working sets of the 8- and 16-row tiles): the second
 // wave hands over its G_r accumulators.
+// fp32 heads beyond 512 units: all four waves share one tile, a quarter of k each (D / 4 registers), and three of them hand
+// their sums over; D = 16 * KW (compiled for D = 1024: 64 workgroups per head), more than the 32 compute units of an XCD: such a group
+// spreads over the device (decode_block) and exchanges at agent scope.
 constexpr int fwd_k_split(int GR, int D, int WAVES, int UTW, int TR, int esize) {
   if (esize == 2) return GR == 4 && D == 1024 && WAVES == 4 && UTW == 1 ? 2 : 1;
-  return esize == 4 && TR == 4 && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 ? 2 : 1;
+  return esize == 4 && TR == 4 && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 ? (D > 512 ? 4 : 2) : 1;
 }
 constexpr bool fwd_form_4x4x1(int GR, int D, int WAVES, int UTW, int TR, int esize) {
   return esize == 4 && TR == 4 && GR >= 3 && WAVES <= 4 && UTW * D / fwd_k_split(GR, D, WAVES, UTW, TR, esize) <= 384;
@@ -107,9 +110,10 @@ constexpr bool bwd_producer_stores(int GR, int nc, int D, int WAVES, int UTW, in
 // the first wave of a pair alone owns the pair's elements (gate math, loads, stores, receive).  D = 16 * (WAVES / 2) * KW.
 // The same for the 16-bit kernels of the 4-gate cells at D = 1024 (16x16x32 form, every tile height): each wave of a
 // pair keeps the fragments of one half of the 32 destination workgroups, 256 registers, none of them in LDS.
+// fp32 heads beyond 512 units: one tile position, every fourth group of 4 destinations per wave (G_r * D / 16 registers).
 constexpr int bwd_dest_split(int GR, int D, int WAVES, int UTW, int KW, int TR, int esize, bool rc) {
   if (esize == 2) return !rc && GR == 4 && D == 1024 && WAVES == 4 && UTW == 1 && KW == 32 ? 2 : 1;
-  return esize == 4 && TR == 4 && !rc && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 && KW >= 8 ? 2 : 1;
+  return esize == 4 && TR == 4 && !rc && GR >= 3 && WAVES == 4 && UTW == 1 && D >= 384 && KW >= 8 ? (D > 512 ? 4 : 2) : 1;
 }
 // Backward kernel: LDS bytes of the two dWx hand-over buffers of the producer-store instantiations
 // ([gate][row][unit], and [row][unit] for the GRU's g-gate cotangent), behind the operand hand-over buffers
@@ -153,23 +157,28 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
   X(160, 2, 2, 1, 5, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 8) X(192, 0, 4, 1, 3, 16) \
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 32, 16)
-// fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave (D in the 4x4x1 form of the 4-row tiles), so
-// D = 512 is as far as the fused kernels go; larger heads run on the alternating backend.  Forward, D = 384 .. 512:
-// workgroups of two wave pairs, 4-row tiles only (see fwd_k_split; D = 16 * (WAVES / 2) * KW)
+// fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave (D in the 4x4x1 form of the 4-row tiles).
+// Forward, D = 384 .. 512: workgroups of two wave pairs, 4-row tiles only (see fwd_k_split; D = 16 * (WAVES / 2) * KW);
+// D = 1024: one tile per workgroup, k split over its four waves, groups that span the device (D = 16 * KW; the reverse
+// kernels of the 4-gate cells at D = 640 and 768 in that form spill, so those head dims stay with the alternating backend)
 #define FRNN_PLANS_GR4_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
-  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
-// (backward, D = 384 .. 512: workgroups of two wave pairs, 4-row tiles only; see bwd_dest_split)
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
+  X(1024, 0, 4, 1, 64, 4)
+// (backward, D = 384 .. 512: workgroups of two wave pairs, D = 1024: one tile position per workgroup, 4-row tiles
+// only; see bwd_dest_split)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
   X(320, 2, 1, 1, 20, 4) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
-  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
+  X(1024, 0, 4, 1, 64, 4)
 // slstm fp32 backward: the same without the 20-workgroup tiling of D = 320 (with four states its kernel spills)
 #define FRNN_BWD_PLANS_SLSTM_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
-  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
+  X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
+  X(1024, 0, 4, 1, 64, 4)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
@@ -180,11 +189,13 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 16, 16)
 #define FRNN_PLANS_GR3_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
-  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
+  X(1024, 0, 4, 1, 64, 4)
 #define FRNN_BWD_PLANS_GR3_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
-  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4)
+  X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
+  X(1024, 0, 4, 1, 64, 4)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \

@@ -56,12 +56,14 @@ def test_supported_table(lib):
     assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0 and lib.frnn_fused_supported(G, 0, 32, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 2048) == _lib.E_UNSUPPORTED  # too large to keep on chip
-    # fp32: R is twice the size, so the gated cells stop at D = 512 (the reference's test grid, tests/test_lstm.py:9-46,
-    # runs fp32 up to there and at 1024, which is left to the alternating backend), the elman cell at 1024
+    # fp32: R is twice the size: the gated cells run up to D = 512 and at D = 1024 (the head dims of the reference's test
+    # grid, tests/test_lstm.py:9-46; at 1024 a head takes 64 workgroups, spread over the device), the elman cell at 1024
     for f in (L, S, G, E):
         for D in (32, 64, 96, 128, 160, 192, 256, 320, 384, 448, 512):
             assert lib.frnn_fused_supported(f, 1, 8, 1, D) == 0, (f, D)
     assert lib.frnn_fused_supported(L, 1, 8, 1, 640) == _lib.E_UNSUPPORTED
+    for f in (L, S, G):
+        assert lib.frnn_fused_supported(f, 1, 8, 2, 1024) == 0, f
     assert lib.frnn_fused_supported(E, 1, 8, 1, 768) == 0 and lib.frnn_fused_supported(E, 1, 8, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 48) == _lib.E_UNSUPPORTED
     assert b"head dim" in lib.frnn_last_error()

@@ -14,7 +14,7 @@ pytestmark = pytest.mark.gpu
 KDT = {"bfloat16": torch.bfloat16, "float32": torch.float32}
 # (the fp32 case and bf16 D = 1024: the kernels whose waves work in pairs, 14 and 32 workgroups per head, where the second
 # wave of a pair takes part in every barrier of the first and must leave the time loop with it)
-SHAPES = [("bfloat16", 256), ("float32", 448), ("bfloat16", 1024)]
+SHAPES = [("bfloat16", 256), ("float32", 448), ("bfloat16", 1024), ("float32", 1024)]
 
 
 def _forward(gpu, inp, grad, dtype="bfloat16"):

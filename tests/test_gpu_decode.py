@@ -22,6 +22,7 @@ CASES = [(f, B, N, D, "bfloat16") for f in ("lstm", "slstm", "gru", "elman") for
 CASES += [("lstm", 5, 2, 64, "float32"), ("gru", 4, 1, 256, "float16"), ("slstm", 4, 1, 128, "float32"),
           ("elman", 6, 1, 512, "bfloat16"), ("lstm", 1, 12, 32, "bfloat16"),
           ("lstm", 5, 1, 448, "float32"), ("gru", 4, 1, 512, "float32"),  # (fp32 from D = 384: waves in pairs, each with half of k)
+          ("lstm", 6, 1, 1024, "float32"),  # (64 workgroups per head, spread over the device)
           ("lstm", 3, 1, 1024, "bfloat16")]                               # (the same in the 16-bit kernels at D = 1024)
 
 

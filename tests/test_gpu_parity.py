@@ -81,6 +81,10 @@ FUSED_SMALL = [
     ("gru", 9, 4, 1, 512, "float32"),
     ("elman", 7, 5, 1, 768, "float32"),
     ("elman", 10, 4, 1, 1024, "float32"),
+    ("lstm", 6, 5, 1, 1024, "float32"),      # 64 workgroups per head, spread over the device; 4 waves split k / the destinations
+    ("slstm", 9, 4, 1, 1024, "float32"),     # 3 groups, the last with one valid row
+    ("gru", 17, 3, 1, 1024, "float32"),      # 5 groups: two launches
+    ("lstm", 3, 4, 2, 1024, "float32"),
     ("lstm", 37, 4, 1, 512, "float32"),      # 10 groups of 4 rows, the last with one valid row
     ("gru", 70, 4, 1, 384, "float32"),       # 18 groups of 12 workgroups: two launches
     # elman fp32 from D = 128 on: D / 64 workgroups of one tile per wave

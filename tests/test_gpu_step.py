@@ -20,6 +20,7 @@ CASES = [
     ("elman", 32, 1, 1024, "bfloat16", "hip_fused"),
     ("lstm", 1, 12, 64, "bfloat16", "hip_fused"),
     ("slstm", 6, 1, 448, "float32", "hip_fused"),    # fp32 from D = 384: pairs of waves, each with half of k
+    ("gru", 5, 1, 1024, "float32", "hip_fused"),     # fp32 D = 1024: four waves per tile, a quarter of k each
     ("lstm", 8, 3, 256, "bfloat16", "hip"),
     ("gru", 5, 2, 96, "float32", "hip"),
     ("slstm", 4, 2, 64, "bfloat16", "hip"),
