@@ -140,7 +140,8 @@ def run_gpu(w, backend, steps, warmup, device, recompute=False):
     for i in range(held):
         per_kernel.setdefault(lib.frnn_profile_name(i).decode(), []).append(lib.frnn_profile_ms(i))
     lib.frnn_profile_enable(0)
-    calls = max(1, min(steps, held // entries_per_step))
+    # (steps that the ring of launches holds: a fraction when a step has more entries than fit a whole number of times)
+    calls = max(1.0, min(float(steps), held / entries_per_step))
     kern = {k: (sum(v) / len(v), max(1, round(len(v) / calls))) for k, v in per_kernel.items()}
     return (t1 - t0) * 1e3 / steps, kern
 

@@ -47,7 +47,7 @@ constexpr int fwd_lds_ksteps(int GR, int D, int WAVES, int UTW, int esize) {
 // the split 256 per wave, nothing of it in LDS, and room for the working sets of the 8- and 16-row tiles): the second
 // wave hands over its G_r accumulators.
 // fp32 heads beyond 512 units: all four waves share one tile, a quarter of k each (D / 4 registers), and three of them hand
-// their sums over; D = 16 * KW (compiled for D = 1024: 64 workgroups per head), more than the 32 compute units of an XCD: such a group
+// their sums over; D = 16 * KW (D = 640, 768, 1024: 40, 48, 64 workgroups per head), more than the 32 compute units of an XCD: such a group
 // spreads over the device (decode_block) and exchanges at agent scope.
 constexpr int fwd_k_split(int GR, int D, int WAVES, int UTW, int TR, int esize) {
   if (esize == 2) return GR == 4 && D == 1024 && WAVES == 4 && UTW == 1 ? 2 : 1;
@@ -159,26 +159,25 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
   X(256, 0, 4, 1, 4, 16) X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 6, 16) X(448, 0, 4, 1, 7, 16) X(512, 0, 4, 1, 8, 16) X(640, 0, 4, 1, 10, 16) X(768, 0, 4, 1, 12, 8) X(1024, 0, 4, 1, 32, 16)
 // fp32: a 16-unit tile of a gated cell takes G_r * D / 4 registers of a wave (D in the 4x4x1 form of the 4-row tiles).
 // Forward, D = 384 .. 512: workgroups of two wave pairs, 4-row tiles only (see fwd_k_split; D = 16 * (WAVES / 2) * KW);
-// D = 1024: one tile per workgroup, k split over its four waves, groups that span the device (D = 16 * KW; the reverse
-// kernels of the 4-gate cells at D = 640 and 768 in that form spill, so those head dims stay with the alternating backend)
+// D = 640 .. 1024: one tile per workgroup, k split over its four waves, groups that span the device (D = 16 * KW)
 #define FRNN_PLANS_GR4_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
-  X(1024, 0, 4, 1, 64, 4)
-// (backward, D = 384 .. 512: workgroups of two wave pairs, D = 1024: one tile position per workgroup, 4-row tiles
+  X(640, 0, 4, 1, 40, 4) X(768, 0, 4, 1, 48, 4) X(1024, 0, 4, 1, 64, 4)
+// (backward, D = 384 .. 512: workgroups of two wave pairs, D = 640 .. 1024: one tile position per workgroup, 4-row tiles
 // only; see bwd_dest_split)
 #define FRNN_BWD_PLANS_GR4_F32(X) \
   X(320, 2, 1, 1, 20, 4) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
-  X(1024, 0, 4, 1, 64, 4)
+  X(640, 0, 4, 1, 40, 4) X(768, 0, 4, 1, 48, 4) X(1024, 0, 4, 1, 64, 4)
 // slstm fp32 backward: the same without the 20-workgroup tiling of D = 320 (with four states its kernel spills)
 #define FRNN_BWD_PLANS_SLSTM_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 8) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 8) \
   X(320, 0, 4, 1, 5, 8) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
-  X(1024, 0, 4, 1, 64, 4)
+  X(640, 0, 4, 1, 40, 4) X(768, 0, 4, 1, 48, 4) X(1024, 0, 4, 1, 64, 4)
 // ---- 3 recurrent gate rows per unit (gru) ----------------------------------------------------
 #define FRNN_PLANS_GR3_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \
@@ -190,12 +189,12 @@ constexpr bool fwd_own_slice_first(int GR, int D, int WAVES, int UTW, int KW, in
 #define FRNN_PLANS_GR3_F32(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
-  X(1024, 0, 4, 1, 64, 4)
+  X(640, 0, 4, 1, 40, 4) X(768, 0, 4, 1, 48, 4) X(1024, 0, 4, 1, 64, 4)
 #define FRNN_BWD_PLANS_GR3_F32(X) \
   X(64, 2, 2, 1, 2, 16) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 2, 1, 3, 16) X(128, 0, 4, 1, 2, 16) X(160, 0, 2, 1, 5, 16) X(192, 0, 4, 1, 3, 16) X(256, 0, 4, 1, 4, 16) \
   X(320, 0, 4, 1, 5, 16) X(384, 0, 4, 1, 12, 4) X(448, 0, 4, 1, 14, 4) X(512, 0, 4, 1, 16, 4) \
-  X(1024, 0, 4, 1, 64, 4)
+  X(640, 0, 4, 1, 40, 4) X(768, 0, 4, 1, 48, 4) X(1024, 0, 4, 1, 64, 4)
 // ---- 1 recurrent gate row per unit (elman) ---------------------------------------------------
 #define FRNN_PLANS_GR1_BF16(X) \
   X(32, 0, 2, 1, 1, 16) X(64, 0, 4, 1, 1, 16) X(96, 0, 6, 1, 1, 16) X(128, 0, 8, 1, 1, 16) X(160, 0, 10, 1, 1, 16) X(192, 0, 12, 1, 1, 16) \

@@ -56,14 +56,15 @@ def test_supported_table(lib):
     assert lib.frnn_fused_supported(E, 0, 32, 1, 1024) == 0 and lib.frnn_fused_supported(G, 0, 32, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 2048) == _lib.E_UNSUPPORTED  # too large to keep on chip
-    # fp32: R is twice the size: the gated cells run up to D = 512 and at D = 1024 (the head dims of the reference's test
-    # grid, tests/test_lstm.py:9-46; at 1024 a head takes 64 workgroups, spread over the device), the elman cell at 1024
+    # fp32: R is twice the size: the gated cells run every head dim of the 16-bit list (the reference's test grid,
+    # tests/test_lstm.py:9-46, has 32, 64, 512 and 1024; beyond 512 a head takes 40 to 64 workgroups, spread over the device)
     for f in (L, S, G, E):
         for D in (32, 64, 96, 128, 160, 192, 256, 320, 384, 448, 512):
             assert lib.frnn_fused_supported(f, 1, 8, 1, D) == 0, (f, D)
-    assert lib.frnn_fused_supported(L, 1, 8, 1, 640) == _lib.E_UNSUPPORTED
     for f in (L, S, G):
-        assert lib.frnn_fused_supported(f, 1, 8, 2, 1024) == 0, f
+        for D in (640, 768, 1024):
+            assert lib.frnn_fused_supported(f, 1, 8, 2, D) == 0, (f, D)
+    assert lib.frnn_fused_supported(L, 1, 8, 1, 896) == _lib.E_UNSUPPORTED
     assert lib.frnn_fused_supported(E, 1, 8, 1, 768) == 0 and lib.frnn_fused_supported(E, 1, 8, 1, 1024) == 0
     assert lib.frnn_fused_supported(L, 0, 8, 1, 48) == _lib.E_UNSUPPORTED
     assert b"head dim" in lib.frnn_last_error()

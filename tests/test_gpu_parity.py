@@ -85,6 +85,10 @@ FUSED_SMALL = [
     ("slstm", 9, 4, 1, 1024, "float32"),     # 3 groups, the last with one valid row
     ("gru", 17, 3, 1, 1024, "float32"),      # 5 groups: two launches
     ("lstm", 3, 4, 2, 1024, "float32"),
+    ("lstm", 7, 4, 1, 640, "float32"),       # 40 workgroups per head: 10 groups of 4 destinations, 3 + 3 + 2 + 2 over the waves
+    ("slstm", 5, 5, 1, 768, "float32"),      # 48 workgroups per head
+    ("gru", 25, 3, 1, 768, "float32"),       # 7 groups: two launches of at most 5
+    ("slstm", 4, 4, 1, 640, "float32"),
     ("lstm", 37, 4, 1, 512, "float32"),      # 10 groups of 4 rows, the last with one valid row
     ("gru", 70, 4, 1, 384, "float32"),       # 18 groups of 12 workgroups: two launches
     # elman fp32 from D = 128 on: D / 64 workgroups of one tile per wave
