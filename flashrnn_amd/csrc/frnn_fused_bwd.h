@@ -122,7 +122,11 @@ fused_bwd_kernel(const BwdArgs a) {
   constexpr int NCA = NCX > 0 ? NCX : 1;
   // remote sources polled together: every round of polling costs at least one trip to L2 and back,
   // so as few rounds as 16 words per lane and probe allow, of equal size (no dummy loads)
-  constexpr int RC_MAX = 16 / (UTW * (TR / 4)) > 0 ? 16 / (UTW * (TR / 4)) : 1;
+  // (16 words per lane and probe; 32 for the 16-bit kernels at 8- and 16-row tiles, 2 and 4 words per source, where the
+  // rounds halve: reverse kernel, B256 T512, GRU D = 1024 3.44 -> 3.18 ms, sLSTM D = 768 1.43 -> 1.37, LSTM D = 640 1.85 -> 1.83,
+  // D = 512 1.04 -> 1.03, D = 768 no change; not the kernels whose wave pairs share the receive: LSTM D = 1024 1.54 -> 1.62)
+  constexpr int RCW = sizeof(T) == 2 && TR >= 8 && DSP == 1 ? 32 : 16;
+  constexpr int RC_MAX = RCW / (UTW * (TR / 4)) > 0 ? RCW / (UTW * (TR / 4)) : 1;
   constexpr int ROUNDS = KW == 1 ? 1 : (KW - 1 + RC_MAX - 1) / RC_MAX;
   constexpr int PSRC = KW == 1 ? 1 : (KW - 1 + ROUNDS - 1) / ROUNDS;  // sources polled per round
   constexpr size_t INW = bwd_inbox_words(D, KW);
