@@ -24,6 +24,9 @@ CASES = [
     ("slstm", 7, 10, 2, 192, "bfloat16", "hip_fused"),
     ("elman", 9, 8, 1, 512, "bfloat16", "hip_fused"),   # under forward_clipval: gate cache with the unclamped h
     ("elman", 5, 7, 2, 64, "float32", "hip_fused"),
+    ("lstm", 5, 6, 1, 448, "float32", "hip_fused"),      # workgroups of two wave pairs
+    ("slstm", 6, 5, 1, 1024, "bfloat16", "hip_fused"),   # the same in the 16-bit kernels
+    ("gru", 5, 5, 1, 1024, "float32", "hip_fused"),      # four waves per tile, groups that span the device
     ("lstm", 5, 6, 2, 64, "bfloat16", "hip"),
     ("gru", 3, 7, 2, 96, "float32", "hip"),
     ("slstm", 4, 6, 1, 64, "float32", "hip"),
