@@ -140,7 +140,8 @@ static int fwd_poll_delay_default(int function, int dtype, const Plan& p, int ti
   if (p.kw <= 1) return 0;
   // groups that span the device exchange through memory, at agent scope: a round trip takes several times as long as
   // one to the L2 of an XCD (lstm fp32 D=1024, forward, 1024 steps: delay 0 6.09 ms, 8 4.81, 16 4.37, 24 3.92, 32 4.00, 48 4.36)
-  if (p.kw > kXcdWorkgroups) return 24;
+  // (the other cells and D = 768 also best at 24, within 1 %; 40 workgroups per head, D = 640: 18 2.64 ms, 24 2.74)
+  if (p.kw > kXcdWorkgroups) return p.kw <= 40 ? 18 : 24;
   const bool elman = function == FRNN_ELMAN || function == FRNN_ELMAN_CLIP;
   // kernels that multiply the workgroup's own slice in front of the wait: little is left to sleep through
   if (fwd_own_slice_first(cell_dims(function).GR, p.D, p.waves, p.utw, p.kw, tile_rows, dtype == FRNN_F32 ? 4 : 2)) {
